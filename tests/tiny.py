@@ -1,0 +1,56 @@
+"""The tiny configurations the tests run: two Qwen3 shapes that differ in every size and
+option, plus helpers that make weights and model folders for them."""
+from __future__ import annotations
+
+import os
+import tempfile
+from typing import Dict
+
+import torch
+
+from zinfer_amd.config import Qwen3Config
+from zinfer_amd.models.build import declare_tensors
+from zinfer_amd.weights import draw_tensors, write_model_dir
+
+TINY_A = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2,
+              hidden_size=64, num_attention_heads=4, num_key_value_heads=2, head_dim=16,
+              intermediate_size=192, vocab_size=512, rope_theta=10000.0, rms_norm_eps=1e-6,
+              tie_word_embeddings=True, max_position_embeddings=256, torch_dtype="float32")
+
+TINY_B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=3,
+              hidden_size=96, num_attention_heads=8, num_key_value_heads=2, head_dim=32,
+              intermediate_size=320, vocab_size=1000, rope_theta=1000000.0, rms_norm_eps=1e-5,
+              tie_word_embeddings=False, max_position_embeddings=512, torch_dtype="float32")
+
+# a third shape with sizes that are no power of two anywhere: 3 query heads on 1 kv head,
+# head_dim 48, hidden 80, vocabulary 777
+TINY_C = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2,
+              hidden_size=80, num_attention_heads=3, num_key_value_heads=1, head_dim=48,
+              intermediate_size=112, vocab_size=777, rope_theta=50000.0, rms_norm_eps=3e-6,
+              tie_word_embeddings=False, max_position_embeddings=384, torch_dtype="float32")
+
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+PAGE_SIZE = {"A": 16, "B": 8, "C": 16}
+SEEDS = {"A": 11, "B": 22, "C": 33}
+
+
+def config_of(name: str) -> Qwen3Config:
+    return Qwen3Config.from_dict(CONFIGS[name])
+
+
+def weights_of(name: str, dtype=torch.float32) -> Dict[str, torch.Tensor]:
+    cfg = config_of(name)
+    spec = cfg.model_spec()
+    return draw_tensors(declare_tensors(spec), SEEDS[name], dtype, tied=spec.tie_word_embeddings)
+
+
+def model_dir_of(name: str, root: str, dtype=torch.float32) -> str:
+    path = os.path.join(root, f"tiny_{name}_{str(dtype).split('.')[-1]}")
+    if not os.path.exists(os.path.join(path, "model.safetensors")):
+        write_model_dir(path, config_of(name), SEEDS[name], dtype)
+    return path
+
+
+def random_tokens(n: int, vocab: int, seed: int):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()

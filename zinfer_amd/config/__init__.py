@@ -1,0 +1,6 @@
+from .registry import (ArchitectureEntry, entry_for, load_config, read_config_json,
+                       register_architecture, registered_architectures,
+                       unregister_architecture)
+from .specs import (GqaAttentionSpec, ModelSpec, NoPositionSpec, PreNormBlockSpec, RmsNormSpec,
+                    RotaryHalfSplitSpec, ScheduleEntry, SwiGluSpec)
+from .qwen3 import Qwen3Config

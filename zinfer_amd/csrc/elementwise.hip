@@ -1,0 +1,229 @@
+// Embedding gather, RMSNorm, per-head norm + rotation + cache write, SwiGLU, row gather,
+// arg-max.  Formulas follow the reference's CPU kernels (src/kernel/core/cpu.zig,
+// src/kernel/attention/rope.zig); all arithmetic is 32-bit, storage is float or bfloat16.
+#include "zf_common.h"
+
+// ---------------------------------------------------------------- embedding: x[t,:] = E[id[t],:]
+template <typename TW>
+__global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ ids,
+                             float* __restrict__ out, int H) {
+  const int t = blockIdx.x;
+  const TW* row = table + (size_t)ids[t] * H;
+  float* o = out + (size_t)t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = load_as_float<TW>(row + i);
+}
+
+extern "C" int zf_embed(const void* table, int table_dtype, const int* ids, float* out, int T,
+                        int H, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (table_dtype == ZF_F32)
+    hipLaunchKernelGGL(embed_kernel<float>, dim3(T), dim3(256), 0, stream, (const float*)table,
+                       ids, out, H);
+  else
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(T), dim3(256), 0, stream,
+                       (const bf16_t*)table, ids, out, H);
+  ZF_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------- RMSNorm over rows of width W
+// n_i = x_i * w_i / sqrt(mean(x^2) + eps)      (cpu.zig:38-48,73-110)
+template <typename TO>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ gain,
+                               TO* __restrict__ out, int W, float eps) {
+  __shared__ float red[16];
+  const float* row = x + (size_t)blockIdx.x * W;
+  TO* o = out + (size_t)blockIdx.x * W;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    const float v = row[i];
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += blockDim.x)
+    store_from_float<TO>(o + i, row[i] * inv * gain[i]);
+}
+
+extern "C" int zf_rmsnorm(const float* x, const float* gain, void* out, int out_dtype, int T,
+                          int W, float eps, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (out_dtype == ZF_F32)
+    hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(T), dim3(256), 0, stream, x, gain,
+                       (float*)out, W, eps);
+  else
+    hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(T), dim3(256), 0, stream, x, gain,
+                       (bf16_t*)out, W, eps);
+  ZF_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------- per-head norm, rotation, cache write
+// One wave per (token, head).  Heads 0..nH-1 are query heads, the next nKV key heads, the
+// last nKV value heads, each a contiguous slice of hd elements of the token's row of `qkv`.
+//   q, k: optional RMSNorm over the head (cpu.zig:50-71), optional half-split rotation
+//         (x_i, x_{i+hd/2}) <- (x_i c - x_{i+hd/2} s, x_{i+hd/2} c + x_i s)   (rope.zig:92-109)
+//   q -> q_out (or back in place when q_out is null)
+//   k, v -> page `slot / page_size`, row `slot % page_size` of the pools laid out
+//           [page, kv head, row, hd]   (or k back in place when slot_mapping is null)
+template <typename T>
+__global__ void qk_norm_rope_kv_write_kernel(
+    T* __restrict__ qkv, const float* __restrict__ q_gain, const float* __restrict__ k_gain,
+    float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int* __restrict__ positions, const int* __restrict__ slot_mapping,
+    T* __restrict__ k_pool, T* __restrict__ v_pool, T* __restrict__ q_out, int nH, int nKV,
+    int hd, int page_size) {
+  const int t = blockIdx.x;
+  const int head = blockIdx.y;
+  const int lane = threadIdx.x;
+  const int half = hd / 2;
+  const int row_width = (nH + 2 * nKV) * hd;
+  T* src = qkv + (size_t)t * row_width + (size_t)head * hd;
+
+  if (head >= nH + nKV) {  // value head: copy into the cache
+    if (slot_mapping == nullptr) return;
+    const int kvh = head - nH - nKV;
+    const int slot = slot_mapping[t];
+    const int page = slot / page_size, r = slot % page_size;
+    T* dst = v_pool + (((size_t)page * nKV + kvh) * page_size + r) * hd;
+    for (int i = lane; i < hd; i += ZF_WAVE) dst[i] = src[i];
+    return;
+  }
+  const bool is_q = head < nH;
+  const float* gain = is_q ? q_gain : k_gain;
+  T* dst;
+  if (is_q) {
+    dst = q_out ? q_out + (size_t)t * nH * hd + (size_t)head * hd : src;
+  } else if (slot_mapping) {
+    const int kvh = head - nH;
+    const int slot = slot_mapping[t];
+    const int page = slot / page_size, r = slot % page_size;
+    dst = k_pool + (((size_t)page * nKV + kvh) * page_size + r) * hd;
+  } else {
+    dst = src;
+  }
+  float inv = 1.0f;
+  if (gain) {
+    float ss = 0.f;
+    for (int i = lane; i < hd; i += ZF_WAVE) {
+      const float v = load_as_float<T>(src + i);
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    inv = 1.0f / sqrtf(ss / (float)hd + eps);
+  }
+  const int pos = positions[t];
+  for (int i = lane; i < half; i += ZF_WAVE) {
+    float x0 = load_as_float<T>(src + i);
+    float x1 = load_as_float<T>(src + i + half);
+    if (gain) {
+      x0 = x0 * inv * gain[i];
+      x1 = x1 * inv * gain[i + half];
+    }
+    if (cos_t) {
+      const float c = cos_t[(size_t)pos * half + i], s = sin_t[(size_t)pos * half + i];
+      const float r0 = x0 * c - x1 * s;
+      const float r1 = x1 * c + x0 * s;
+      x0 = r0;
+      x1 = r1;
+    }
+    store_from_float<T>(dst + i, x0);
+    store_from_float<T>(dst + i + half, x1);
+  }
+}
+
+extern "C" int zf_qk_norm_rope_kv_write(void* qkv, int dtype, const float* q_gain,
+                                        const float* k_gain, float eps, const float* cos_t,
+                                        const float* sin_t, const int* positions,
+                                        const int* slot_mapping, void* k_pool, void* v_pool,
+                                        void* q_out, int T, int nH, int nKV, int hd,
+                                        int page_size, hipStream_t stream) {
+  if (T <= 0) return 0;
+  dim3 grid(T, nH + 2 * nKV);
+  if (dtype == ZF_F32)
+    hipLaunchKernelGGL(qk_norm_rope_kv_write_kernel<float>, grid, dim3(ZF_WAVE), 0, stream,
+                       (float*)qkv, q_gain, k_gain, eps, cos_t, sin_t, positions, slot_mapping,
+                       (float*)k_pool, (float*)v_pool, (float*)q_out, nH, nKV, hd, page_size);
+  else
+    hipLaunchKernelGGL(qk_norm_rope_kv_write_kernel<bf16_t>, grid, dim3(ZF_WAVE), 0, stream,
+                       (bf16_t*)qkv, q_gain, k_gain, eps, cos_t, sin_t, positions, slot_mapping,
+                       (bf16_t*)k_pool, (bf16_t*)v_pool, (bf16_t*)q_out, nH, nKV, hd, page_size);
+  ZF_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------- SwiGLU on [T, 2I] -> [T, I]
+// a_j = g_j / (1 + exp(-g_j)) * u_j     (cpu.zig:130-147); gate is the first I columns.
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t n) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  const size_t t = idx / I, j = idx % I;
+  const float g = load_as_float<T>(gu + t * 2 * I + j);
+  const float u = load_as_float<T>(gu + t * 2 * I + I + j);
+  store_from_float<T>(out + idx, g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int zf_swiglu(const void* gu, void* out, int dtype, int T, int I,
+                         hipStream_t stream) {
+  const size_t n = (size_t)T * I;
+  if (n == 0) return 0;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (dtype == ZF_F32)
+    hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(256), 0, stream,
+                       (const float*)gu, (float*)out, I, n);
+  else
+    hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream,
+                       (const bf16_t*)gu, (bf16_t*)out, I, n);
+  ZF_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------- out[r,:] = x[idx[r],:]
+__global__ void gather_rows_kernel(const float* __restrict__ x, const int* __restrict__ idx,
+                                   float* __restrict__ out, int H) {
+  const float* row = x + (size_t)idx[blockIdx.x] * H;
+  float* o = out + (size_t)blockIdx.x * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = row[i];
+}
+
+extern "C" int zf_gather_rows(const float* x, const int* idx, float* out, int n, int H,
+                              hipStream_t stream) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(gather_rows_kernel, dim3(n), dim3(256), 0, stream, x, idx, out, H);
+  ZF_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------- arg-max, first maximum wins
+// (src/model/layers/logits.zig:47-59: strict > while walking upwards)
+__global__ void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V) {
+  __shared__ float sval[256];
+  __shared__ int sidx[256];
+  const float* row = logits + (size_t)blockIdx.x * V;
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = threadIdx.x; i < V; i += blockDim.x) {
+    const float v = row[i];
+    if (v > best) {
+      best = v;
+      bi = i;
+    }
+  }
+  sval[threadIdx.x] = best;
+  sidx[threadIdx.x] = bi;
+  __syncthreads();
+  for (int s = blockDim.x / 2; s > 0; s >>= 1) {
+    if (threadIdx.x < s) {
+      const float ov = sval[threadIdx.x + s];
+      const int oi = sidx[threadIdx.x + s];
+      if (ov > sval[threadIdx.x] || (ov == sval[threadIdx.x] && oi < sidx[threadIdx.x])) {
+        sval[threadIdx.x] = ov;
+        sidx[threadIdx.x] = oi;
+      }
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = sidx[0] == 0x7fffffff ? 0 : sidx[0];
+}
+
+extern "C" int zf_argmax(const float* logits, int* out, int n, int V, hipStream_t stream) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(argmax_kernel, dim3(n), dim3(256), 0, stream, logits, out, V);
+  ZF_CHECK_LAUNCH();
+}

@@ -1,0 +1,72 @@
+"""What one step runs: for each request its next tokens, and where logits are wanted."""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+
+@dataclass
+class StepEntry:
+    """``tokens`` are the request's next tokens (a portion of its prompt, or one decoded
+    token); ``want`` the places among them whose logits are asked for."""
+    request_id: object
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class KVStepTables:
+    block_table: torch.Tensor     # int32 [n_seqs, max_pages]; -1 where no page is held
+    slot_mapping: torch.Tensor    # int32 [T]: page * page_size + row, for the write
+    max_pages: int
+
+
+class Scratch:
+    """Named work buffers that live across steps and grow when a step needs more, so that a
+    step allocates nothing once sizes have settled."""
+
+    def __init__(self, device):
+        self.device = device
+        self._bufs: Dict[str, torch.Tensor] = {}
+
+    def get(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+        n = 1
+        for d in shape:
+            n *= int(d)
+        nbytes = max(n, 1) * torch.empty((), dtype=dtype).element_size()
+        buf = self._bufs.get(name)
+        if buf is None or buf.numel() < nbytes:
+            buf = torch.empty(((nbytes + 255) // 256 * 256,), dtype=torch.uint8, device=self.device)
+            self._bufs[name] = buf
+        return buf[:n * torch.empty((), dtype=dtype).element_size()].view(dtype).view(*shape)
+
+
+@dataclass
+class StepContext:
+    """Everything the parts may read about the step.  Device tensors are int32."""
+    n_tokens: int
+    n_seqs: int
+    n_want: int
+    token_ids: torch.Tensor       # [T]
+    positions: torch.Tensor       # [T] absolute position of each token in its request
+    seq_index: torch.Tensor       # [T] which sequence of this step a token belongs to
+    q_start: torch.Tensor         # [n_seqs + 1] first token of each sequence in the batch
+    ctx_len: torch.Tensor         # [n_seqs] tokens the request holds after this step
+    state_slots: torch.Tensor     # [n_seqs] slot of each request's fixed-size state
+    want_rows: torch.Tensor       # [n_want] token rows whose logits are wanted
+    kv: List[KVStepTables]
+    max_q_len: int
+    max_ctx_len: int
+    q_lens: List[int]             # host copies, for parts that loop on the host
+    ctx_lens: List[int]
+    slots: List[int]
+    _scratch: Scratch = None
+
+    def scratch(self, name: str, shape, dtype) -> torch.Tensor:
+        return self._scratch.get(name, shape, dtype)
+
+    def kv_tables(self, group: int) -> KVStepTables:
+        return self.kv[group]

@@ -1,0 +1,190 @@
+"""The step function: a batch of (request, its next tokens) run as one batch from the cache.
+
+The reference's counterpart runs one token of one request (`src/model/runtime/
+optimized_decoder/runtime.zig:103-148`) and loops it for a prompt (`:150-163`); its limits
+are kept as errors raised before anything is launched: a token id beyond the vocabulary
+(`:109`), a position beyond the table (`src/kernel/attention/rope.zig:135`), a full cache
+(`src/model/runtime/optimized_kv_cache/cache.zig:96`).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache import NO_PAGE, CacheManager
+from ..errors import (CacheFull, PositionOutOfBounds, StepError, TokenIdOutOfBounds)
+from ..models.decoder import DecoderModel
+from .batch import KVStepTables, Scratch, StepContext, StepEntry
+
+
+def _pad4(n: int) -> int:
+    return (n + 3) // 4 * 4
+
+
+class Engine:
+    """Owns a model, its cache and work buffers; ``step`` is the only way tokens run."""
+
+    def __init__(self, model: DecoderModel, *, page_size: int = 16, num_pages: int = 256,
+                 max_requests: int = 64, kv_dtype: Optional[torch.dtype] = None,
+                 poison_freed: bool = False):
+        self.model = model
+        self.device = model.ctx.device
+        spec = model.spec
+        needs = model.cache_needs()
+        reads = [e.cache_of for e in spec.schedule]
+        self.cache = CacheManager(needs, reads, page_size, num_pages, max_requests,
+                                  kv_dtype or model.ctx.compute_dtype, self.device,
+                                  poison_freed=poison_freed)
+        self.views = [self.cache.view(pos) for pos in range(len(spec.schedule))]
+        self.page_size = page_size
+        self._scratch = Scratch(self.device)
+        self._meta_host: Optional[torch.Tensor] = None
+        self._meta_dev: Optional[torch.Tensor] = None
+        self.steps_run = 0
+
+    # ------------------------------------------------------------------ requests
+    def has_request(self, rid) -> bool:
+        return self.cache.has_request(rid)
+
+    def length(self, rid) -> int:
+        return self.cache.length(rid)
+
+    def release(self, rid) -> None:
+        self.cache.release(rid)
+
+    # ------------------------------------------------------------------ the step
+    def step(self, entries: Sequence[StepEntry], end: Sequence[object] = ()) -> torch.Tensor:
+        """Runs the tokens of ``entries`` as one batch and returns float32 logits
+        [number of wanted places, vocab] in the order of the entries and of their ``want``.
+        Requests in ``end`` give back what they hold after the step.  On an error nothing
+        has run and the cache is as before."""
+        spec = self.model.spec
+        seen = set()
+        wanted_len = []
+        for e in entries:
+            if e.request_id in seen:
+                raise StepError(f"request {e.request_id!r} appears twice in one step")
+            seen.add(e.request_id)
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"request {e.request_id!r}: a portion must hold a token")
+            for t in e.tokens:
+                if not (0 <= int(t) < spec.vocab_size):
+                    raise TokenIdOutOfBounds(f"TokenIdOutOfBounds: token {t} of request "
+                                             f"{e.request_id!r}, vocabulary {spec.vocab_size}")
+            for w in e.want:
+                if not (0 <= int(w) < n):
+                    raise StepError(f"request {e.request_id!r}: want {w} outside its {n} tokens")
+            start = self.cache.length(e.request_id) if self.cache.has_request(e.request_id) else 0
+            if start + n > spec.max_positions:
+                raise PositionOutOfBounds(
+                    f"PositionOutOfBounds: request {e.request_id!r} would reach position "
+                    f"{start + n - 1}, max_position_embeddings is {spec.max_positions}")
+            wanted_len.append((e.request_id, start + n))
+        for rid in end:
+            if rid not in seen and not self.cache.has_request(rid):
+                raise StepError(f"request {rid!r} cannot end: it is not live")
+        if not self.cache.can_reserve(wanted_len):
+            raise CacheFull(f"CacheFull: the step needs more pages or request slots than are "
+                            f"free (free pages per group: {self.cache.num_free_pages()})")
+        if entries:
+            for rid, new_len in wanted_len:
+                if not self.cache.has_request(rid):
+                    self.cache.add_request(rid)
+                self.cache.reserve(rid, new_len)
+            ctx = self._build_context(entries)
+            logits = self.model.forward(ctx, self.views)
+            for rid, new_len in wanted_len:
+                self.cache.commit(rid, new_len)
+            self.steps_run += 1
+        else:
+            logits = torch.empty((0, spec.vocab_size), dtype=torch.float32, device=self.device)
+        for rid in end:
+            self.cache.release(rid)
+        return logits
+
+    # ------------------------------------------------------------------ metadata
+    def _build_context(self, entries: Sequence[StepEntry]) -> StepContext:
+        ps = self.page_size
+        n_seqs = len(entries)
+        q_lens = [len(e.tokens) for e in entries]
+        T = sum(q_lens)
+        starts = [self.cache.length(e.request_id) for e in entries]
+        ctx_lens = [s + n for s, n in zip(starts, q_lens)]
+        slots = [self.cache.state_slot(e.request_id) for e in entries]
+        want_rows: List[int] = []
+        q_start = [0]
+        for e, n in zip(entries, q_lens):
+            want_rows.extend(q_start[-1] + int(w) for w in e.want)
+            q_start.append(q_start[-1] + n)
+        n_want = len(want_rows)
+        n_groups = len(self.cache.groups)
+        max_pages = max((c + ps - 1) // ps for c in ctx_lens)
+
+        # one packed int32 buffer, one copy to the device
+        sizes = [("token_ids", T), ("positions", T), ("seq_index", T), ("q_start", n_seqs + 1),
+                 ("ctx_len", n_seqs), ("state_slots", n_seqs), ("want_rows", max(n_want, 1))]
+        for g in range(n_groups):
+            sizes += [(f"slot_mapping{g}", T), (f"block_table{g}", n_seqs * max_pages)]
+        offs, total = {}, 0
+        for name, n in sizes:
+            offs[name] = (total, n)
+            total += _pad4(n)
+        host = np.zeros((total,), dtype=np.int32)
+
+        def put(name, values):
+            o, n = offs[name]
+            host[o:o + len(values)] = values
+
+        put("token_ids", np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries]))
+        put("positions", np.concatenate([np.arange(s, s + n, dtype=np.int32)
+                                         for s, n in zip(starts, q_lens)]))
+        put("seq_index", np.repeat(np.arange(n_seqs, dtype=np.int32), q_lens))
+        put("q_start", np.asarray(q_start, dtype=np.int32))
+        put("ctx_len", np.asarray(ctx_lens, dtype=np.int32))
+        put("state_slots", np.asarray(slots, dtype=np.int32))
+        put("want_rows", np.asarray(want_rows, dtype=np.int32))
+        for g in range(n_groups):
+            bt = np.full((n_seqs, max_pages), NO_PAGE, dtype=np.int32)
+            sm = np.empty((T,), dtype=np.int32)
+            for i, e in enumerate(entries):
+                table = np.asarray(self.cache.table(g, e.request_id), dtype=np.int32)
+                bt[i, :len(table)] = table[:max_pages]
+                pos = np.arange(starts[i], ctx_lens[i])
+                sm[q_start[i]:q_start[i + 1]] = table[pos // ps] * ps + pos % ps
+            if (sm < 0).any():
+                raise StepError("a token would be written to a page that is not held")
+            put(f"slot_mapping{g}", sm)
+            put(f"block_table{g}", bt.reshape(-1))
+
+        dev = self._upload(host)
+
+        def view(name):
+            o, n = offs[name]
+            return dev[o:o + n]
+
+        kv = [KVStepTables(view(f"block_table{g}").view(n_seqs, max_pages),
+                           view(f"slot_mapping{g}"), max_pages) for g in range(n_groups)]
+        return StepContext(
+            n_tokens=T, n_seqs=n_seqs, n_want=n_want, token_ids=view("token_ids"),
+            positions=view("positions"), seq_index=view("seq_index"), q_start=view("q_start"),
+            ctx_len=view("ctx_len"), state_slots=view("state_slots"),
+            want_rows=view("want_rows")[:n_want], kv=kv, max_q_len=max(q_lens),
+            max_ctx_len=max(ctx_lens), q_lens=q_lens, ctx_lens=ctx_lens, slots=slots,
+            _scratch=self._scratch)
+
+    def _upload(self, host: np.ndarray) -> torch.Tensor:
+        n = host.shape[0]
+        if self.device.type == "cpu":
+            return torch.from_numpy(host.copy())
+        if self._meta_host is None or self._meta_host.numel() < n:
+            cap = max(n * 2, 4096)
+            self._meta_host = torch.empty((cap,), dtype=torch.int32, pin_memory=True)
+            self._meta_dev = torch.empty((cap,), dtype=torch.int32, device=self.device)
+        # the previous step's copy must have left the pinned buffer before it is rewritten
+        torch.cuda.current_stream(self.device).synchronize()
+        self._meta_host[:n].numpy()[:] = host
+        self._meta_dev[:n].copy_(self._meta_host[:n], non_blocking=True)
+        return self._meta_dev[:n]

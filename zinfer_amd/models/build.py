@@ -1,0 +1,51 @@
+"""From a model folder (or a typed configuration and tensors) to a bound model."""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..config import load_config
+from ..config.specs import ModelSpec
+from ..parts import BuildContext, TensorDecl
+from ..weights.loader import load_tensors
+from .decoder import DecoderModel
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
+           "fp32": torch.float32, "f32": torch.float32}
+
+
+def parse_dtype(name) -> torch.dtype:
+    if isinstance(name, torch.dtype):
+        if name not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"compute dtype must be bfloat16 or float32, not {name}")
+        return name
+    try:
+        return _DTYPES[str(name).lower()]
+    except KeyError:
+        raise ValueError(f"dtype {name!r}: choose bfloat16 or float32") from None
+
+
+def declare_tensors(spec: ModelSpec) -> Dict[str, TensorDecl]:
+    """The tensors a model of ``spec`` binds; no device is touched."""
+    ctx = BuildContext(torch.float32, torch.device("meta"))
+    return DecoderModel(spec, ctx).declare()
+
+
+def build_model(spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype, device) -> DecoderModel:
+    ctx = BuildContext(parse_dtype(dtype), torch.device(device))
+    model = DecoderModel(spec, ctx)
+    model.bind(tensors)
+    return model
+
+
+def load_model(model_dir: str, dtype="bfloat16", device="cuda:0"):
+    """(typed configuration, bound model) of a folder with config.json and model.safetensors;
+    the architecture is chosen by config.json."""
+    config = load_config(model_dir)
+    spec = config.model_spec()
+    ctx = BuildContext(parse_dtype(dtype), torch.device(device))
+    model = DecoderModel(spec, ctx)
+    tensors = load_tensors(model_dir, model.declare())
+    model.bind(tensors)
+    return config, model

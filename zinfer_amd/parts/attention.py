@@ -1,0 +1,104 @@
+from __future__ import annotations
+
+import math
+from typing import Dict
+
+import torch
+
+from .. import ops
+from ..config.specs import GqaAttentionSpec
+from ..errors import ConfigError
+from .base import KVNeed, Mixer, TensorDecl, build_part, register_part
+from .linear import Linear, place_gain, place_matrix
+
+
+class GqaAttention(Mixer):
+    """Causal grouped-query attention over a paged cache, in the reference's order
+    (`src/model/runtime/optimized_decoder/layer.zig:110-142,188`): q/k/v projections,
+    optional per-head RMSNorm of q and k, position encoding of q and k, append (k, v) at the
+    token's position, softmax(q K^T / sqrt(hd)) V over the positions up to the token's own
+    (query head h reads kv head h // G), output projection added to the residual."""
+
+    def __init__(self, spec: GqaAttentionSpec, ctx, prefix):
+        super().__init__(spec, ctx, prefix)
+        s = spec
+        if s.n_heads == 0 or s.n_kv_heads == 0 or s.head_dim == 0:
+            raise ConfigError("InvalidDimensions: heads and head_dim must not be 0")
+        if s.n_heads % s.n_kv_heads != 0:
+            raise ConfigError(f"InvalidGrouping: {s.n_heads} query heads, {s.n_kv_heads} kv heads")
+        if s.window is not None and s.window < 1:
+            raise ConfigError(f"window={s.window} must be at least 1")
+        self.q_width = s.n_heads * s.head_dim
+        self.kv_width = s.n_kv_heads * s.head_dim
+        self.scale = s.scale if s.scale is not None else 1.0 / math.sqrt(float(s.head_dim))
+        self.position = build_part("position", s.position, ctx, prefix)
+
+    def declare(self) -> Dict[str, TensorDecl]:
+        s, p = self.spec, self.prefix
+        d = {p + "q_proj.weight": TensorDecl((self.q_width, s.hidden_size)),
+             p + "k_proj.weight": TensorDecl((self.kv_width, s.hidden_size)),
+             p + "v_proj.weight": TensorDecl((self.kv_width, s.hidden_size)),
+             p + "o_proj.weight": TensorDecl((s.hidden_size, self.q_width))}
+        if s.qk_norm_eps is not None:
+            d[p + "q_norm.weight"] = TensorDecl((s.head_dim,), init="gain")
+            d[p + "k_norm.weight"] = TensorDecl((s.head_dim,), init="gain")
+        d.update(self.position.declare())
+        return d
+
+    def bind(self, tensors) -> None:
+        p = self.prefix
+        q, k, v = (tensors[p + n] for n in ("q_proj.weight", "k_proj.weight", "v_proj.weight"))
+        if not (q.dtype == k.dtype == v.dtype):
+            q, k, v = q.float(), k.float(), v.float()
+        # rows of q, k and v one below the other: each output element keeps its own dot
+        # product, so fusing changes no value
+        self.qkv = Linear(place_matrix(torch.cat([q, k, v], dim=0), self.ctx))
+        self.o = Linear(place_matrix(tensors[p + "o_proj.weight"], self.ctx))
+        if self.spec.qk_norm_eps is not None:
+            self.q_gain = place_gain(tensors[p + "q_norm.weight"], self.ctx)
+            self.k_gain = place_gain(tensors[p + "k_norm.weight"], self.ctx)
+        else:
+            self.q_gain = self.k_gain = None
+        self.position.bind(tensors)
+
+    def cache_need(self):
+        return KVNeed(self.spec.n_kv_heads, self.spec.head_dim, self.spec.window)
+
+    def forward(self, h, residual, step, cache) -> None:
+        s = self.spec
+        T = h.shape[0]
+        act = self.ctx.act_dtype
+        qkv = step.scratch("qkv", (T, self.q_width + 2 * self.kv_width), act)
+        self.qkv.forward(h, qkv)
+        q = step.scratch("q", (T, self.q_width), act)
+        tables = self.position.rotation_tables()
+        kv = step.kv_tables(cache.group)
+        eps = float(s.qk_norm_eps) if s.qk_norm_eps is not None else 0.0
+        if tables is not None or not self.position.custom_apply:
+            cos, sin = tables if tables is not None else (None, None)
+            ops.qk_norm_rope_kv_write(
+                qkv, self.q_gain, self.k_gain, eps, cos, sin, step.positions,
+                kv.slot_mapping if cache.writes else None, cache.k_pool, cache.v_pool, q,
+                s.n_heads, s.n_kv_heads, s.head_dim, cache.page_size)
+        else:
+            # a position encoding of its own: norm in place, let it change q and k, then store
+            ops.qk_norm_rope_kv_write(qkv, self.q_gain, self.k_gain, eps, None, None,
+                                      step.positions, None, cache.k_pool, cache.v_pool, None,
+                                      s.n_heads, s.n_kv_heads, s.head_dim, cache.page_size)
+            self.position.apply(qkv[:, :self.q_width].unflatten(1, (s.n_heads, s.head_dim)),
+                                qkv[:, self.q_width:self.q_width + self.kv_width]
+                                .unflatten(1, (s.n_kv_heads, s.head_dim)), step.positions)
+            ops.qk_norm_rope_kv_write(qkv, None, None, 0.0, None, None, step.positions,
+                                      kv.slot_mapping if cache.writes else None,
+                                      cache.k_pool, cache.v_pool, q,
+                                      s.n_heads, s.n_kv_heads, s.head_dim, cache.page_size)
+        attn = step.scratch("attn", (T, self.q_width), act)
+        ops.paged_attention(q, cache.k_pool, cache.v_pool, kv.block_table, step.q_start,
+                            step.ctx_len, step.seq_index, attn, float(self.scale),
+                            0 if s.window is None else int(s.window),
+                            s.n_heads, s.n_kv_heads, s.head_dim, cache.page_size,
+                            step.max_q_len, step.max_ctx_len)
+        self.o.forward(attn, residual, accumulate=True)
+
+
+register_part("mixer", GqaAttentionSpec, GqaAttention)

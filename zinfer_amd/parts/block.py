@@ -1,0 +1,44 @@
+from __future__ import annotations
+
+from typing import Dict
+
+from ..config.specs import PreNormBlockSpec
+from .base import Block, TensorDecl, build_part, register_part
+
+
+class PreNormBlock(Block):
+    """x += mixer(norm(x)); x += feed_forward(norm(x)): the residual is the un-normed input
+    (`src/model/runtime/optimized_decoder/layer.zig:108,188-201`).  The residual stream ``x``
+    is float32; both sums happen in 32-bit inside the parts."""
+
+    def __init__(self, spec: PreNormBlockSpec, ctx, prefix):
+        super().__init__(spec, ctx, prefix)
+        self.mixer_norm = build_part("norm", spec.mixer_norm, ctx, prefix + spec.mixer_norm_prefix)
+        self.mixer = build_part("mixer", spec.mixer, ctx, prefix + spec.mixer_prefix)
+        self.ff_norm = build_part("norm", spec.ff_norm, ctx, prefix + spec.ff_norm_prefix)
+        self.feed_forward = build_part("feed_forward", spec.feed_forward, ctx,
+                                       prefix + spec.ff_prefix)
+        self.parts = (self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward)
+
+    def declare(self) -> Dict[str, TensorDecl]:
+        d: Dict[str, TensorDecl] = {}
+        for part in self.parts:
+            d.update(part.declare())
+        return d
+
+    def bind(self, tensors) -> None:
+        for part in self.parts:
+            part.bind(tensors)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def forward(self, x, step, cache) -> None:
+        h = step.scratch("normed", x.shape, self.ctx.act_dtype)
+        self.mixer_norm.forward(x, h)
+        self.mixer.forward(h, x, step, cache)
+        self.ff_norm.forward(x, h)
+        self.feed_forward.forward(h, x, step)
+
+
+register_part("block", PreNormBlockSpec, PreNormBlock)

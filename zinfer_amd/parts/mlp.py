@@ -1,0 +1,44 @@
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from .. import ops
+from ..config.specs import SwiGluSpec
+from .base import FeedForward, TensorDecl, register_part
+from .linear import Linear, place_matrix
+
+
+class SwiGluMlp(FeedForward):
+    """d = W_down (silu(W_gate m) * W_up m), added to the residual
+    (`src/model/runtime/optimized_decoder/layer.zig:194-201`, `src/kernel/core/cpu.zig:130-147`).
+    gate and up rows are stacked into one matrix at load: each output keeps its own dot
+    product."""
+
+    def declare(self) -> Dict[str, TensorDecl]:
+        s, p = self.spec, self.prefix
+        return {p + "gate_proj.weight": TensorDecl((s.intermediate_size, s.hidden_size)),
+                p + "up_proj.weight": TensorDecl((s.intermediate_size, s.hidden_size)),
+                p + "down_proj.weight": TensorDecl((s.hidden_size, s.intermediate_size))}
+
+    def bind(self, tensors) -> None:
+        p = self.prefix
+        g, u = tensors[p + "gate_proj.weight"], tensors[p + "up_proj.weight"]
+        if g.dtype != u.dtype:
+            g, u = g.float(), u.float()
+        self.gate_up = Linear(place_matrix(torch.cat([g, u], dim=0), self.ctx))
+        self.down = Linear(place_matrix(tensors[p + "down_proj.weight"], self.ctx))
+
+    def forward(self, h, residual, step) -> None:
+        T = h.shape[0]
+        I = self.spec.intermediate_size
+        act = self.ctx.act_dtype
+        gu = step.scratch("gate_up", (T, 2 * I), act)
+        self.gate_up.forward(h, gu)
+        a = step.scratch("ff_act", (T, I), act)
+        ops.swiglu(gu, a)
+        self.down.forward(a, residual, accumulate=True)
+
+
+register_part("feed_forward", SwiGluSpec, SwiGluMlp)

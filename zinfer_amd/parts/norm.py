@@ -1,0 +1,28 @@
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from .. import ops
+from ..config.specs import RmsNormSpec
+from .base import Norm, TensorDecl, register_part
+from .linear import place_gain
+
+
+class RmsNorm(Norm):
+    """n = x * w / sqrt(mean(x^2) + eps) (`src/kernel/core/cpu.zig:38-48,73-110`); reads the
+    float32 residual stream, writes the activation dtype."""
+
+    def declare(self) -> Dict[str, TensorDecl]:
+        return {self.prefix + "weight": TensorDecl((self.spec.width,), init="gain")}
+
+    def bind(self, tensors) -> None:
+        self.gain = place_gain(tensors[self.prefix + "weight"], self.ctx)
+
+    def forward(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        ops.rmsnorm(x, self.gain, float(self.spec.eps), out)
+        return out
+
+
+register_part("norm", RmsNormSpec, RmsNorm)
