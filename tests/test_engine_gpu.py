@@ -1,0 +1,182 @@
+"""The engine on the GPU against the plain implementation, in 32-bit and in bfloat16: each
+request alone and whole; most of it in one step and the last 32 tokens one by one; portions
+of changing size down to two tokens; mixed batches of up to four live requests with so few
+pages that they are used again; long decoding; the first tokens of a sequence."""
+import numpy as np
+import pytest
+import torch
+
+import plain
+import tiny
+import traces
+from gpu_util import DEV, rel_err
+
+pytestmark = pytest.mark.gpu
+
+# float32: every kernel accumulates in 32-bit; what is left is summation order.
+LOGITS_TOL_F32 = 2e-5
+# bfloat16: activations are rounded to 8 mantissa bits (2^-9 relative, ~1.1e-3 rms) about
+# seven times per layer; over 2-3 layers and the head that is ~1e-2 of the largest logit at
+# the worst of ~10^5 entries.  The plain side uses the same bfloat16-rounded weights.
+LOGITS_TOL_BF16 = 2e-2
+
+LENGTHS = {"A": (5, 17, 40, 70), "B": (1, 9, 33, 64, 130), "C": (3, 48, 65, 100)}
+_plain_cache = {}
+
+
+def _setup(name, dtype, tmp_path_factory):
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    root = tmp_path_factory.getbasetemp()
+    path = tiny.model_dir_of(name, str(root), store)
+    cfg = tiny.CONFIGS[name]
+    requests = {f"r{i}": tiny.random_tokens(n, cfg["vocab_size"], 100 + i)
+                for i, n in enumerate(LENGTHS[name])}
+    key = (name, dtype)
+    if key not in _plain_cache:
+        w = tiny.weights_of(name, store)
+        _plain_cache[key] = {rid: plain.model_forward_batched(cfg, w, toks).numpy()
+                             for rid, toks in requests.items()}
+    return path, cfg, requests, _plain_cache[key]
+
+
+DEVICE = [DEV]      # the CPU tests of the host logic put "cpu" here (kernels emulated)
+
+
+def _replay(path, dtype, steps, page_size, max_tokens=None, poison=True):
+    from zinfer_amd.engine.replay import make_engine
+    from zinfer_amd.engine import StepEntry
+    max_tokens = max_tokens or traces.peak_tokens(steps, 64)
+    eng = make_engine(path, dtype, max_tokens, DEVICE[0], page_size=page_size,
+                      poison_freed=poison)
+    outputs = {}
+    for st in steps:
+        entries = [StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]]
+        logits = eng.step(entries, end=st["end"])
+        if logits.shape[0]:
+            outputs[st["step"]] = logits.cpu().numpy().copy()
+    eng.cache.check()
+    assert not eng.cache.requests, "every request ended, nothing may be held"
+    return outputs, eng
+
+
+def _compare(steps, outputs, ref, vocab, tolerance):
+    got = traces.collect(steps, outputs, vocab)
+    assert set(got) == set(ref)
+    worst = 0.0
+    for rid in ref:
+        assert got[rid].shape == ref[rid].shape
+        assert np.isfinite(got[rid]).all(), f"{rid}: logits are not finite"
+        diff = np.abs(got[rid].astype(np.float64) - ref[rid])
+        err = diff.max(axis=1) / np.abs(ref[rid]).max()
+        bad = np.nonzero(err > tolerance)[0]
+        assert bad.size == 0, (f"request {rid}: first wrong position {bad[0]} of "
+                               f"{len(err)} (error {err[bad[0]]:.3g} > {tolerance})")
+        worst = max(worst, float(err.max()))
+    return worst
+
+
+MODES = {"whole": traces.whole, "prefill_then_32": traces.prefill_then_single,
+         "portions": traces.changing_portions, "mixed": traces.mixed,
+         "token_by_token": traces.token_by_token}
+
+
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_replay_modes(name, dtype, mode, tmp_path_factory):
+    path, cfg, requests, ref = _setup(name, dtype, tmp_path_factory)
+    steps = MODES[mode](requests)
+    outputs, eng = _replay(path, dtype, steps, tiny.PAGE_SIZE[name])
+    tolerance = LOGITS_TOL_F32 if dtype == "float32" else LOGITS_TOL_BF16
+    worst = _compare(steps, outputs, ref, cfg["vocab_size"], tolerance)
+    print(f"{name} {dtype} {mode}: worst error {worst:.3g}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixed_many_requests_reuse_pages(dtype, tmp_path_factory):
+    """Nine requests through a pool that holds four: every page is used several times."""
+    name = "B"
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    path = tiny.model_dir_of(name, str(tmp_path_factory.getbasetemp()), store)
+    cfg = tiny.CONFIGS[name]
+    lens = (40, 64, 23, 90, 17, 128, 55, 8, 77)
+    requests = {f"m{i}": tiny.random_tokens(n, cfg["vocab_size"], 300 + i)
+                for i, n in enumerate(lens)}
+    w = tiny.weights_of(name, store)
+    ref = {rid: plain.model_forward_batched(cfg, w, t).numpy() for rid, t in requests.items()}
+    for seed in (1, 2):
+        steps = traces.mixed(requests, max_live=4, seed=seed)
+        assert max(len(st["entries"]) for st in steps) == 4
+        outputs, eng = _replay(path, dtype, steps, tiny.PAGE_SIZE[name])
+        _compare(steps, outputs, ref, cfg["vocab_size"],
+                 LOGITS_TOL_F32 if dtype == "float32" else LOGITS_TOL_BF16)
+        pages = eng.cache.groups[0].pages
+        total = sum((n + eng.page_size - 1) // eng.page_size for n in lens)
+        assert pages.num_pages < total <= pages.handed_out, \
+            "the pool must be too small to avoid reuse"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(dtype, tmp_path_factory):
+    """A short prompt, then 300 tokens one by one across many pages."""
+    name = "B"
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    path = tiny.model_dir_of(name, str(tmp_path_factory.getbasetemp()), store)
+    cfg = tiny.CONFIGS[name]
+    toks = tiny.random_tokens(305, cfg["vocab_size"], 77)
+    ref = {"long": plain.model_forward_batched(cfg, tiny.weights_of(name, store), toks).numpy()}
+    steps = traces.prefill_then_single({"long": toks}, tail=300)
+    outputs, _ = _replay(path, dtype, steps, tiny.PAGE_SIZE[name])
+    _compare(steps, outputs, ref, cfg["vocab_size"],
+             LOGITS_TOL_F32 if dtype == "float32" else LOGITS_TOL_BF16)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_first_tokens_and_cut_invariance_f32(name, tmp_path_factory):
+    """The first tokens of a sequence (positions 0, 1, 2), and: in 32-bit the logits of a
+    position are the same to the last bit however the tokens were cut into steps."""
+    path, cfg, requests, ref = _setup(name, "float32", tmp_path_factory)
+    outs = {}
+    for mode in ("whole", "portions", "token_by_token", "mixed"):
+        steps = MODES[mode](requests)
+        outputs, _ = _replay(path, "float32", steps, tiny.PAGE_SIZE[name])
+        outs[mode] = traces.collect(steps, outputs, cfg["vocab_size"])
+    for rid in requests:
+        first = outs["whole"][rid][:3]
+        assert np.abs(first - ref[rid][:3]).max() <= LOGITS_TOL_F32 * np.abs(ref[rid]).max()
+        for mode in ("portions", "token_by_token", "mixed"):
+            assert np.array_equal(outs["whole"][rid], outs[mode][rid]), \
+                f"{rid}: {mode} differs from whole in 32-bit"
+
+
+def test_page_size_does_not_matter(tmp_path_factory):
+    path, cfg, requests, ref = _setup("A", "float32", tmp_path_factory)
+    steps = traces.changing_portions(requests)
+    a, _ = _replay(path, "float32", steps, 16)
+    b, _ = _replay(path, "float32", steps, 4)
+    for k in a:
+        assert np.array_equal(a[k], b[k])
+
+
+def test_step_errors_leave_cache_untouched(tmp_path_factory):
+    from zinfer_amd import CacheFull, PositionOutOfBounds, StepError, TokenIdOutOfBounds
+    from zinfer_amd.engine import StepEntry
+    from zinfer_amd.engine.replay import make_engine
+    path, cfg, requests, ref = _setup("A", "float32", tmp_path_factory)
+    eng = make_engine(path, "float32", 64, DEVICE[0])
+    with pytest.raises(TokenIdOutOfBounds):
+        eng.step([StepEntry("x", [1, cfg["vocab_size"]], [])])
+    with pytest.raises(StepError):
+        eng.step([StepEntry("x", [], [])])
+    with pytest.raises(StepError):
+        eng.step([StepEntry("x", [1, 2], [2])])
+    with pytest.raises(CacheFull):
+        eng.step([StepEntry("x", [1] * 65, [])])
+    with pytest.raises(PositionOutOfBounds):
+        eng.step([StepEntry("x", [1] * 300, [])])
+    assert not eng.cache.requests and eng.cache.num_free_pages() == [4]
+    eng.step([StepEntry("x", [1] * 60, [])])
+    with pytest.raises(CacheFull):
+        eng.step([StepEntry("x", [1] * 5, [])])
+    assert eng.length("x") == 60
+    eng.cache.check()

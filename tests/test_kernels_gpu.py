@@ -1,0 +1,319 @@
+"""Each HIP kernel alone against its plain torch reference (tests/kernel_refs.py), at sizes
+other than the engine's tiny configurations: widths and vocabularies that are no power of
+two, head sizes in steps of 16, any number of heads and groups."""
+import math
+
+import pytest
+import torch
+
+import kernel_refs as ref
+from gpu_util import DEV, rel_err, tol
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def _ops():
+    import zinfer_amd.ops as ops
+    return ops
+
+
+def _rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("V,H,T", [(1000, 96, 7), (777, 80, 33), (50, 4100, 3)])
+def test_embed(dtype, V, H, T):
+    table = _rand((V, H), dtype, 1)
+    ids = torch.randint(0, V, (T,), generator=torch.Generator().manual_seed(2)).int()
+    ids[0], ids[-1] = 0, V - 1
+    want = torch.empty((T, H))
+    ref.embed(table, ids, want)
+    got = torch.empty((T, H), device=DEV)
+    _ops().embed(table.to(DEV), ids.to(DEV), got)
+    assert torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("T,W,eps", [(5, 80, 1e-6), (3, 4096, 1e-5), (17, 1000, 3e-6), (1, 7, 0.0)])
+def test_rmsnorm(out_dtype, T, W, eps):
+    x = _rand((T, W), torch.float32, 3, 2.0)
+    gain = 1 + 0.1 * _rand((W,), torch.float32, 4)
+    want = torch.empty((T, W), dtype=out_dtype)
+    ref.rmsnorm(x, gain, eps, want)
+    got = torch.empty((T, W), dtype=out_dtype, device=DEV)
+    _ops().rmsnorm(x.to(DEV), gain.to(DEV), eps, got)
+    assert rel_err(got, want) <= tol(out_dtype)
+
+
+def test_rmsnorm_reference_vector():
+    """[3, 4] with gains [1, 2], eps 0 -> [0.84852814, 2.2627418]
+    (the reference's own test, src/kernel/core/cpu.zig:193-204)."""
+    x = torch.tensor([[3.0, 4.0]], device=DEV)
+    out = torch.empty_like(x)
+    _ops().rmsnorm(x, torch.tensor([1.0, 2.0], device=DEV), 0.0, out)
+    assert torch.allclose(out.cpu(), torch.tensor([[0.84852814, 2.2627418]]), atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,I", [(3, 112), (9, 1000), (1, 5)])
+def test_swiglu(dtype, T, I):
+    gu = _rand((T, 2 * I), dtype, 5, 3.0)
+    want = torch.empty((T, I), dtype=dtype)
+    ref.swiglu(gu, want)
+    got = torch.empty((T, I), dtype=dtype, device=DEV)
+    _ops().swiglu(gu.to(DEV), got)
+    assert rel_err(got, want) <= tol(dtype)
+
+
+def test_swiglu_reference_vector():
+    """gate [0, 1, -1], up [1, 2, 3] -> [0, 1.4621172, -0.8068243] (cpu.zig:233-245)."""
+    gu = torch.tensor([[0.0, 1.0, -1.0, 1.0, 2.0, 3.0]], device=DEV)
+    out = torch.empty((1, 3), device=DEV)
+    _ops().swiglu(gu, out)
+    assert torch.allclose(out.cpu(), torch.tensor([[0.0, 1.4621172, -0.8068243]]), atol=1e-6)
+
+
+@pytest.mark.parametrize("a_dtype,w_dtype,o_dtype", [
+    (torch.float32, torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16, torch.bfloat16),
+    (torch.bfloat16, torch.bfloat16, torch.float32), (torch.bfloat16, torch.float32, torch.bfloat16),
+    (torch.float32, torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("M,N,K", [(1, 1000, 96), (7, 77, 80), (65, 130, 33), (130, 64, 4100),
+                                   (2, 3, 5)])
+def test_gemm(a_dtype, w_dtype, o_dtype, M, N, K):
+    a = _rand((M, K), a_dtype, 6)
+    w = _rand((N, K), w_dtype, 7, 0.05)
+    want = torch.empty((M, N), dtype=o_dtype)
+    ref.gemm(a, w, want)
+    got = torch.full((M, N), float("nan"), dtype=o_dtype, device=DEV)
+    _ops().gemm(a.to(DEV), w.to(DEV), got)
+    assert rel_err(got, want) <= tol(o_dtype)
+
+
+@pytest.mark.parametrize("a_dtype", DTYPES)
+def test_gemm_accumulate_and_one_hot(a_dtype):
+    """out += a w^T in 32-bit; a one-hot row picks a column of W (the reference's
+    probe-linear, src/app/cli/inspect.zig:109-151)."""
+    M, N, K = 5, 70, 48
+    w = _rand((N, K), a_dtype, 8)
+    a = torch.zeros((M, K), dtype=a_dtype)
+    for m in range(M):
+        a[m, (m * 11) % K] = 1.0
+    base = _rand((M, N), torch.float32, 9)
+    got = base.clone().to(DEV)
+    _ops().gemm(a.to(DEV), w.to(DEV), got, accumulate=True)
+    want = base + torch.stack([w[:, (m * 11) % K].float() for m in range(M)])
+    assert rel_err(got, want) <= 1e-6
+
+
+def test_gemm_reference_vector():
+    """[[1,2,3],[4,5,6]] . [1, .5, -1] = [-1, .5] (src/kernel/core/cpu.zig:177-191)."""
+    w = torch.tensor([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]], device=DEV)
+    a = torch.tensor([[1.0, 0.5, -1.0]], device=DEV)
+    out = torch.empty((1, 2), device=DEV)
+    _ops().gemm(a, w, out)
+    assert torch.allclose(out.cpu(), torch.tensor([[-1.0, 0.5]]), atol=1e-6)
+
+
+def test_gemm_row_does_not_depend_on_batch():
+    """A row's result is bitwise the same alone and inside a larger batch (float32 path)."""
+    a = _rand((70, 200), torch.float32, 10).to(DEV)
+    w = _rand((90, 200), torch.float32, 11).to(DEV)
+    full = torch.empty((70, 90), device=DEV)
+    _ops().gemm(a, w, full)
+    for m in (0, 33, 69):
+        one = torch.empty((1, 90), device=DEV)
+        _ops().gemm(a[m:m + 1].contiguous(), w, one)
+        assert torch.equal(one[0], full[m])
+
+
+def _paged_setup(dtype, nH, nKV, hd, page_size, ctx_lens, q_lens, seed, num_pages=None):
+    """Random q and contiguous K/V per sequence, scattered into pages in a shuffled order."""
+    g = torch.Generator().manual_seed(seed)
+    n = len(ctx_lens)
+    pages_per = [(c + page_size - 1) // page_size for c in ctx_lens]
+    total = sum(pages_per)
+    num_pages = num_pages or total + 3
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    max_pages = max(pages_per)
+    bt = torch.full((n, max_pages), -1, dtype=torch.int32)
+    k_pool = torch.full((num_pages, nKV, page_size, hd), float("nan")).to(dtype)
+    v_pool = torch.full((num_pages, nKV, page_size, hd), float("nan")).to(dtype)
+    Ks, Vs = [], []
+    cur = 0
+    for s in range(n):
+        K = _rand((ctx_lens[s], nKV, hd), dtype, seed * 100 + s)
+        V = _rand((ctx_lens[s], nKV, hd), dtype, seed * 100 + 50 + s)
+        Ks.append(K); Vs.append(V)
+        for i in range(pages_per[s]):
+            pg = perm[cur]; cur += 1
+            bt[s, i] = pg
+            lo, hi = i * page_size, min((i + 1) * page_size, ctx_lens[s])
+            k_pool[pg, :, :hi - lo] = K[lo:hi].transpose(0, 1)
+            v_pool[pg, :, :hi - lo] = V[lo:hi].transpose(0, 1)
+    T = sum(q_lens)
+    q = _rand((T, nH * hd), dtype, seed + 7)
+    q_start = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+    seq_index = torch.repeat_interleave(torch.arange(n, dtype=torch.int32),
+                                        torch.tensor(q_lens))
+    return dict(q=q, k_pool=k_pool.view(num_pages, -1), v_pool=v_pool.view(num_pages, -1),
+                block_table=bt, q_start=q_start, ctx_len=torch.tensor(ctx_lens, dtype=torch.int32),
+                seq_index=seq_index.int(), Ks=Ks, Vs=Vs)
+
+
+def _run_attention(s, dtype, nH, nKV, hd, page_size, window, q_lens, ctx_lens):
+    scale = 1.0 / math.sqrt(hd)
+    T = s["q"].shape[0]
+    want = torch.empty((T, nH * hd), dtype=dtype)
+    ref.paged_attention(s["q"], s["k_pool"], s["v_pool"], s["block_table"], s["q_start"],
+                        s["ctx_len"], s["seq_index"], want, scale, window, nH, nKV, hd,
+                        page_size, max(q_lens), max(ctx_lens))
+    got = torch.full((T, nH * hd), float("nan"), dtype=dtype, device=DEV)
+    d = {k: v.to(DEV) for k, v in s.items() if isinstance(v, torch.Tensor)}
+    _ops().paged_attention(d["q"], d["k_pool"], d["v_pool"], d["block_table"], d["q_start"],
+                           d["ctx_len"], d["seq_index"], got, scale, window, nH, nKV, hd,
+                           page_size, max(q_lens), max(ctx_lens))
+    return got, want
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nH,nKV,hd,page_size,window", [
+    (4, 2, 16, 16, 0), (8, 2, 32, 8, 0), (3, 1, 48, 16, 0), (6, 3, 80, 4, 0),
+    (8, 8, 64, 16, 0), (5, 5, 128, 32, 0), (4, 1, 112, 16, 0), (4, 2, 32, 16, 19),
+    (2, 1, 64, 8, 8), (6, 2, 96, 16, 100)])
+def test_paged_attention_mixed_batch(dtype, nH, nKV, hd, page_size, window):
+    """Portions of prompts (some starting mid-context) beside single decode tokens."""
+    ctx_lens = [37, 150, 1, 64, 129, 16]
+    q_lens = [37, 1, 1, 5, 129 - 100, 2]
+    s = _paged_setup(dtype, nH, nKV, hd, page_size, ctx_lens, q_lens, seed=3)
+    got, want = _run_attention(s, dtype, nH, nKV, hd, page_size, window, q_lens, ctx_lens)
+    assert not torch.isnan(got.float()).any(), "a slot outside the context was read"
+    assert rel_err(got, want) <= tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_far_key_stands_out(dtype):
+    """One key among hundreds is aligned with the query and scaled up, so that the softmax
+    puts all weight on it: the output must be that position's value row.  The position is
+    put at a page's first row, a page's last row and the very first token in turn."""
+    nH, nKV, hd, ps = 4, 2, 64, 16
+    ctx = 700
+    for target in (16 * 20, 16 * 31 - 1, 0, ctx - 1):
+        s = _paged_setup(dtype, nH, nKV, hd, ps, [ctx], [1], seed=5)
+        q = s["q"].view(1, nH, hd).float()
+        kp = s["k_pool"].view(-1, nKV, ps, hd)
+        page = int(s["block_table"][0, target // ps])
+        for kvh in range(nKV):
+            direction = q[0, kvh * 2] / q[0, kvh * 2].norm()
+            kp[page, kvh, target % ps] = (direction * 400.0).to(dtype)
+        got, want = _run_attention(s, dtype, nH, nKV, hd, ps, 0, [1], [ctx])
+        for h in (0, 2):   # the heads whose query the key was aligned with
+            v_row = s["Vs"][0][target, h // 2].float()
+            assert torch.allclose(got.cpu().float()[0, h * hd:(h + 1) * hd], v_row, atol=2e-2), \
+                f"target {target}, head {h}"
+        assert rel_err(got, want) <= tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_window_edge(dtype):
+    """A huge key just outside the window must have no influence; the one just inside takes
+    all the weight."""
+    nH, nKV, hd, ps, window = 2, 1, 32, 8, 24
+    ctx = 100
+    pos = ctx - 1
+    for target, inside in ((pos - window, False), (pos - window + 1, True)):
+        s = _paged_setup(dtype, nH, nKV, hd, ps, [ctx], [1], seed=6)
+        q = s["q"].view(1, nH, hd).float()
+        kp = s["k_pool"].view(-1, nKV, ps, hd)
+        page = int(s["block_table"][0, target // ps])
+        kp[page, 0, target % ps] = (q[0, 0] / q[0, 0].norm() * 400.0).to(dtype)
+        got, want = _run_attention(s, dtype, nH, nKV, hd, ps, window, [1], [ctx])
+        v_row = s["Vs"][0][target, 0].float()
+        close = torch.allclose(got.cpu().float()[0, :hd], v_row, atol=2e-2)
+        assert close == inside
+        assert rel_err(got, want) <= tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nH,nKV,hd,page_size,use_norm,use_rope", [
+    (4, 2, 16, 16, True, True), (8, 2, 32, 8, True, True), (3, 1, 48, 16, True, True),
+    (5, 5, 128, 4, False, True), (6, 2, 80, 16, True, False), (2, 2, 256, 16, True, True)])
+def test_qk_norm_rope_kv_write(dtype, nH, nKV, hd, page_size, use_norm, use_rope):
+    from zinfer_amd.parts.position import rotary_tables
+    T, num_pages, eps = 11, 9, 1e-5
+    width = (nH + 2 * nKV) * hd
+    qkv = _rand((T, width), dtype, 12)
+    qg = (1 + 0.1 * _rand((hd,), torch.float32, 13)) if use_norm else None
+    kg = (1 + 0.1 * _rand((hd,), torch.float32, 14)) if use_norm else None
+    cos, sin = rotary_tables(hd, 10000.0, 300) if use_rope else (None, None)
+    positions = torch.tensor([0, 1, 2, 299, 150, 7, 8, 9, 63, 64, 65], dtype=torch.int32)
+    slots = torch.randperm(num_pages * page_size, generator=torch.Generator().manual_seed(1))[:T].int()
+    row = nKV * page_size * hd
+    pools = [torch.zeros((num_pages, row), dtype=dtype) for _ in range(4)]
+    q_want = torch.empty((T, nH * hd), dtype=dtype)
+    ref.qk_norm_rope_kv_write(qkv.clone(), qg, kg, eps, cos, sin, positions, slots, pools[0],
+                              pools[1], q_want, nH, nKV, hd, page_size)
+    dv = lambda t: None if t is None else t.to(DEV)
+    q_got = torch.empty((T, nH * hd), dtype=dtype, device=DEV)
+    kp, vp = pools[2].to(DEV), pools[3].to(DEV)
+    _ops().qk_norm_rope_kv_write(qkv.to(DEV), dv(qg), dv(kg), eps, dv(cos), dv(sin),
+                                 positions.to(DEV), slots.to(DEV), kp, vp, q_got, nH, nKV, hd,
+                                 page_size)
+    assert rel_err(q_got, q_want) <= tol(dtype)
+    assert rel_err(kp, pools[0]) <= tol(dtype)
+    assert torch.equal(vp.cpu(), pools[1])
+    # in place, nothing stored: q and k come back in the qkv buffer, v is untouched
+    want_inplace = qkv.clone()
+    ref.qk_norm_rope_kv_write(want_inplace, qg, kg, eps, cos, sin, positions, None, pools[0],
+                              pools[1], None, nH, nKV, hd, page_size)
+    got_inplace = qkv.to(DEV)
+    _ops().qk_norm_rope_kv_write(got_inplace, dv(qg), dv(kg), eps, dv(cos), dv(sin),
+                                 positions.to(DEV), None, kp, vp, None, nH, nKV, hd, page_size)
+    assert rel_err(got_inplace, want_inplace) <= tol(dtype)
+
+
+def test_rope_reference_vector():
+    """[1, 2, 3, 4] at position 1, theta 1e4: h0 = cos1 - 3 sin1, h1 = 2 cos(.01) - 4 sin(.01),
+    h2 = 3 cos1 + sin1, h3 = 4 cos(.01) + 2 sin(.01) (src/kernel/attention/rope.zig:174-190)."""
+    from zinfer_amd.parts.position import rotary_tables
+    cos, sin = rotary_tables(4, 10000.0, 4)
+    qkv = torch.tensor([[1.0, 2.0, 3.0, 4.0] * 3], device=DEV)   # one q, one k, one v head
+    pos = torch.tensor([1], dtype=torch.int32, device=DEV)
+    dummy = torch.zeros((1, 16), device=DEV)
+    _ops().qk_norm_rope_kv_write(qkv, None, None, 0.0, cos.to(DEV), sin.to(DEV), pos, None, dummy,
+                                 dummy, None, 1, 1, 4, 4)
+    a = 1.0 / math.sqrt(10000.0)
+    want = [math.cos(1) - 3 * math.sin(1), 2 * math.cos(a) - 4 * math.sin(a),
+            3 * math.cos(1) + math.sin(1), 4 * math.cos(a) + 2 * math.sin(a)]
+    assert torch.allclose(qkv.cpu()[0, :4], torch.tensor(want), atol=1e-6)
+    assert torch.allclose(qkv.cpu()[0, 4:8], torch.tensor(want), atol=1e-6)
+    assert torch.equal(qkv.cpu()[0, 8:], torch.tensor([1.0, 2.0, 3.0, 4.0]))
+
+
+def test_gather_rows_and_argmax():
+    x = _rand((9, 130), torch.float32, 15)
+    idx = torch.tensor([8, 0, 3, 3], dtype=torch.int32)
+    out = torch.empty((4, 130), device=DEV)
+    _ops().gather_rows(x.to(DEV), idx.to(DEV), out)
+    assert torch.equal(out.cpu(), x[idx.long()])
+    logits = _rand((6, 1000), torch.float32, 16)
+    logits[0, 17] = logits[0, 900] = 50.0      # a tie: the first maximum wins
+    logits[1, 999] = 60.0
+    logits[2, 0] = 60.0
+    logits[3] = -float("inf")
+    got = torch.empty((6,), dtype=torch.int32, device=DEV)
+    _ops().argmax(logits.to(DEV), got)
+    want = torch.argmax(logits, dim=-1).int()
+    want[3] = 0
+    assert torch.equal(got.cpu(), want)
+    assert got[0].item() == 17
+
+
+def test_cpu_tensor_is_refused():
+    """There is no CPU path: a tensor that is not on the GPU is an error, not a fallback."""
+    from zinfer_amd.errors import KernelUnavailable
+    with pytest.raises(KernelUnavailable):
+        _ops().rmsnorm(torch.zeros((1, 4)), torch.ones(4), 1e-6, torch.zeros((1, 4)))

@@ -19,6 +19,7 @@ class PageAllocator:
         self._free: List[int] = list(range(num_pages - 1, -1, -1))
         self._held = [False] * num_pages
         self.high_water = 0
+        self.handed_out = 0          # pages handed out over the allocator's life
 
     @property
     def num_free(self) -> int:
@@ -38,6 +39,7 @@ class PageAllocator:
             assert not self._held[p], f"page {p} handed out twice"
             self._held[p] = True
             out.append(p)
+        self.handed_out += n
         self.high_water = max(self.high_water, self.num_held)
         return out
 

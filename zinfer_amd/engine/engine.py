@@ -105,6 +105,16 @@ class Engine:
             self.cache.release(rid)
         return logits
 
+    def argmax(self, logits: torch.Tensor) -> List[int]:
+        """First-maximum arg-max of every row, on the device; only the ids come back."""
+        from .. import ops
+        n = logits.shape[0]
+        if n == 0:
+            return []
+        out = self._scratch.get("argmax", (n,), torch.int32)
+        ops.argmax(logits, out)
+        return out.tolist()
+
     # ------------------------------------------------------------------ metadata
     def _build_context(self, entries: Sequence[StepEntry]) -> StepContext:
         ps = self.page_size

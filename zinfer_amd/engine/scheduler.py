@@ -1,0 +1,222 @@
+"""The scheduler above the step function: admits requests, cuts prompts into portions under
+a token budget, decodes, finishes and frees.
+
+What the reference has of this (`src/model/runtime/optimized_decoder/batch.zig`): a fixed
+number of slots (`:31-73`), first-come admission into a freed slot (`:194-199`), one token
+per active request per round (`:116-136`), finish on an end-of-sequence id, which is checked
+before it is forwarded and neither stored nor counted (`:120-125`), or after
+``max_new_tokens`` (`:131-135`).  Its prefill is the whole prompt at once and its cache can
+never run out; portions, the budget and what happens when pages run out are this engine's:
+
+* a waiting request is admitted only when its next portion fits into free pages;
+* when a running request cannot get the page it needs, the most recently admitted running
+  request is preempted: its pages are freed, it keeps its generated tokens and its random
+  stream, goes to the front of the waiting queue and later recomputes prompt + generated;
+* a request that cannot fit even alone raises CacheFull.
+"""
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Deque, Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ..errors import CacheFull, StepError
+from ..sampling import SamplingParams, Xoshiro256pp, sample_token
+from .batch import StepEntry
+
+
+@dataclass
+class Request:
+    id: object
+    prompt: List[int]
+    params: SamplingParams
+    generated: List[int] = field(default_factory=list)
+    n_computed: int = 0                # tokens whose keys and values are in the cache
+    rng: Xoshiro256pp = None
+    finished: bool = False
+    finish_reason: Optional[str] = None
+    preemptions: int = 0
+
+    @property
+    def tokens(self) -> List[int]:
+        return self.prompt + self.generated
+
+    @property
+    def pending(self) -> int:
+        return len(self.prompt) + len(self.generated) - self.n_computed
+
+
+@dataclass
+class PlannedEntry:
+    request: Request
+    n_tokens: int
+    samples: bool                      # the portion reaches the end of the known tokens
+
+
+class Scheduler:
+    def __init__(self, engine, *, max_step_tokens: int = 2048, chunk_size: Optional[int] = None,
+                 max_seqs: int = 64, eos_token_ids: Sequence[int] = ()):
+        if max_step_tokens < 1 or max_seqs < 1:
+            raise ValueError("max_step_tokens and max_seqs must be at least 1")
+        self.engine = engine
+        self.cache = engine.cache
+        self.max_step_tokens = max_step_tokens
+        self.chunk_size = chunk_size or max_step_tokens
+        self.max_seqs = min(max_seqs, self.cache.max_requests)
+        self.eos_token_ids = tuple(eos_token_ids)
+        self.waiting: Deque[Request] = deque()
+        self.running: List[Request] = []           # in admission order
+        self.finished: Dict[object, Request] = {}
+        self._next_id = 0
+        self.n_steps = 0
+        self.n_preemptions = 0
+
+    # ------------------------------------------------------------------ requests
+    def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None,
+                    request_id=None) -> object:
+        prompt = [int(t) for t in prompt]
+        if not prompt:
+            raise StepError("a prompt must hold at least one token")
+        params = params or SamplingParams()
+        rid = request_id if request_id is not None else self._next_id
+        index = self._next_id
+        self._next_id += 1
+        # every request has a stream of its own, so its output does not depend on the batch
+        rng = Xoshiro256pp((params.seed ^ (index * 0x9E3779B97F4A7C15)) & ((1 << 64) - 1))
+        self.waiting.append(Request(rid, prompt, params, rng=rng))
+        return rid
+
+    def has_work(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    # ------------------------------------------------------------------ planning
+    def plan(self) -> List[PlannedEntry]:
+        """Decides what the next step runs.  May preempt; admits from the waiting queue."""
+        while True:
+            planned: List[PlannedEntry] = []
+            budget = self.max_step_tokens
+            wanted: List[Tuple[object, int]] = []
+
+            def try_add(req: Request, n: int) -> bool:
+                trial = wanted + [(req.id, req.n_computed + n)]
+                if not self.cache.can_reserve(trial):
+                    return False
+                wanted.append(trial[-1])
+                planned.append(PlannedEntry(req, n, n == req.pending))
+                return True
+
+            starved: Optional[Request] = None
+            # 1. requests that decode: one token each
+            for req in self.running:
+                if req.pending == 1 and req.generated and budget > 0:
+                    if try_add(req, 1):
+                        budget -= 1
+                    elif starved is None:
+                        starved = req
+            # 2. running requests still in their prompt (or recomputing)
+            for req in self.running:
+                if any(p.request is req for p in planned) or req is starved:
+                    continue
+                if req.pending == 1 and req.generated:
+                    continue
+                n = min(req.pending, self.chunk_size, budget)
+                if n <= 0:
+                    continue
+                if try_add(req, n):
+                    budget -= n
+                elif starved is None:
+                    starved = req
+            # 3. admission, first come first served, only if the next portion fits
+            while self.waiting and budget > 0 and len(self.running) < self.max_seqs \
+                    and starved is None:
+                req = self.waiting[0]
+                n = min(req.pending, self.chunk_size, budget)
+                if not try_add(req, n):
+                    break
+                budget -= n
+                self.waiting.popleft()
+                self.running.append(req)
+            if starved is not None and len(self.running) > 1:
+                # a running request cannot get its pages: the newest running request yields
+                self._preempt(self.running[-1])
+                continue
+            if not planned:
+                blocked = starved or (self.waiting[0] if self.waiting else None)
+                if blocked is not None and not self.running or \
+                        (starved is not None and len(self.running) == 1):
+                    raise CacheFull(
+                        f"CacheFull: request {blocked.id!r} needs "
+                        f"{blocked.n_computed + min(blocked.pending, self.chunk_size)} tokens of "
+                        "cache but does not fit even alone")
+            return planned
+
+    def _preempt(self, req: Request) -> None:
+        self.running.remove(req)
+        if self.cache.has_request(req.id):
+            self.cache.release(req.id)
+        req.n_computed = 0
+        req.preemptions += 1
+        self.n_preemptions += 1
+        self.waiting.appendleft(req)
+
+    # ------------------------------------------------------------------ one iteration
+    def step(self) -> List[Request]:
+        """Plans, runs one step, samples, finishes.  Returns the requests finished by it."""
+        planned = self.plan()
+        if not planned:
+            return []
+        entries = []
+        for p in planned:
+            toks = p.request.tokens[p.request.n_computed:p.request.n_computed + p.n_tokens]
+            entries.append(StepEntry(p.request.id, toks, [p.n_tokens - 1] if p.samples else []))
+        logits = self.engine.step(entries)
+        self.n_steps += 1
+        sampling = [p for p in planned if p.samples]
+        next_tokens = self._sample(logits, sampling)
+        done: List[Request] = []
+        for p in planned:
+            p.request.n_computed += p.n_tokens
+        for p, tok in zip(sampling, next_tokens):
+            req = p.request
+            reason = None
+            if not req.params.ignore_eos and (tok in self.eos_token_ids
+                                              or tok in req.params.stop_token_ids):
+                reason = "eos"                    # not stored, not counted
+            else:
+                req.generated.append(tok)
+                if len(req.generated) >= req.params.max_new_tokens:
+                    reason = "length"
+                elif len(req.prompt) + len(req.generated) > self.engine.model.spec.max_positions:
+                    reason = "context"
+            if reason is not None:
+                self._finish(req, reason)
+                done.append(req)
+        return done
+
+    def _finish(self, req: Request, reason: str) -> None:
+        req.finished = True
+        req.finish_reason = reason
+        self.running.remove(req)
+        self.cache.release(req.id)
+        self.finished[req.id] = req
+
+    def _sample(self, logits: torch.Tensor, sampling: List[PlannedEntry]) -> List[int]:
+        if not sampling:
+            return []
+        if all(p.request.params.greedy and not p.request.params.has_penalties for p in sampling):
+            return self.engine.argmax(logits)
+        rows = logits.detach().to("cpu", torch.float32).numpy()
+        out = []
+        for i, p in enumerate(sampling):
+            req = p.request
+            out.append(sample_token(rows[i], req.tokens, req.params, req.rng))
+        return out
+
+    def run(self) -> Dict[object, Request]:
+        """Steps until every request has finished."""
+        while self.has_work():
+            self.step()
+        return self.finished

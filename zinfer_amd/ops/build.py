@@ -31,6 +31,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
 
 _libs: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
+_dir_lock = threading.Lock()
 
 
 def _hipcc() -> str:
@@ -50,21 +51,30 @@ def _source_hash(module: str) -> str:
     return h.hexdigest()
 
 
+_lib_dir: Optional[str] = None
+
+
 def lib_dir() -> str:
     """Where built libraries live: ``zinfer_amd/_lib`` if it can be written, else a per-user
     temporary folder."""
-    pkg = os.path.join(os.path.dirname(CSRC), "_lib")
-    try:
-        os.makedirs(pkg, exist_ok=True)
-        probe = os.path.join(pkg, f".w{os.getpid()}")
-        with open(probe, "w"):
-            pass
-        os.remove(probe)
-        return pkg
-    except OSError:
-        d = os.path.join(tempfile.gettempdir(), f"zinfer_amd-lib-{os.getuid()}")
-        os.makedirs(d, exist_ok=True)
-        return d
+    global _lib_dir
+    if _lib_dir is not None:
+        return _lib_dir
+    with _dir_lock:
+        if _lib_dir is not None:
+            return _lib_dir
+        pkg = os.path.join(os.path.dirname(CSRC), "_lib")
+        try:
+            os.makedirs(pkg, exist_ok=True)
+            fd, probe = tempfile.mkstemp(prefix=".w", dir=pkg)
+            os.close(fd)
+            os.remove(probe)
+            _lib_dir = pkg
+        except OSError:
+            d = os.path.join(tempfile.gettempdir(), f"zinfer_amd-lib-{os.getuid()}")
+            os.makedirs(d, exist_ok=True)
+            _lib_dir = d
+        return _lib_dir
 
 
 def _paths(module: str, directory: Optional[str] = None):
