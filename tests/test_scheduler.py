@@ -1,0 +1,169 @@
+"""The scheduler's decisions, with a stand-in for the engine (the cache manager is the real
+one): admission, portions under the token budget, decode, finish and free, and what happens
+when pages run out."""
+import numpy as np
+import pytest
+import torch
+
+from zinfer_amd import CacheFull
+from zinfer_amd.cache import CacheManager
+from zinfer_amd.engine.scheduler import Scheduler
+from zinfer_amd.parts import KVNeed
+from zinfer_amd.sampling import SamplingParams
+
+V = 50
+
+
+class FakeEngine:
+    """Keeps the real cache manager; logits put all weight on (last token + 1) % V, so that
+    generation is predictable and does not depend on the batch."""
+
+    class _Spec:
+        vocab_size = V
+        max_positions = 1000
+        eos_token_ids = ()
+
+    class _Model:
+        pass
+
+    def __init__(self, num_pages, page_size=4, max_requests=8):
+        self.cache = CacheManager([KVNeed(1, 4)], [None], page_size, num_pages, max_requests,
+                                  torch.float32, "cpu")
+        self.model = self._Model()
+        self.model.spec = self._Spec()
+        self.log = []
+
+    def step(self, entries, end=()):
+        self.log.append([(e.request_id, len(e.tokens), list(e.want)) for e in entries])
+        rows = []
+        for e in entries:
+            if not self.cache.has_request(e.request_id):
+                self.cache.add_request(e.request_id)
+            new_len = self.cache.length(e.request_id) + len(e.tokens)
+            self.cache.reserve(e.request_id, new_len)
+            self.cache.commit(e.request_id, new_len)
+            for w in e.want:
+                row = np.zeros(V, np.float32)
+                row[(e.tokens[w] + 1) % V] = 10.0
+                rows.append(row)
+        self.cache.check()
+        return torch.from_numpy(np.stack(rows)) if rows else torch.zeros((0, V))
+
+    def argmax(self, logits):
+        return torch.argmax(logits, dim=-1).tolist()
+
+
+GREEDY = dict(temperature=0.0, ignore_eos=True)
+
+
+def test_whole_prompt_then_decode_no_wasted_forward():
+    eng = FakeEngine(num_pages=16)
+    s = Scheduler(eng, max_step_tokens=64)
+    rid = s.add_request([3, 4, 5], SamplingParams(max_new_tokens=4, **GREEDY))
+    out = s.run()
+    assert out[rid].generated == [6, 7, 8, 9] and out[rid].finish_reason == "length"
+    # one prefill step and three decode steps: the fourth token needs no forward of its own
+    assert [len(st) for st in eng.log] == [1, 1, 1, 1] and eng.log[0][0][1] == 3
+    assert eng.cache.num_free_pages() == [16] and not eng.cache.requests
+
+
+def test_portions_under_the_token_budget_and_mixed_steps():
+    eng = FakeEngine(num_pages=64)
+    s = Scheduler(eng, max_step_tokens=10, chunk_size=6)
+    a = s.add_request(list(range(1, 15)), SamplingParams(max_new_tokens=3, **GREEDY))   # 14 tokens
+    b = s.add_request([7, 8], SamplingParams(max_new_tokens=5, **GREEDY))
+    s.run()
+    # step 0: a gets a portion of 6, b its 2 tokens (budget 10); b samples, a does not
+    assert eng.log[0] == [(a, 6, []), (b, 2, [1])]
+    # step 1: b decodes (1 token, first), a's next portion of 6 beside it
+    assert eng.log[1] == [(b, 1, [0]), (a, 6, [])]
+    # step 2: a's last 2 prompt tokens reach the end of its prompt -> it samples
+    assert eng.log[2] == [(b, 1, [0]), (a, 2, [1])]
+    for st in eng.log:
+        assert sum(n for _, n, _ in st) <= 10
+    assert s.finished[a].generated == [15, 16, 17] and s.finished[b].generated == [9, 10, 11, 12, 13]
+
+
+def test_first_come_first_served_and_max_seqs():
+    eng = FakeEngine(num_pages=64)
+    s = Scheduler(eng, max_step_tokens=100, max_seqs=2)
+    ids = [s.add_request([i + 1], SamplingParams(max_new_tokens=2, **GREEDY)) for i in range(4)]
+    s.step()
+    assert [r.id for r in s.running] == ids[:2] and [r.id for r in s.waiting] == ids[2:]
+    s.run()
+    order = [rid for st in eng.log for rid, _, _ in st]
+    assert order.index(ids[2]) > order.index(ids[1])
+    assert all(s.finished[i].generated == [i + 2, i + 3] for i in range(4))
+
+
+def test_eos_is_neither_stored_nor_counted():
+    eng = FakeEngine(num_pages=16)
+    s = Scheduler(eng, max_step_tokens=32, eos_token_ids=(8,))
+    a = s.add_request([5], SamplingParams(temperature=0.0, max_new_tokens=10))
+    b = s.add_request([5], SamplingParams(temperature=0.0, max_new_tokens=10, ignore_eos=True))
+    c = s.add_request([5], SamplingParams(temperature=0.0, max_new_tokens=10, stop_token_ids=(7,)))
+    s.run()
+    assert s.finished[a].generated == [6, 7] and s.finished[a].finish_reason == "eos"
+    assert len(s.finished[b].generated) == 10
+    assert s.finished[c].generated == [6]
+
+
+def test_admission_waits_for_pages():
+    eng = FakeEngine(num_pages=4, page_size=4)          # 16 tokens of cache
+    s = Scheduler(eng, max_step_tokens=64)
+    a = s.add_request(list(range(1, 11)), SamplingParams(max_new_tokens=2, **GREEDY))  # 3 pages
+    b = s.add_request(list(range(1, 9)), SamplingParams(max_new_tokens=2, **GREEDY))   # 2 pages
+    s.step()
+    assert [r.id for r in s.running] == [a] and [r.id for r in s.waiting] == [b]
+    s.run()
+    assert s.n_preemptions == 0
+    assert s.finished[a].generated == [11, 12] and s.finished[b].generated == [9, 10]
+
+
+def test_out_of_pages_preempts_the_newest_and_recomputes():
+    eng = FakeEngine(num_pages=4, page_size=4)
+    s = Scheduler(eng, max_step_tokens=64)
+    a = s.add_request([1, 2, 3, 4, 5, 6, 7], SamplingParams(max_new_tokens=6, **GREEDY))
+    b = s.add_request([21, 22, 23, 24, 25, 26, 27], SamplingParams(max_new_tokens=6, **GREEDY))
+    s.run()
+    assert s.n_preemptions >= 1 and s.finished[b].preemptions >= 1 and s.finished[a].preemptions == 0
+    assert s.finished[a].generated == [8, 9, 10, 11, 12, 13]
+    assert s.finished[b].generated == [28, 29, 30, 31, 32, 33]     # unchanged by the preemption
+    # after the preemption b came back with prompt + generated as one portion
+    recompute = [st for st in eng.log if any(rid == b and n > 7 for rid, n, _ in st)]
+    assert recompute, "b must have recomputed its prompt and generated tokens"
+    assert eng.cache.num_free_pages() == [4]
+
+
+def test_a_request_that_cannot_fit_alone_raises_cache_full():
+    eng = FakeEngine(num_pages=2, page_size=4)
+    s = Scheduler(eng, max_step_tokens=64)
+    s.add_request(list(range(1, 12)), SamplingParams(max_new_tokens=2, **GREEDY))
+    with pytest.raises(CacheFull):
+        s.run()
+    eng2 = FakeEngine(num_pages=2, page_size=4)
+    s2 = Scheduler(eng2, max_step_tokens=64)
+    s2.add_request([1, 2, 3, 4, 5, 6, 7], SamplingParams(max_new_tokens=5, **GREEDY))
+    with pytest.raises(CacheFull):
+        s2.run()                                    # grows beyond the pool while decoding
+
+
+def test_sampled_output_does_not_depend_on_the_batch():
+    def run(n_others):
+        eng = FakeEngine(num_pages=64)
+        # flat logits: the random stream alone decides
+        eng.step_orig = eng.step
+
+        def flat(entries, end=()):
+            out = eng.step_orig(entries, end)
+            return torch.zeros_like(out)
+        eng.step = flat
+        s = Scheduler(eng, max_step_tokens=64)
+        rid = s.add_request([1, 2], SamplingParams(temperature=1.0, seed=9, max_new_tokens=8,
+                                                   ignore_eos=True))
+        for i in range(n_others):
+            s.add_request([3 + i], SamplingParams(temperature=1.0, seed=9, max_new_tokens=5,
+                                                  ignore_eos=True))
+        return s.run()[rid].generated
+    assert run(0) == run(3)
+    assert len(set(run(0))) > 1

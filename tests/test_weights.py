@@ -1,0 +1,145 @@
+"""Weights: the safetensors container and its errors, binding by name with one error that
+lists everything wrong, dtype policy, the random-weights mode."""
+import json
+import struct
+
+import pytest
+import torch
+
+import tiny
+from zinfer_amd import FormatError, WeightError
+from zinfer_amd.models.build import build_model, declare_tensors
+from zinfer_amd.weights import (SafetensorsFile, draw_tensors, load_tensors, write_model_dir,
+                                write_safetensors)
+
+
+def _container(header: dict, payload: bytes = b"", raw_header: bytes = None) -> bytes:
+    blob = raw_header if raw_header is not None else json.dumps(header).encode()
+    return struct.pack("<Q", len(blob)) + blob + payload
+
+
+def test_round_trip_and_reference_vectors(tmp_path):
+    """A synthetic two-tensor file as in the reference's test (src/format/safetensors.zig:
+    339-376); bfloat16 [1.0, -2.5] reads back exactly (src/tensor/storage/store.zig:525-560)."""
+    p = str(tmp_path / "m.safetensors")
+    t = {"a": torch.tensor([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]]),
+         "b": torch.tensor([1.0, -2.5], dtype=torch.bfloat16),
+         "ids": torch.arange(5, dtype=torch.int64)}
+    write_safetensors(p, t, metadata={"format": "pt"})
+    with SafetensorsFile(p) as f:
+        assert f.metadata == {"format": "pt"}
+        assert f.infos["a"].dtype == "F32" and f.infos["a"].shape == (2, 3)
+        assert f.infos["b"].dtype == "BF16"
+        for k in t:
+            assert torch.equal(f.tensor(k), t[k])
+    from safetensors.torch import load_file       # an independent reader agrees
+    other = load_file(p)
+    assert all(torch.equal(other[k], t[k]) for k in t)
+
+
+@pytest.mark.parametrize("code,blob", [
+    ("InvalidSafetensorsFile", b"\x01\x02"),
+    ("InvalidHeaderLength", struct.pack("<Q", 100) + b"{}"),
+    ("HeaderTooLarge", struct.pack("<Q", 1 << 40) + b"{}"),
+    ("InvalidHeaderJson", _container({}, raw_header=b"[1]")),
+    ("InvalidHeaderJson", _container({}, raw_header=b"{not json")),
+    ("InvalidMetadataEntry", _container({"__metadata__": {"a": 1}})),
+    ("InvalidTensorEntry", _container({"t": 5})),
+    ("MissingTensorField", _container({"t": {"dtype": "F32", "shape": [1]}})),
+    ("InvalidTensorField", _container({"t": {"dtype": "F32", "shape": [1], "data_offsets": [0]}})),
+    ("InvalidTensorField", _container({"t": {"dtype": 3, "shape": [1], "data_offsets": [0, 4]}})),
+    ("UnsupportedDType", _container({"t": {"dtype": "F128", "shape": [1], "data_offsets": [0, 4]}})),
+    ("InvalidIntegerValue", _container({"t": {"dtype": "F32", "shape": [-1], "data_offsets": [0, 4]}})),
+    ("InvalidDataOffsets", _container({"t": {"dtype": "F32", "shape": [1], "data_offsets": [4, 0]}}, b"\0" * 4)),
+    ("TensorOutOfBounds", _container({"t": {"dtype": "F32", "shape": [2], "data_offsets": [0, 8]}}, b"\0" * 4)),
+    ("TensorByteSizeMismatch", _container({"t": {"dtype": "F32", "shape": [2], "data_offsets": [0, 4]}}, b"\0" * 4)),
+    ("OverlappingTensorData", _container({"a": {"dtype": "F32", "shape": [2], "data_offsets": [0, 8]},
+                                          "b": {"dtype": "F32", "shape": [1], "data_offsets": [4, 8]}}, b"\0" * 8)),
+    ("NonContiguousTensorData", _container({"a": {"dtype": "F32", "shape": [1], "data_offsets": [4, 8]}}, b"\0" * 8)),
+    ("NonContiguousTensorData", _container({"a": {"dtype": "F32", "shape": [1], "data_offsets": [0, 4]}}, b"\0" * 8)),
+])
+def test_container_errors(tmp_path, code, blob):
+    """The reference's parse and layout errors (src/format/safetensors.zig:38,139-336)."""
+    p = tmp_path / "bad.safetensors"
+    p.write_bytes(blob)
+    with pytest.raises(FormatError) as e:
+        SafetensorsFile(str(p))
+    assert e.value.code == code
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    cfg = tiny.config_of("A")
+    decls = declare_tensors(cfg.model_spec())
+    tensors = draw_tensors(decls, 1, torch.bfloat16, tied=True)
+    del tensors["model.layers.1.mlp.up_proj.weight"]
+    del tensors["model.norm.weight"]
+    tensors["model.layers.0.self_attn.q_norm.weight"] = torch.ones(8, dtype=torch.bfloat16)
+    tensors["model.layers.0.self_attn.k_proj.weight"] = torch.ones(16, 64, dtype=torch.bfloat16)
+    tensors["model.layers.7.extra.weight"] = torch.ones(3)
+    (tmp_path / "config.json").write_text(json.dumps(tiny.TINY_A))
+    write_safetensors(str(tmp_path / "model.safetensors"), tensors)
+    with pytest.raises(WeightError) as e:
+        load_tensors(str(tmp_path), decls)
+    msg = str(e.value)
+    for needle in ("model.layers.1.mlp.up_proj.weight", "model.norm.weight", "missing (2)",
+                   "model.layers.7.extra.weight", "unexpected (1)",
+                   "model.layers.0.self_attn.q_norm.weight: expected shape [16], file has [8]",
+                   "model.layers.0.self_attn.k_proj.weight: expected shape [32, 64], file has [16, 64]"):
+        assert needle in msg, needle
+    with pytest.raises(WeightError, match="no model.safetensors"):
+        load_tensors(str(tmp_path / "x"), decls)
+
+
+def test_tied_head_is_optional_untied_is_not(tmp_path):
+    for name, tied in (("A", True), ("B", False)):
+        cfg = tiny.config_of(name)
+        decls = declare_tensors(cfg.model_spec())
+        assert decls["lm_head.weight"].optional == tied
+        tensors = draw_tensors(decls, 1, torch.float32, tied=tied)
+        assert ("lm_head.weight" in tensors) == (not tied)
+    d = tmp_path / "b"
+    write_model_dir(str(d), tiny.config_of("B"), 3)
+    t = {}
+    with SafetensorsFile(str(d / "model.safetensors")) as f:
+        t = {k: f.tensor(k) for k in f.names() if k != "lm_head.weight"}
+    write_safetensors(str(d / "model.safetensors"), t)
+    with pytest.raises(WeightError, match="lm_head.weight"):
+        load_tensors(str(d), declare_tensors(tiny.config_of("B").model_spec()))
+
+
+def test_dtypes_are_kept(tmp_path):
+    """bfloat16 stays bfloat16, a tensor stored in 32-bit stays so, integers become int32."""
+    cfg = tiny.config_of("A")
+    decls = declare_tensors(cfg.model_spec())
+    tensors = draw_tensors(decls, 1, torch.bfloat16, tied=True)
+    tensors["model.norm.weight"] = tensors["model.norm.weight"].float()
+    tensors["model.layers.0.mlp.down_proj.weight"] = \
+        tensors["model.layers.0.mlp.down_proj.weight"].float()
+    (tmp_path / "config.json").write_text(json.dumps(tiny.TINY_A))
+    write_safetensors(str(tmp_path / "model.safetensors"), tensors)
+    got = load_tensors(str(tmp_path), decls)
+    assert got["model.norm.weight"].dtype == torch.float32
+    assert got["model.layers.0.mlp.down_proj.weight"].dtype == torch.float32
+    assert got["model.embed_tokens.weight"].dtype == torch.bfloat16
+    model = build_model(cfg.model_spec(), got, "bfloat16", "cpu")
+    assert model.blocks[0].feed_forward.down.weight.dtype == torch.float32
+    assert model.blocks[1].feed_forward.down.weight.dtype == torch.bfloat16
+    assert model.blocks[0].mixer.qkv.weight.shape == (4 * 16 + 2 * 2 * 16, 64)
+    assert model.head.weight is model.embedding          # tied: the embedding is the head
+    model32 = build_model(cfg.model_spec(), got, "float32", "cpu")
+    assert model32.embedding.dtype == torch.float32
+
+
+def test_random_weights_mode(tmp_path):
+    a = write_model_dir(str(tmp_path / "a"), tiny.config_of("B"), seed=5, dtype=torch.bfloat16)
+    b = write_model_dir(str(tmp_path / "b"), tiny.config_of("B"), seed=5, dtype=torch.bfloat16)
+    c = write_model_dir(str(tmp_path / "c"), tiny.config_of("B"), seed=6, dtype=torch.bfloat16)
+    decls = declare_tensors(tiny.config_of("B").model_spec())
+    ta, tb, tc = (load_tensors(p, decls) for p in (a, b, c))
+    assert all(torch.equal(ta[k], tb[k]) for k in ta)
+    assert not torch.equal(ta["lm_head.weight"], tc["lm_head.weight"])
+    w = ta["model.layers.1.mlp.gate_proj.weight"].float()
+    assert abs(float(w.std()) - 0.02) < 0.002 and abs(float(w.mean())) < 0.001
+    g = ta["model.layers.2.self_attn.k_norm.weight"].float()
+    assert float(g.min()) >= 0.9 - 1e-2 and float(g.max()) <= 1.1 + 1e-2 and g.shape == (32,)
+    assert json.load(open(tmp_path / "a" / "config.json"))["torch_dtype"] == "bfloat16"

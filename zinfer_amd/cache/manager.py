@@ -127,13 +127,13 @@ class CacheManager:
             grp.tables[rid] = []
 
     def pages_missing(self, rid, new_len: int) -> List[int]:
-        """Pages each group would have to hand out for ``rid`` to hold ``new_len`` tokens."""
-        length = self.requests[rid]["length"] if rid in self.requests else 0
-        if rid not in self.requests:
-            return [sum(1 for i in range(grp.first_needed_page(0),
-                                         (new_len + self.page_size - 1) // self.page_size))
-                    for grp in self.groups]
-        return [grp.pages_missing(rid, length, new_len) for grp in self.groups]
+        """Pages each group would have to hand out for ``rid`` (live or not yet) to hold
+        ``new_len`` tokens."""
+        if rid in self.requests:
+            length = self.requests[rid]["length"]
+            return [grp.pages_missing(rid, length, new_len) for grp in self.groups]
+        last = (new_len + self.page_size - 1) // self.page_size
+        return [last - grp.first_needed_page(0) for grp in self.groups]
 
     def can_reserve(self, wanted: Sequence[Tuple[object, int]]) -> bool:
         """Whether all ``(request, new_len)`` of a step fit together."""
