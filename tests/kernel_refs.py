@@ -59,22 +59,23 @@ def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, cos, sin, positions, slot_ma
         qkv[:, :qw] = q.reshape(T, qw).to(qkv.dtype)
     if slot_mapping is not None:
         kp = k_pool.view(-1, n_kv_heads, page_size, hd)
-        vp = v_pool.view(-1, n_kv_heads, page_size, hd)
+        vp = v_pool.view(-1, n_kv_heads, hd, page_size)     # values: rows of a page contiguous
         page = (slot_mapping // page_size).long()
         row = (slot_mapping % page_size).long()
         kp[page, :, row] = k.to(kp.dtype)
-        vp[page, :, row] = v.to(vp.dtype)
+        vp[page, :, :, row] = v.to(vp.dtype)
     else:
         qkv[:, qw:qw + kw] = k.reshape(T, kw).to(qkv.dtype)
 
 
 def paged_attention(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index, out, scale,
-                    window, n_heads, n_kv_heads, head_dim, page_size, max_q_len, max_ctx_len):
+                    window, n_heads, n_kv_heads, head_dim, page_size, max_q_len, max_ctx_len,
+                    n_single=None):
     T = q.shape[0]
     hd = head_dim
     G = n_heads // n_kv_heads
     kp = k_pool.view(-1, n_kv_heads, page_size, hd)
-    vp = v_pool.view(-1, n_kv_heads, page_size, hd)
+    vp = v_pool.view(-1, n_kv_heads, hd, page_size)
     for t in range(T):
         s = int(seq_index[t])
         q_len = int(q_start[s + 1] - q_start[s])
@@ -85,7 +86,7 @@ def paged_attention(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index,
         assert (pages >= 0).all(), "attention would read a page that is not held"
         rows = keys % page_size
         K = kp[pages, :, rows].to(F64)      # [n, nKV, hd]
-        V = vp[pages, :, rows].to(F64)
+        V = vp[pages, :, :, rows].to(F64)
         qt = q[t].to(F64).reshape(n_heads, hd)
         Kx = K.repeat_interleave(G, dim=1)  # [n, nH, hd]
         Vx = V.repeat_interleave(G, dim=1)

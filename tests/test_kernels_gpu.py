@@ -93,6 +93,23 @@ def test_gemm(a_dtype, w_dtype, o_dtype, M, N, K):
     assert rel_err(got, want) <= tol(o_dtype)
 
 
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 64, 65, 130, 300, 517])
+@pytest.mark.parametrize("N,K", [(1000, 136), (96, 64), (777, 320), (4100, 4096), (256, 1032)])
+@pytest.mark.parametrize("o_dtype,accumulate", [(torch.bfloat16, False), (torch.float32, False),
+                                                (torch.float32, True)])
+def test_gemm_bf16_mfma_paths(M, N, K, o_dtype, accumulate):
+    """The bfloat16 MFMA kernels (weight streaming up to 64 rows, tiled above) at sizes that
+    are no multiples of their tiles, with each epilogue."""
+    a = _rand((M, K), torch.bfloat16, 20)
+    w = _rand((N, K), torch.bfloat16, 21, 0.05)
+    base = _rand((M, N), torch.float32, 22).to(o_dtype)
+    want = base.clone()
+    ref.gemm(a, w, want, accumulate)
+    got = base.clone().to(DEV)
+    _ops().gemm(a.to(DEV), w.to(DEV), got, accumulate)
+    assert rel_err(got, want) <= (tol(o_dtype) if not accumulate else 2e-5)
+
+
 @pytest.mark.parametrize("a_dtype", DTYPES)
 def test_gemm_accumulate_and_one_hot(a_dtype):
     """out += a w^T in 32-bit; a one-hot row picks a column of W (the reference's
@@ -141,7 +158,7 @@ def _paged_setup(dtype, nH, nKV, hd, page_size, ctx_lens, q_lens, seed, num_page
     max_pages = max(pages_per)
     bt = torch.full((n, max_pages), -1, dtype=torch.int32)
     k_pool = torch.full((num_pages, nKV, page_size, hd), float("nan")).to(dtype)
-    v_pool = torch.full((num_pages, nKV, page_size, hd), float("nan")).to(dtype)
+    v_pool = torch.full((num_pages, nKV, hd, page_size), float("nan")).to(dtype)
     Ks, Vs = [], []
     cur = 0
     for s in range(n):
@@ -153,7 +170,7 @@ def _paged_setup(dtype, nH, nKV, hd, page_size, ctx_lens, q_lens, seed, num_page
             bt[s, i] = pg
             lo, hi = i * page_size, min((i + 1) * page_size, ctx_lens[s])
             k_pool[pg, :, :hi - lo] = K[lo:hi].transpose(0, 1)
-            v_pool[pg, :, :hi - lo] = V[lo:hi].transpose(0, 1)
+            v_pool[pg, :, :, :hi - lo] = V[lo:hi].permute(1, 2, 0)
     T = sum(q_lens)
     q = _rand((T, nH * hd), dtype, seed + 7)
     q_start = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
@@ -175,7 +192,8 @@ def _run_attention(s, dtype, nH, nKV, hd, page_size, window, q_lens, ctx_lens):
     d = {k: v.to(DEV) for k, v in s.items() if isinstance(v, torch.Tensor)}
     _ops().paged_attention(d["q"], d["k_pool"], d["v_pool"], d["block_table"], d["q_start"],
                            d["ctx_len"], d["seq_index"], got, scale, window, nH, nKV, hd,
-                           page_size, max(q_lens), max(ctx_lens))
+                           page_size, max(q_lens), max(ctx_lens),
+                           n_single=sum(1 for n in q_lens if n == 1))
     return got, want
 
 
@@ -192,6 +210,29 @@ def test_paged_attention_mixed_batch(dtype, nH, nKV, hd, page_size, window):
     got, want = _run_attention(s, dtype, nH, nKV, hd, page_size, window, q_lens, ctx_lens)
     assert not torch.isnan(got.float()).any(), "a slot outside the context was read"
     assert rel_err(got, want) <= tol(dtype)
+
+
+@pytest.mark.parametrize("nH,nKV,hd,page_size,window", [
+    (8, 2, 32, 16, 0), (32, 8, 128, 16, 0), (6, 6, 64, 32, 0), (16, 1, 64, 16, 0),
+    (9, 3, 256, 16, 0), (8, 2, 64, 16, 37), (4, 4, 128, 48, 300), (36, 4, 32, 16, 0)])
+@pytest.mark.parametrize("kind", ["decode", "prefill", "mixed"])
+def test_paged_attention_mfma(nH, nKV, hd, page_size, window, kind):
+    """The bfloat16 MFMA kernels: decode tokens over contexts that end at, before and after a
+    split's and a page's edge; portions that start mid-context; both in one batch."""
+    dtype = torch.bfloat16
+    if kind == "decode":
+        ctx_lens = [1, 15, 16, 17, 255, 256, 257, 600, 1025]
+        q_lens = [1] * len(ctx_lens)
+    elif kind == "prefill":
+        ctx_lens = [37, 150, 64, 129, 700, 2]
+        q_lens = [37, 50, 33, 129 - 100, 200, 2]
+    else:
+        ctx_lens = [37, 300, 1, 64, 129, 513, 16]
+        q_lens = [37, 1, 1, 5, 29, 1, 2]
+    s = _paged_setup(dtype, nH, nKV, hd, page_size, ctx_lens, q_lens, seed=9)
+    got, want = _run_attention(s, dtype, nH, nKV, hd, page_size, window, q_lens, ctx_lens)
+    assert not torch.isnan(got.float()).any(), "a slot outside the context was read"
+    assert rel_err(got, want) <= 2 * tol(dtype)     # probabilities are rounded once more
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

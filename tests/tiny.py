@@ -29,9 +29,16 @@ TINY_C = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden
               intermediate_size=112, vocab_size=777, rope_theta=50000.0, rms_norm_eps=3e-6,
               tie_word_embeddings=False, max_position_embeddings=384, torch_dtype="float32")
 
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
-PAGE_SIZE = {"A": 16, "B": 8, "C": 16}
-SEEDS = {"A": 11, "B": 22, "C": 33}
+# a fourth shape whose sizes the bfloat16 MFMA kernels cover (head_dim 64, pages of 16, widths
+# that are multiples of 8), so that those kernels run inside the engine tests as well
+TINY_D = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2,
+              hidden_size=192, num_attention_heads=6, num_key_value_heads=2, head_dim=64,
+              intermediate_size=456, vocab_size=1210, rope_theta=100000.0, rms_norm_eps=2e-6,
+              tie_word_embeddings=True, max_position_embeddings=640, torch_dtype="bfloat16")
+
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16}
+SEEDS = {"A": 11, "B": 22, "C": 33, "D": 44}
 
 
 def config_of(name: str) -> Qwen3Config:

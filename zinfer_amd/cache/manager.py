@@ -7,8 +7,10 @@ The reference keeps one contiguous buffer per request and layer, sized at creati
 that has run out.  Paging, groups and slots are this engine's own.
 
 Layout of a group's pool, per run of a layer: keys ``[num_pages, n_kv_heads, page_size,
-head_dim]`` and values the same; token ``p`` of a request lies in page
-``table[p // page_size]`` at row ``p % page_size``.
+head_dim]`` and values ``[num_pages, n_kv_heads, head_dim, page_size]`` (the positions of a
+page contiguous, as the attention kernels' second matrix product reads them); token ``p`` of
+a request lies in page ``table[p // page_size]`` at row ``p % page_size``.  The manager only
+hands out pages; the layout inside a page belongs to the kernels.
 """
 from __future__ import annotations
 

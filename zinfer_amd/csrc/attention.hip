@@ -1,6 +1,7 @@
 // Causal grouped-query attention over a paged cache.
 //
-// Pools are laid out [page, kv head, row, hd]; token p of a sequence lies in page
+// The key pool is laid out [page, kv head, row, hd], the value pool [page, kv head, hd, row]
+// (rows of a page contiguous); token p of a sequence lies in page
 // block_table[seq][p / page_size], row p % page_size.  A token at position p attends to the
 // positions lo..p of its own sequence, lo = 0 or p - window + 1 (src/kernel/attention/
 // basic.zig:27-76 of the reference: scores scaled after the dot product, softmax with the
@@ -20,7 +21,7 @@ __global__ __launch_bounds__(ZF_WAVE) void paged_attention_wave_kernel(
   extern __shared__ float smem[];  // q: hd floats, p: 64 floats, acc handled in registers
   float* qs = smem;
   float* ps = smem + hd;
-  int* rows = (int*)(ps + ZF_WAVE);  // element offset of each key's row in the pool / hd
+  int* rows = (int*)(ps + ZF_WAVE);  // (page * nKV + kvh) * page_size + row of each key
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int s = seq_index[t];
   const int q_len = q_start[s + 1] - q_start[s];
@@ -65,11 +66,12 @@ __global__ __launch_bounds__(ZF_WAVE) void paged_attention_wave_kernel(
     for (int i = 0; i < 8; ++i) acc[i] *= corr;
     for (int j = 0; j < nk; ++j) {
       const float pj = ps[j];
-      const T* vr = v_pool + (size_t)rows[j] * hd;
+      const int rj = rows[j];
+      const T* vr = v_pool + (size_t)(rj / page_size) * page_size * hd + rj % page_size;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const int d = lane + i * ZF_WAVE;
-        if (d < hd) acc[i] = fmaf(pj, load_as_float<T>(vr + d), acc[i]);
+        if (d < hd) acc[i] = fmaf(pj, load_as_float<T>(vr + (size_t)d * page_size), acc[i]);
       }
     }
   }
@@ -101,5 +103,388 @@ extern "C" int zf_paged_attention_wave(const void* q, const void* k_pool, const 
                        (const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool,
                        block_table, q_start, ctx_len, seq_index, (bf16_t*)out, scale, window, nH,
                        nKV, hd, page_size, max_pages);
+  ZF_CHECK_LAUNCH();
+}
+
+// =====================================================================================
+//  bfloat16 MFMA kernels.  Both compute the transposed score tile S^T = K Q^T, so that a
+//  lane's score registers all belong to one query (its column): the soft-max runs in
+//  registers, the probabilities are already in the operand order of the second product
+//  O^T = V^T P^T, and the output accumulators of a lane belong to that same query, so the
+//  running rescale is a per-lane factor.  V^T is what the value pool stores
+//  ([page, kv head, hd, row]).  No LDS is used; K, V and Q go from global memory (L2) straight
+//  into MFMA operands.  page_size must be a multiple of 16, hd one of 32, 64, 128, 256.
+//  Soft-max in 32-bit with exp2 and the scale folded into the exponent.
+// =====================================================================================
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
+}
+
+// keeps elements [n_lo, n_hi) of the 4 bfloat16 in v (element 0 in the low bits), zeroes the rest
+__device__ __forceinline__ u32x2_t keep_range4(u32x2_t v, int n_lo, int n_hi) {
+  uint64_t x = ((uint64_t)v[1] << 32) | v[0];
+  n_lo = max(0, min(4, n_lo));
+  n_hi = max(0, min(4, n_hi));
+  uint64_t m = 0;
+  if (n_hi > n_lo) {
+    const uint64_t hi = n_hi == 4 ? ~0ull : ((1ull << (16 * n_hi)) - 1);
+    const uint64_t lo = (1ull << (16 * n_lo)) - 1;
+    m = hi & ~lo;
+  }
+  x &= m;
+  return u32x2_t{(uint32_t)x, (uint32_t)(x >> 32)};
+}
+
+// ---------------------------------------------------------------- decode: one query token
+// Grid (sequence, kv head, split).  A split covers the keys [split * split_keys,
+// (split + 1) * split_keys) of the context, so which keys a split holds depends on the
+// context length only.  One wave per workgroup: the G query heads of the kv head are the
+// columns of 16x16x32 MFMAs (G <= 16).  Each split writes an un-normalised partial
+// (max, sum, O[G, hd]); attn_decode_merge_kernel combines the splits in split order.
+template <int HD>
+__global__ __launch_bounds__(64) void attn_decode_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool,
+    const bf16_t* __restrict__ v_pool, const int* __restrict__ block_table,
+    const int* __restrict__ q_start, const int* __restrict__ ctx_len, float* __restrict__ ws_o,
+    float* __restrict__ ws_ml, float scale_log2e, int window, int nH, int nKV, int ps,
+    int max_pages, int max_splits, int split_keys) {
+  const int s = blockIdx.x, kvh = blockIdx.y, sp = blockIdx.z;
+  if (q_start[s + 1] - q_start[s] != 1) return;
+  const int ctx = ctx_len[s], pos = ctx - 1;
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int k_begin = max(lo, sp * split_keys), k_end = min(ctx, (sp + 1) * split_keys);
+  if (k_begin >= k_end) return;
+  const int G = nH / nKV;
+  const int lane = threadIdx.x, j = lane % 16, qd = lane / 16;
+  const int t = q_start[s];
+  const int* table = block_table + (size_t)s * max_pages;
+
+  bf16x8_t qf[HD / 32];
+  {
+    const bf16_t* qrow = q + ((size_t)t * nH + kvh * G + min(j, G - 1)) * HD + 8 * qd;
+#pragma unroll
+    for (int st = 0; st < HD / 32; ++st) {
+      u32x4_t v = *(const u32x4_t*)(qrow + st * 32);
+      if (j >= G) v = u32x4_t{0, 0, 0, 0};
+      qf[st] = *(bf16x8_t*)&v;
+    }
+  }
+  f32x4_t o[HD / 16];
+#pragma unroll
+  for (int dt = 0; dt < HD / 16; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  for (int kb = (k_begin / 32) * 32; kb < k_end; kb += 32) {
+    f32x4_t st[2];
+    int page[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      // the 16 keys kb + 16 h .. + 15 lie in one page; a half outside [k_begin, k_end) may have
+      // no page at all: read the page of a key that certainly exists and mask everything
+      const int base = kb + 16 * h;
+      const bool any = base < k_end && base + 16 > k_begin;
+      const int safe = any ? max(base, k_begin) : k_begin;
+      page[h] = table[safe / ps];
+      const int key = min(max(base + j, k_begin), k_end - 1);
+      const int kpage = any ? page[h] : table[key / ps];
+      const bf16_t* krow = k_pool + (((size_t)kpage * nKV + kvh) * ps + key % ps) * HD + 8 * qd;
+      st[h] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int stp = 0; stp < HD / 32; ++stp) {
+        const u32x4_t kv = *(const u32x4_t*)(krow + stp * 32);
+        st[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&kv, qf[stp], st[h], 0,
+                                                        0, 0);
+      }
+    }
+    // st[h][r]: key kb + 16 h + 4 qd + r, query column j
+    float sc[8];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int key = kb + 16 * h + 4 * qd + r;
+        const float v = (key >= k_begin && key < k_end) ? st[h][r] * scale_log2e : -INFINITY;
+        sc[h * 4 + r] = v;
+        tmax = fmaxf(tmax, v);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m, tmax);
+    const float corr = exp2f(m - m_new);
+    float psum = 0.f;
+    float p[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      p[e] = exp2f(sc[e] - m_new);
+      psum += p[e];
+    }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * corr + psum;
+    m = m_new;
+    u32x4_t pk = u32x4_t{pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]),
+                         pack_bf16(p[6], p[7])};
+    const bf16x8_t pf = *(bf16x8_t*)&pk;
+    // V^T operand: row d = 16 dt + j, keys kb + 16 h + 4 qd .. + 3 for h = 0, 1
+    const bf16_t* vb[2];
+    int n_lo[2], n_hi[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int base = kb + 16 * h + 4 * qd;
+      n_lo[h] = k_begin - base;
+      n_hi[h] = k_end - base;
+      const int off = (kb + 16 * h) % ps + 4 * qd;
+      vb[h] = v_pool + ((size_t)page[h] * nKV + kvh) * ps * HD + (size_t)j * ps + off;
+    }
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt) {
+      u32x2_t v0 = *(const u32x2_t*)(vb[0] + (size_t)dt * 16 * ps);
+      u32x2_t v1 = *(const u32x2_t*)(vb[1] + (size_t)dt * 16 * ps);
+      v0 = keep_range4(v0, n_lo[0], n_hi[0]);
+      v1 = keep_range4(v1, n_lo[1], n_hi[1]);
+      u32x4_t vv = u32x4_t{v0[0], v0[1], v1[0], v1[1]};
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[dt][r] *= corr;
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8_t*)&vv, pf, o[dt], 0, 0, 0);
+    }
+  }
+  if (j < G) {
+    const int head = kvh * G + j;
+    const size_t slot = ((size_t)s * nH + head) * max_splits + sp;
+    float* dst = ws_o + slot * HD;
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) dst[dt * 16 + 4 * qd + r] = o[dt][r];
+    if (qd == 0) {
+      ws_ml[slot * 2] = m;
+      ws_ml[slot * 2 + 1] = l;
+    }
+  }
+}
+
+// Combines the splits of one (sequence, head) in split order and writes bfloat16.
+__global__ void attn_decode_merge_kernel(const float* __restrict__ ws_o,
+                                         const float* __restrict__ ws_ml,
+                                         const int* __restrict__ q_start,
+                                         const int* __restrict__ ctx_len, bf16_t* __restrict__ out,
+                                         int window, int nH, int hd, int max_splits,
+                                         int split_keys) {
+  const int s = blockIdx.x, head = blockIdx.y;
+  if (q_start[s + 1] - q_start[s] != 1) return;
+  const int ctx = ctx_len[s], pos = ctx - 1;
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int first = lo / split_keys, last = pos / split_keys;
+  const size_t base = ((size_t)s * nH + head) * max_splits;
+  float mx = -INFINITY;
+  for (int sp = first; sp <= last; ++sp) mx = fmaxf(mx, ws_ml[(base + sp) * 2]);
+  float denom = 0.f;
+  for (int sp = first; sp <= last; ++sp)
+    denom += exp2f(ws_ml[(base + sp) * 2] - mx) * ws_ml[(base + sp) * 2 + 1];
+  const float inv = 1.0f / denom;
+  bf16_t* orow = out + ((size_t)q_start[s] * nH + head) * hd;
+  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+    float acc = 0.f;
+    for (int sp = first; sp <= last; ++sp)
+      acc += exp2f(ws_ml[(base + sp) * 2] - mx) * ws_o[(base + sp) * hd + d];
+    orow[d] = float_to_bf16(acc * inv);
+  }
+}
+
+extern "C" int zf_attn_decode_bf16(const void* q, const void* k_pool, const void* v_pool,
+                                   const int* block_table, const int* q_start,
+                                   const int* ctx_len, void* out, float* ws_o, float* ws_ml,
+                                   float scale, int window, int n_seqs, int nH, int nKV, int hd,
+                                   int page_size, int max_pages, int max_splits, int split_keys,
+                                   hipStream_t stream) {
+  if (n_seqs <= 0) return 0;
+  if (page_size % 16 != 0 || nKV <= 0 || nH % nKV != 0 || nH / nKV > 16 || split_keys % 32 != 0)
+    return -2;
+  const float scale_log2e = scale * 1.4426950408889634f;
+  dim3 grid(n_seqs, nKV, max_splits);
+#define ZF_DEC(HD)                                                                              \
+  hipLaunchKernelGGL(attn_decode_kernel<HD>, grid, dim3(64), 0, stream, (const bf16_t*)q,       \
+                     (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, q_start,        \
+                     ctx_len, ws_o, ws_ml, scale_log2e, window, nH, nKV, page_size, max_pages,  \
+                     max_splits, split_keys)
+  if (hd == 32) ZF_DEC(32);
+  else if (hd == 64) ZF_DEC(64);
+  else if (hd == 128) ZF_DEC(128);
+  else if (hd == 256) ZF_DEC(256);
+  else return -2;
+#undef ZF_DEC
+  hipLaunchKernelGGL(attn_decode_merge_kernel, dim3(n_seqs, nH), dim3(64), 0, stream, ws_o, ws_ml,
+                     q_start, ctx_len, (bf16_t*)out, window, nH, hd, max_splits, split_keys);
+  ZF_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------- prefill: portions of prompts
+// Grid (sequence, tile of 32 queries, kv head); wave w of a workgroup takes the query heads
+// w, w + waves, ... of the kv head.  32x32x16 MFMAs: S^T tile of 32 keys x 32 queries,
+// O^T tiles of 32 head elements x 32 queries.  A query at position p reads keys lo..p; a
+// portion may start anywhere in the context (earlier pages plus its own tokens).
+// Sequences with a single query token are left to the decode kernel when skip_single is set.
+template <int HD>
+__global__ __launch_bounds__(512) void attn_prefill_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool,
+    const bf16_t* __restrict__ v_pool, const int* __restrict__ block_table,
+    const int* __restrict__ q_start, const int* __restrict__ ctx_len, bf16_t* __restrict__ out,
+    float scale_log2e, int window, int nH, int nKV, int ps, int max_pages, int skip_single) {
+  const int s = blockIdx.x, qt = blockIdx.y, kvh = blockIdx.z;
+  const int q_len = q_start[s + 1] - q_start[s];
+  if (q_len == 1 && skip_single) return;
+  const int qbase = qt * 32;
+  if (qbase >= q_len) return;
+  const int ctx = ctx_len[s];
+  const int pos0 = ctx - q_len + qbase;              // position of the tile's first query
+  const int nq = min(32, q_len - qbase);
+  const int p_max = pos0 + nq - 1;
+  const int G = nH / nKV;
+  const int wave = threadIdx.x / 64, nwaves = blockDim.x / 64;
+  const int lane = threadIdx.x % 64, j = lane % 32, hf = lane / 32;
+  const bool q_valid = j < nq;
+  const int p_j = pos0 + min(j, nq - 1);
+  const int lo_j = (window > 0 && p_j - window + 1 > 0) ? p_j - window + 1 : 0;
+  const int lo_min = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int* table = block_table + (size_t)s * max_pages;
+  const int t_row = q_start[s] + qbase + min(j, nq - 1);
+
+  for (int g = wave; g < G; g += nwaves) {
+    const int head = kvh * G + g;
+    bf16x8_t qf[HD / 16];
+    {
+      const bf16_t* qrow = q + ((size_t)t_row * nH + head) * HD + 8 * hf;
+#pragma unroll
+      for (int st = 0; st < HD / 16; ++st) {
+        u32x4_t v = *(const u32x4_t*)(qrow + st * 16);
+        if (!q_valid) v = u32x4_t{0, 0, 0, 0};
+        qf[st] = *(bf16x8_t*)&v;
+      }
+    }
+    f32x16_t o[HD / 32];
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    for (int kb = (lo_min / 32) * 32; kb <= p_max; kb += 32) {
+      // S^T: rows are the keys kb + (lane % 32), clamped into the keys that exist
+      f32x16_t st;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) st[r] = 0.f;
+      {
+        const int key = min(max(kb + j, lo_min), p_max);
+        const int kpage = table[key / ps];
+        const bf16_t* krow = k_pool + (((size_t)kpage * nKV + kvh) * ps + key % ps) * HD + 8 * hf;
+#pragma unroll
+        for (int stp = 0; stp < HD / 16; ++stp) {
+          const u32x4_t kv = *(const u32x4_t*)(krow + stp * 16);
+          st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&kv, qf[stp], st, 0, 0, 0);
+        }
+      }
+      // st[r]: key kb + 8 (r / 4) + 4 hf + r % 4, query column j
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = kb + 8 * (r / 4) + 4 * hf + r % 4;
+        const float v = (key <= p_j && key >= lo_j) ? st[r] * scale_log2e : -INFINITY;
+        st[r] = v;
+        tmax = fmaxf(tmax, v);
+      }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(m, tmax);
+      // a query whose window lies wholly beyond this tile has no key here yet
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float corr = exp2f(m - m_use);
+      float psum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        st[r] = exp2f(st[r] - m_use);
+        psum += st[r];
+      }
+      psum += __shfl_xor(psum, 32, 64);
+      l = l * corr + psum;
+      m = m_new;
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[dt][r] *= corr;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        // keys kb + 16 u .. + 15 (one page); slots e = 0..7 <-> st[8 u + e]:
+        // keys kb + 16 u + 4 hf + e (e < 4) and kb + 16 u + 8 + 4 hf + (e - 4)
+        u32x4_t pk = u32x4_t{pack_bf16(st[8 * u + 0], st[8 * u + 1]),
+                             pack_bf16(st[8 * u + 2], st[8 * u + 3]),
+                             pack_bf16(st[8 * u + 4], st[8 * u + 5]),
+                             pack_bf16(st[8 * u + 6], st[8 * u + 7])};
+        const bf16x8_t pf = *(bf16x8_t*)&pk;
+        const int base = kb + 16 * u;
+        const bool any = base <= p_max && base + 16 > lo_min;
+        const int safe = any ? max(base, lo_min) : p_max;
+        const int vpage = table[safe / ps];
+        const int off = base % ps + 4 * hf;
+        const bf16_t* vb = v_pool + ((size_t)vpage * nKV + kvh) * ps * HD + (size_t)j * ps + off;
+        // keys at or beyond ctx hold nothing of this request; keys below lo_min may lie in
+        // a page that was given back: both are zeroed (0 * NaN would poison the sum)
+        const int a0 = base + 4 * hf, a1 = a0 + 8;
+        const int hi_lim = any ? ctx : 0;
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt) {
+          u32x2_t v0 = *(const u32x2_t*)(vb + (size_t)dt * 32 * ps);
+          u32x2_t v1 = *(const u32x2_t*)(vb + (size_t)dt * 32 * ps + 8);
+          v0 = keep_range4(v0, lo_min - a0, hi_lim - a0);
+          v1 = keep_range4(v1, lo_min - a1, hi_lim - a1);
+          u32x4_t vv = u32x4_t{v0[0], v0[1], v1[0], v1[1]};
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8_t*)&vv, pf, o[dt], 0, 0, 0);
+        }
+      }
+    }
+    if (q_valid) {
+      const float inv = 1.0f / l;
+      bf16_t* orow = out + ((size_t)t_row * nH + head) * HD;
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+          const int d = dt * 32 + 8 * r4 + 4 * hf;
+          u32x2_t w = u32x2_t{pack_bf16(o[dt][r4 * 4 + 0] * inv, o[dt][r4 * 4 + 1] * inv),
+                              pack_bf16(o[dt][r4 * 4 + 2] * inv, o[dt][r4 * 4 + 3] * inv)};
+          *(u32x2_t*)(orow + d) = w;
+        }
+    }
+  }
+}
+
+extern "C" int zf_attn_prefill_bf16(const void* q, const void* k_pool, const void* v_pool,
+                                    const int* block_table, const int* q_start,
+                                    const int* ctx_len, void* out, float scale, int window,
+                                    int n_seqs, int max_q_len, int nH, int nKV, int hd,
+                                    int page_size, int max_pages, int skip_single,
+                                    hipStream_t stream) {
+  if (n_seqs <= 0 || max_q_len <= 0) return 0;
+  if (page_size % 16 != 0 || nKV <= 0 || nH % nKV != 0) return -2;
+  const float scale_log2e = scale * 1.4426950408889634f;
+  const int G = nH / nKV;
+  dim3 grid(n_seqs, (max_q_len + 31) / 32, nKV);
+  dim3 block(64 * (G < 8 ? G : 8));
+#define ZF_PRE(HD)                                                                              \
+  hipLaunchKernelGGL(attn_prefill_kernel<HD>, grid, block, 0, stream, (const bf16_t*)q,         \
+                     (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, q_start,        \
+                     ctx_len, (bf16_t*)out, scale_log2e, window, nH, nKV, page_size, max_pages, \
+                     skip_single)
+  if (hd == 32) ZF_PRE(32);
+  else if (hd == 64) ZF_PRE(64);
+  else if (hd == 128) ZF_PRE(128);
+  else if (hd == 256) ZF_PRE(256);
+  else return -2;
+#undef ZF_PRE
   ZF_CHECK_LAUNCH();
 }

@@ -62,8 +62,11 @@ extern "C" int zf_rmsnorm(const float* x, const float* gain, void* out, int out_
 //   q, k: optional RMSNorm over the head (cpu.zig:50-71), optional half-split rotation
 //         (x_i, x_{i+hd/2}) <- (x_i c - x_{i+hd/2} s, x_{i+hd/2} c + x_i s)   (rope.zig:92-109)
 //   q -> q_out (or back in place when q_out is null)
-//   k, v -> page `slot / page_size`, row `slot % page_size` of the pools laid out
-//           [page, kv head, row, hd]   (or k back in place when slot_mapping is null)
+//   k -> page `slot / page_size`, row `slot % page_size` of the key pool laid out
+//        [page, kv head, row, hd]   (or back in place when slot_mapping is null)
+//   v -> the value pool, laid out [page, kv head, hd, row]: the rows (positions) of a page
+//        are contiguous for each element of the head, which is the operand order the
+//        attention kernels' second matrix product wants
 template <typename T>
 __global__ void qk_norm_rope_kv_write_kernel(
     T* __restrict__ qkv, const float* __restrict__ q_gain, const float* __restrict__ k_gain,
@@ -83,8 +86,8 @@ __global__ void qk_norm_rope_kv_write_kernel(
     const int kvh = head - nH - nKV;
     const int slot = slot_mapping[t];
     const int page = slot / page_size, r = slot % page_size;
-    T* dst = v_pool + (((size_t)page * nKV + kvh) * page_size + r) * hd;
-    for (int i = lane; i < hd; i += ZF_WAVE) dst[i] = src[i];
+    T* dst = v_pool + ((size_t)page * nKV + kvh) * page_size * hd + r;
+    for (int i = lane; i < hd; i += ZF_WAVE) dst[(size_t)i * page_size] = src[i];
     return;
   }
   const bool is_q = head < nH;

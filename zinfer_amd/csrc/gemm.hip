@@ -98,3 +98,363 @@ extern "C" int zf_gemm_fma(const void* A, int a_dtype, const void* W, int w_dtyp
   }
   ZF_CHECK_LAUNCH();
 }
+
+// =====================================================================================
+//  bfloat16 MFMA kernels (gfx950): v_mfma_f32_32x32x16_bf16 and v_mfma_f32_16x16x32_bf16,
+//  fp32 accumulation.  A is [M, K] bfloat16, W is [N, K] bfloat16, both with K contiguous,
+//  which is the operand order the instruction wants: every lane feeds 8 consecutive k of
+//  one row of A and of one row of W.
+// =====================================================================================
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+
+#define EPI_STORE_BF16 0
+#define EPI_STORE_F32 1
+#define EPI_ACC_F32 2
+
+// ---------------------------------------------------------------- large M: LDS-tiled
+// Block tile BM x BN x 64, waves laid out (BM/WM) x (BN/WN), each wave WM x WN through
+// 32x32x16 MFMAs.  Tiles are staged through LDS with rows padded to 72 elements (144 bytes)
+// so that the 16-byte operand reads of 8 neighbouring rows fall on distinct banks; the next
+// tile's global loads are in flight while the current one is multiplied.
+#define TK 64
+#define LDS_ROW 72
+
+template <int BM, int BN, int WM, int WN, int EPI>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
+    int N, int K, int tiles_m, int tiles_n) {
+  constexpr int NWM = BM / WM, NWN = BN / WN;
+  constexpr int NT = NWM * NWN * 64;
+  constexpr int FM = WM / 32, FN = WN / 32;
+  constexpr int A_CHUNKS = BM * 8 / NT;   // 16-byte chunks per thread per tile
+  constexpr int B_CHUNKS = BN * 8 / NT;
+  static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0, "tile does not divide over the threads");
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  bf16_t* lds = (bf16_t*)lds_raw;
+  // stage s: A at s*(BM+BN)*LDS_ROW, W after it
+  constexpr int STAGE = (BM + BN) * LDS_ROW;
+
+  // XCD-aware tile order: consecutive workgroups go to different XCDs (8 of them, each with
+  // its own L2), so workgroup b works on tile (b % 8) * per_xcd + b / 8: one XCD then walks
+  // neighbouring tiles, grouped 8 tiles of M deep so that they share W tiles in its L2.
+  const int nblocks = tiles_m * tiles_n;
+  int b = blockIdx.x;
+  {
+    const int base = nblocks / 8, rem = nblocks % 8;
+    const int xcd = b % 8, idx = b / 8;
+    b = xcd * base + min(xcd, rem) + idx;   // XCD x owns base (+1 if x < rem) tiles in a row
+  }
+  const int GROUP = 8;
+  const int in_group = GROUP * tiles_n;
+  const int g = b / in_group;
+  const int first_m = g * GROUP;
+  const int gsize = min(tiles_m - first_m, GROUP);
+  const int tm = first_m + (b % in_group) % gsize;
+  const int tn = (b % in_group) / gsize;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const int tid = threadIdx.x;
+  const int wave = tid / 64, lane = tid % 64;
+  const int wm = wave / NWN, wn = wave % NWN;
+
+  f32x16_t acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  u32x4_t areg[A_CHUNKS], breg[B_CHUNKS];
+
+  auto gload = [&](int k0) {
+#pragma unroll
+    for (int c = 0; c < A_CHUNKS; ++c) {
+      const int chunk = tid + c * NT;
+      const int row = chunk / 8, kc = (chunk % 8) * 8;
+      const int m = min(m0 + row, M - 1);
+      if (k0 + kc < K)
+        areg[c] = *(const u32x4_t*)(A + (size_t)m * K + k0 + kc);
+      else
+        areg[c] = u32x4_t{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int c = 0; c < B_CHUNKS; ++c) {
+      const int chunk = tid + c * NT;
+      const int row = chunk / 8, kc = (chunk % 8) * 8;
+      const int n = min(n0 + row, N - 1);
+      if (k0 + kc < K)
+        breg[c] = *(const u32x4_t*)(W + (size_t)n * K + k0 + kc);
+      else
+        breg[c] = u32x4_t{0, 0, 0, 0};
+    }
+  };
+  auto lstore = [&](int stage) {
+    bf16_t* a_s = lds + stage * STAGE;
+    bf16_t* b_s = a_s + BM * LDS_ROW;
+#pragma unroll
+    for (int c = 0; c < A_CHUNKS; ++c) {
+      const int chunk = tid + c * NT;
+      const int row = chunk / 8, kc = (chunk % 8) * 8;
+      *(u32x4_t*)(a_s + row * LDS_ROW + kc) = areg[c];
+    }
+#pragma unroll
+    for (int c = 0; c < B_CHUNKS; ++c) {
+      const int chunk = tid + c * NT;
+      const int row = chunk / 8, kc = (chunk % 8) * 8;
+      *(u32x4_t*)(b_s + row * LDS_ROW + kc) = breg[c];
+    }
+  };
+
+  const int ktiles = (K + TK - 1) / TK;
+  gload(0);
+  lstore(0);
+  __syncthreads();
+  for (int kt = 0; kt < ktiles; ++kt) {
+    const int stage = kt & 1;
+    if (kt + 1 < ktiles) gload((kt + 1) * TK);
+    const bf16_t* a_s = lds + stage * STAGE + (wm * WM) * LDS_ROW;
+    const bf16_t* b_s = lds + stage * STAGE + BM * LDS_ROW + (wn * WN) * LDS_ROW;
+#pragma unroll
+    for (int ks = 0; ks < TK / 16; ++ks) {
+      bf16x8_t af[FM], bfr[FN];
+      const int koff = ks * 16 + (lane / 32) * 8;
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+        af[i] = *(const bf16x8_t*)(a_s + (i * 32 + lane % 32) * LDS_ROW + koff);
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+        bfr[j] = *(const bf16x8_t*)(b_s + (j * 32 + lane % 32) * LDS_ROW + koff);
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < ktiles) lstore(stage ^ 1);
+    __syncthreads();
+  }
+
+  // D[i][j] of a 32x32 block: j = lane % 32, i = 8 * (r / 4) + 4 * (lane / 32) + r % 4
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+      const int n = n0 + wn * WN + j * 32 + lane % 32;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
+        if (m < M && n < N) {
+          const size_t off = (size_t)m * N + n;
+          if (EPI == EPI_STORE_BF16)
+            ((bf16_t*)Cv)[off] = float_to_bf16(acc[i][j][r]);
+          else if (EPI == EPI_STORE_F32)
+            ((float*)Cv)[off] = acc[i][j][r];
+          else
+            ((float*)Cv)[off] += acc[i][j][r];
+        }
+      }
+    }
+}
+
+template <int BM, int BN, int WM, int WN>
+static int launch_tile(const void* A, const void* W, void* C, int M, int N, int K, int epi,
+                       hipStream_t stream) {
+  constexpr int NT = (BM / WM) * (BN / WN) * 64;
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  const int nblocks = tiles_m * tiles_n;
+  const size_t smem = (size_t)2 * (BM + BN) * LDS_ROW * sizeof(bf16_t);
+#define ZF_TILE_LAUNCH(E)                                                                      \
+  do {                                                                                         \
+    auto kern = gemm_bf16_tile_kernel<BM, BN, WM, WN, E>;                                      \
+    if (smem > 64 * 1024) {                                                                    \
+      hipError_t e = hipFuncSetAttribute((const void*)kern,                                    \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
+      if (e != hipSuccess) return (int)e;                                                      \
+    }                                                                                          \
+    hipLaunchKernelGGL(kern, dim3(nblocks), dim3(NT), smem, stream, (const bf16_t*)A,          \
+                       (const bf16_t*)W, C, M, N, K, tiles_m, tiles_n);                        \
+  } while (0)
+  if (epi == EPI_STORE_BF16) ZF_TILE_LAUNCH(EPI_STORE_BF16);
+  else if (epi == EPI_STORE_F32) ZF_TILE_LAUNCH(EPI_STORE_F32);
+  else ZF_TILE_LAUNCH(EPI_ACC_F32);
+#undef ZF_TILE_LAUNCH
+  return (int)hipGetLastError();
+}
+
+// variant: 0 = 128x128 (waves 64x64), 1 = 256x128 (waves 128x64), 2 = 256x256 (waves 128x128),
+//          3 = 128x128 (waves 64x32, 8 waves), 4 = 256x256 (waves 128x64, 8 waves)
+extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, int N, int K,
+                                 int epi, int variant, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K % 8 != 0) return -3;
+  switch (variant) {
+    case 0: return launch_tile<128, 128, 64, 64>(A, W, C, M, N, K, epi, stream);
+    case 1: return launch_tile<256, 128, 128, 64>(A, W, C, M, N, K, epi, stream);
+    case 2: return launch_tile<256, 256, 128, 128>(A, W, C, M, N, K, epi, stream);
+    case 3: return launch_tile<128, 128, 64, 32>(A, W, C, M, N, K, epi, stream);
+    case 4: return launch_tile<256, 256, 128, 64>(A, W, C, M, N, K, epi, stream);
+    default: return -4;
+  }
+}
+
+// ---------------------------------------------------------------- small M: weight streaming
+// For M <= 64 the product is bound by reading W once from HBM.  A workgroup owns 16 * RG rows
+// of W (output features) and all M tokens; its 8 waves (times KSPLIT workgroups along
+// gridDim.y) split K between them in steps of 64: each lane loads 2 x 16 bytes of one row, 4
+// lanes cover a 128-byte line.  W is the first MFMA operand, the tokens (read through L2,
+// they are small, and reused for the RG row groups) the second (v_mfma_f32_16x16x32_bf16).
+// The waves' partial sums are added through LDS in wave order; with KSPLIT > 1 the
+// workgroups write float32 partials to a workspace [KSPLIT, M, N] that
+// skinny_reduce_kernel adds in split order.  Nothing depends on timing.  No LDS staging of W:
+// nothing of it is reused.
+template <int MT, int RG, int EPI>
+__global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
+    int N, int K) {
+  __shared__ float part[8][RG * MT][64][4];
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int n0 = blockIdx.x * (16 * RG);
+  const int g = lane / 16;
+  const bf16_t* wrow[RG];
+#pragma unroll
+  for (int r = 0; r < RG; ++r) wrow[r] = W + (size_t)min(n0 + r * 16 + lane % 16, N - 1) * K;
+  const bf16_t* arow[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) arow[t] = A + (size_t)min(t * 16 + lane % 16, M - 1) * K;
+
+  f32x4_t acc[RG][MT];
+#pragma unroll
+  for (int r = 0; r < RG; ++r)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[r][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  const u32x4_t zero = u32x4_t{0, 0, 0, 0};
+  const int kstride = 512 * gridDim.y;
+#pragma unroll 2
+  for (int k0 = (blockIdx.y * 8 + wave) * 64; k0 < K; k0 += kstride) {
+    const int k = k0 + g * 16;
+    u32x4_t w0[RG], w1[RG];
+#pragma unroll
+    for (int r = 0; r < RG; ++r) {
+      w0[r] = (k < K) ? __builtin_nontemporal_load((const u32x4_t*)(wrow[r] + k)) : zero;
+      w1[r] = (k + 8 < K) ? __builtin_nontemporal_load((const u32x4_t*)(wrow[r] + k + 8)) : zero;
+    }
+    u32x4_t a0[MT], a1[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      a0[t] = (k < K) ? *(const u32x4_t*)(arow[t] + k) : zero;
+      a1[t] = (k + 8 < K) ? *(const u32x4_t*)(arow[t] + k + 8) : zero;
+    }
+#pragma unroll
+    for (int r = 0; r < RG; ++r)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            *(bf16x8_t*)&w0[r], *(bf16x8_t*)&a0[t], acc[r][t], 0, 0, 0);
+        acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            *(bf16x8_t*)&w1[r], *(bf16x8_t*)&a1[t], acc[r][t], 0, 0, 0);
+      }
+  }
+#pragma unroll
+  for (int r = 0; r < RG; ++r)
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) part[wave][r * MT + t][lane][e] = acc[r][t][e];
+  __syncthreads();
+  for (int item = tid; item < RG * MT * 64; item += 512) {
+    const int rt = item / 64, l = item % 64;
+    const int r = rt / MT, t = rt % MT;
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 8; ++w)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[e] += part[w][rt][l][e];
+    // D[i][j]: i = 4 * (l / 16) + e is the W row (output feature), j = l % 16 the token
+    const int token = t * 16 + l % 16;
+    if (token < M) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int n = n0 + r * 16 + 4 * (l / 16) + e;
+        if (n < N) {
+          if (gridDim.y > 1) {
+            ((float*)Cv)[((size_t)blockIdx.y * M + token) * N + n] = s[e];   // workspace
+          } else {
+            const size_t off = (size_t)token * N + n;
+            if (EPI == EPI_STORE_BF16)
+              ((bf16_t*)Cv)[off] = float_to_bf16(s[e]);
+            else if (EPI == EPI_STORE_F32)
+              ((float*)Cv)[off] = s[e];
+            else
+              ((float*)Cv)[off] += s[e];
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int EPI>
+__global__ void skinny_reduce_kernel(const float* __restrict__ ws, void* __restrict__ Cv,
+                                     size_t mn, int ksplit) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= mn) return;
+  float s = 0.f;
+  for (int k = 0; k < ksplit; ++k) s += ws[(size_t)k * mn + i];
+  if (EPI == EPI_STORE_BF16)
+    ((bf16_t*)Cv)[i] = float_to_bf16(s);
+  else if (EPI == EPI_STORE_F32)
+    ((float*)Cv)[i] = s;
+  else
+    ((float*)Cv)[i] += s;
+}
+
+template <int MT, int RG>
+static int launch_skinny(const void* A, const void* W, void* C, void* ws, int M, int N, int K,
+                         int epi, int ksplit, hipStream_t stream) {
+  const dim3 grid((N + 16 * RG - 1) / (16 * RG), ksplit), block(512);
+  void* dst = ksplit > 1 ? ws : C;
+  if (epi == EPI_STORE_BF16)
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_STORE_BF16>), grid, block, 0, stream,
+                       (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K);
+  else if (epi == EPI_STORE_F32)
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_STORE_F32>), grid, block, 0, stream,
+                       (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K);
+  else
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_ACC_F32>), grid, block, 0, stream,
+                       (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K);
+  if (ksplit > 1) {
+    const size_t mn = (size_t)M * N;
+    const unsigned blocks = (unsigned)((mn + 255) / 256);
+    if (epi == EPI_STORE_BF16)
+      hipLaunchKernelGGL(skinny_reduce_kernel<EPI_STORE_BF16>, dim3(blocks), dim3(256), 0, stream,
+                         (const float*)ws, C, mn, ksplit);
+    else if (epi == EPI_STORE_F32)
+      hipLaunchKernelGGL(skinny_reduce_kernel<EPI_STORE_F32>, dim3(blocks), dim3(256), 0, stream,
+                         (const float*)ws, C, mn, ksplit);
+    else
+      hipLaunchKernelGGL(skinny_reduce_kernel<EPI_ACC_F32>, dim3(blocks), dim3(256), 0, stream,
+                         (const float*)ws, C, mn, ksplit);
+  }
+  return (int)hipGetLastError();
+}
+
+// rg: row groups of 16 per workgroup (1, 2 or 4); ksplit: workgroups along K (1..16), which
+// needs a float32 workspace of ksplit * M * N elements when > 1.
+extern "C" int zf_gemm_bf16_skinny(const void* A, const void* W, void* C, void* ws, int M, int N,
+                                   int K, int epi, int rg, int ksplit, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K % 8 != 0 || M > 64 || ksplit < 1 || ksplit > 16 || (ksplit > 1 && ws == nullptr))
+    return -3;
+  const int mt = (M + 15) / 16;
+#define ZF_SK(MT, RG) return launch_skinny<MT, RG>(A, W, C, ws, M, N, K, epi, ksplit, stream)
+  if (rg == 1) { if (mt == 1) ZF_SK(1, 1); if (mt == 2) ZF_SK(2, 1); if (mt == 3) ZF_SK(3, 1); ZF_SK(4, 1); }
+  if (rg == 2) { if (mt == 1) ZF_SK(1, 2); if (mt == 2) ZF_SK(2, 2); if (mt == 3) ZF_SK(3, 2); ZF_SK(4, 2); }
+  if (rg == 4) { if (mt == 1) ZF_SK(1, 4); if (mt == 2) ZF_SK(2, 4); if (mt == 3) ZF_SK(3, 4); ZF_SK(4, 4); }
+#undef ZF_SK
+  return -4;
+}

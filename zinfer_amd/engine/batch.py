@@ -63,6 +63,7 @@ class StepContext:
     q_lens: List[int]             # host copies, for parts that loop on the host
     ctx_lens: List[int]
     slots: List[int]
+    n_single: int = 0             # sequences with exactly one token in this step
     _scratch: Scratch = None
 
     def scratch(self, name: str, shape, dtype) -> torch.Tensor:

@@ -183,6 +183,7 @@ class Engine:
             ctx_len=view("ctx_len"), state_slots=view("state_slots"),
             want_rows=view("want_rows")[:n_want], kv=kv, max_q_len=max(q_lens),
             max_ctx_len=max(ctx_lens), q_lens=q_lens, ctx_lens=ctx_lens, slots=slots,
+            n_single=sum(1 for n in q_lens if n == 1),
             _scratch=self._scratch)
 
     def _upload(self, host: np.ndarray) -> torch.Tensor:

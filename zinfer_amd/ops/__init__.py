@@ -144,9 +144,52 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     _check(lib.zf_argmax(_ptr(logits), _ptr(out), n, V, _stream()), "argmax")
 
 
+# ------------------------------------------------------------------------- work buffers
+_workspaces = {}
+
+
+def _workspace(name: str, numel: int, dtype: torch.dtype, device) -> torch.Tensor:
+    """A persistent device buffer of at least ``numel`` elements (grown when needed, never
+    inside a stream capture once sizes have settled)."""
+    key = (name, str(device), dtype)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < numel:
+        buf = torch.empty((max(numel, 1),), dtype=dtype, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
 # ------------------------------------------------------------------------- matrix product
+_EPI_STORE_BF16, _EPI_STORE_F32, _EPI_ACC_F32 = 0, 1, 2
+SKINNY_MAX_M = 64
+
+
+def _skinny_plan(M: int, N: int):
+    """Row groups of 16 per workgroup and workgroups along K for the weight-streaming kernel:
+    enough workgroups to fill 256 CUs, as many rows per workgroup as that allows (the tokens
+    are re-read once per workgroup)."""
+    if M <= 16:
+        rg = 4 if N // 64 >= 256 else 1
+        ks = 2 if (rg == 4 and N // 64 < 1024) else 1
+    else:
+        rg, ks = 4, 1
+        while (N // 64) * ks < 192 and ks < 16:
+            ks *= 2
+    return rg, ks
+
+
+def _tile_variant(M: int, N: int) -> int:
+    """256 x 256 tiles when they still fill the chip, else 128 x 128."""
+    tiles = ((M + 255) // 256) * ((N + 255) // 256)
+    return 4 if tiles >= 160 else 0
+
+
 def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
-    """out = a w^T (w is [N, K]); with ``accumulate`` out += a w^T, in 32-bit."""
+    """out = a w^T (w is [N, K]); with ``accumulate`` out += a w^T, in 32-bit.
+
+    bfloat16 operands with K a multiple of 8 go to the MFMA kernels (weight streaming for up
+    to 64 rows of ``a``, LDS-tiled above); everything else, the whole 32-bit path included,
+    goes to the FMA kernel, whose results do not depend on how rows are batched."""
     _need_gpu(a, w, out)
     M, K = a.shape
     N = w.shape[0]
@@ -156,17 +199,42 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     if accumulate and out.dtype != torch.float32:
         raise KernelUnavailable("gemm: accumulation needs a float32 output")
     lib = build.load("gemm")
+    if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and K % 8 == 0 and M > 0:
+        epi = _EPI_ACC_F32 if accumulate else \
+            (_EPI_STORE_BF16 if out.dtype == torch.bfloat16 else _EPI_STORE_F32)
+        if M <= SKINNY_MAX_M:
+            rg, ks = _skinny_plan(M, N)
+            ws = _workspace("gemm_splitk", ks * M * N, torch.float32, a.device) if ks > 1 else None
+            _check(lib.zf_gemm_bf16_skinny(_ptr(a), _ptr(w), _ptr(out), _ptr(ws), M, N, K, epi,
+                                           rg, ks, _stream()), "gemm (weight streaming)")
+        else:
+            _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, epi,
+                                         _tile_variant(M, N), _stream()), "gemm (tiled)")
+        return
     _check(lib.zf_gemm_fma(_ptr(a), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), M, N, K,
                            1 if accumulate else 0, _stream()), "gemm")
 
 
 # ------------------------------------------------------------------------- attention
+DECODE_SPLIT_KEYS = 256
+
+
+def mfma_attention_covers(dtype, n_heads, n_kv_heads, head_dim, page_size) -> bool:
+    return dtype == torch.bfloat16 and head_dim in (32, 64, 128, 256) and page_size % 16 == 0 \
+        and n_heads // n_kv_heads <= 16
+
+
 def paged_attention(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index, out, scale,
                     window, n_heads, n_kv_heads, head_dim, page_size, max_q_len,
-                    max_ctx_len) -> None:
+                    max_ctx_len, n_single=None) -> None:
     """Causal grouped-query attention of the step's tokens over the paged cache.  Token t of
     sequence s = seq_index[t] has position ctx_len[s] - q_len[s] + (t - q_start[s]) and reads
-    the positions up to its own (the last ``window`` of them if window > 0)."""
+    the positions up to its own (the last ``window`` of them if window > 0).  ``n_single`` is
+    the number of sequences with exactly one token in this step (None: unknown).
+
+    bfloat16 with head_dim 32/64/128/256 and a page size that is a multiple of 16 runs the
+    MFMA kernels: split-context decode for single tokens, the tiled kernel for portions.
+    Everything else runs the 32-bit wave kernel."""
     _need_gpu(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index, out)
     T = q.shape[0]
     if q.shape != (T, n_heads * head_dim) or out.shape != q.shape or out.dtype != q.dtype \
@@ -181,9 +249,34 @@ def paged_attention(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index,
         raise KernelUnavailable(f"paged_attention: head_dim {head_dim} > 512 is not covered")
     if max_ctx_len > block_table.shape[1] * page_size:
         raise KernelUnavailable("paged_attention: block table shorter than the context")
+    n_seqs = ctx_len.shape[0]
+    if q_start.shape[0] != n_seqs + 1 or block_table.shape[0] != n_seqs or seq_index.shape[0] != T:
+        raise KernelUnavailable("paged_attention: per-sequence arrays disagree in length")
     lib = build.load("attention")
+    max_pages = block_table.shape[1]
+    if mfma_attention_covers(q.dtype, n_heads, n_kv_heads, head_dim, page_size):
+        if n_single is None:
+            n_single = n_seqs if max_q_len == 1 else -1      # -1: some, not known how many
+        if n_single != 0:
+            max_splits = (max_ctx_len + DECODE_SPLIT_KEYS - 1) // DECODE_SPLIT_KEYS
+            ws_o = _workspace("attn_o", n_seqs * n_heads * max_splits * head_dim, torch.float32,
+                              q.device)
+            ws_ml = _workspace("attn_ml", n_seqs * n_heads * max_splits * 2, torch.float32,
+                               q.device)
+            _check(lib.zf_attn_decode_bf16(
+                _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), _ptr(q_start),
+                _ptr(ctx_len), _ptr(out), _ptr(ws_o), _ptr(ws_ml), ctypes.c_float(scale),
+                int(window), n_seqs, n_heads, n_kv_heads, head_dim, page_size, max_pages,
+                max_splits, DECODE_SPLIT_KEYS, _stream()), "paged_attention (decode)")
+        if n_single != n_seqs and max_q_len > 1:
+            _check(lib.zf_attn_prefill_bf16(
+                _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), _ptr(q_start),
+                _ptr(ctx_len), _ptr(out), ctypes.c_float(scale), int(window), n_seqs,
+                max_q_len, n_heads, n_kv_heads, head_dim, page_size, max_pages,
+                1 if n_single != 0 else 0, _stream()), "paged_attention (prefill)")
+        return
     _check(lib.zf_paged_attention_wave(
         _ptr(q), _ptr(k_pool), _ptr(v_pool), _dt(q), _ptr(block_table), _ptr(q_start),
         _ptr(ctx_len), _ptr(seq_index), _ptr(out), ctypes.c_float(scale), int(window), T,
-        n_heads, n_kv_heads, head_dim, page_size, block_table.shape[1], _stream()),
+        n_heads, n_kv_heads, head_dim, page_size, max_pages, _stream()),
         "paged_attention")
