@@ -181,3 +181,38 @@ def test_step_errors_leave_cache_untouched(tmp_path_factory):
         eng.step([StepEntry("x", [1] * 5, [])])
     assert eng.length("x") == 60
     eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_equal_eager_steps(dtype, tmp_path_factory):
+    """Decode-only steps run through a captured graph.  Every replay is compared with an
+    engine that launches the same kernels one by one; other work (a prompt portion of
+    another request, a request ending, host synchronisation) happens between the replays."""
+    from zinfer_amd.engine import StepEntry
+    from zinfer_amd.engine.replay import make_engine
+    name = "D"
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    path = tiny.model_dir_of(name, str(tmp_path_factory.getbasetemp()), store)
+    V = tiny.CONFIGS[name]["vocab_size"]
+    a = make_engine(path, dtype, 1024, DEV)
+    b = make_engine(path, dtype, 1024, DEV)
+    b.use_graphs = False
+    reqs = {f"g{i}": tiny.random_tokens(n, V, 500 + i) for i, n in enumerate((70, 33, 120))}
+    extra = tiny.random_tokens(90, V, 600)
+    for eng in (a, b):
+        eng.step([StepEntry(r, t[:20], []) for r, t in reqs.items()])
+    for k in range(20, 33):
+        entries = [StepEntry(r, t[k:k + 1], [0]) for r, t in reqs.items()]
+        la, lb = a.step(entries), b.step(entries)
+        assert torch.equal(la, lb), f"decode step {k}: replay differs from eager launches"
+        torch.cuda.synchronize()
+        if k % 4 == 0:          # eager work between the replays
+            lo = (k - 20) * 5
+            pa = a.step([StepEntry("extra", extra[lo:lo + 20], [19])])
+            pb = b.step([StepEntry("extra", extra[lo:lo + 20], [19])])
+            assert torch.equal(pa, pb)
+        if k == 27:             # one request ends: the batch shape changes, another graph
+            for eng in (a, b):
+                eng.release("g1")
+            reqs.pop("g1")
+    assert a.graph_replays >= 10 and b.graph_replays == 0

@@ -44,15 +44,60 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restr
     store_from_float<TO>(o + i, row[i] * inv * gain[i]);
 }
 
+// Widths that are a multiple of 4 up to 8192: every thread keeps its part of the row in
+// registers (at most 8 float4), so the row is read once and all loads are issued together.
+template <typename TO>
+__global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const float* __restrict__ x,
+                                                          const float* __restrict__ gain,
+                                                          TO* __restrict__ out, int W, float eps) {
+  __shared__ float red[16];
+  const float4* row = (const float4*)(x + (size_t)blockIdx.x * W);
+  const float4* g4 = (const float4*)gain;
+  TO* o = out + (size_t)blockIdx.x * W;
+  const int n4 = W / 4;
+  float4 v[8];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = threadIdx.x + i * 256;
+    v[i] = c < n4 ? row[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)W + eps);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = threadIdx.x + i * 256;
+    if (c < n4) {
+      const float4 g = g4[c];
+      store_from_float<TO>(o + 4 * c + 0, v[i].x * inv * g.x);
+      store_from_float<TO>(o + 4 * c + 1, v[i].y * inv * g.y);
+      store_from_float<TO>(o + 4 * c + 2, v[i].z * inv * g.z);
+      store_from_float<TO>(o + 4 * c + 3, v[i].w * inv * g.w);
+    }
+  }
+}
+
 extern "C" int zf_rmsnorm(const float* x, const float* gain, void* out, int out_dtype, int T,
                           int W, float eps, hipStream_t stream) {
   if (T <= 0) return 0;
-  if (out_dtype == ZF_F32)
-    hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(T), dim3(256), 0, stream, x, gain,
-                       (float*)out, W, eps);
-  else
-    hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(T), dim3(256), 0, stream, x, gain,
-                       (bf16_t*)out, W, eps);
+  const bool vec = (W % 4 == 0) && W <= 8192;
+  if (out_dtype == ZF_F32) {
+    if (vec)
+      hipLaunchKernelGGL(rmsnorm_vec_kernel<float>, dim3(T), dim3(256), 0, stream, x, gain,
+                         (float*)out, W, eps);
+    else
+      hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(T), dim3(256), 0, stream, x, gain,
+                         (float*)out, W, eps);
+  } else {
+    if (vec)
+      hipLaunchKernelGGL(rmsnorm_vec_kernel<bf16_t>, dim3(T), dim3(256), 0, stream, x, gain,
+                         (bf16_t*)out, W, eps);
+    else
+      hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(T), dim3(256), 0, stream, x, gain,
+                         (bf16_t*)out, W, eps);
+  }
   ZF_CHECK_LAUNCH();
 }
 
@@ -194,20 +239,12 @@ extern "C" int zf_gather_rows(const float* x, const int* idx, float* out, int n,
 }
 
 // ---------------------------------------------------------------- arg-max, first maximum wins
-// (src/model/layers/logits.zig:47-59: strict > while walking upwards)
-__global__ void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V) {
-  __shared__ float sval[256];
-  __shared__ int sidx[256];
-  const float* row = logits + (size_t)blockIdx.x * V;
-  float best = -INFINITY;
-  int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) {
-    const float v = row[i];
-    if (v > best) {
-      best = v;
-      bi = i;
-    }
-  }
+// (src/model/layers/logits.zig:47-59: strict > while walking upwards).  Two stages: every
+// workgroup reduces a chunk of a row to (value, index); one workgroup per row reduces the
+// chunks.  Among equal values the lower index wins at every level.
+#define ARGMAX_CHUNK 4096
+
+__device__ __forceinline__ void argmax_block_reduce(float& best, int& bi, float* sval, int* sidx) {
   sval[threadIdx.x] = best;
   sidx[threadIdx.x] = bi;
   __syncthreads();
@@ -222,11 +259,63 @@ __global__ void argmax_kernel(const float* __restrict__ logits, int* __restrict_
     }
     __syncthreads();
   }
-  if (threadIdx.x == 0) out[blockIdx.x] = sidx[0] == 0x7fffffff ? 0 : sidx[0];
+  best = sval[0];
+  bi = sidx[0];
 }
 
-extern "C" int zf_argmax(const float* logits, int* out, int n, int V, hipStream_t stream) {
+__global__ __launch_bounds__(256) void argmax_chunk_kernel(const float* __restrict__ logits,
+                                                           float* __restrict__ pval,
+                                                           int* __restrict__ pidx, int V,
+                                                           int nchunks) {
+  __shared__ float sval[256];
+  __shared__ int sidx[256];
+  const float* row = logits + (size_t)blockIdx.x * V;
+  const int lo = blockIdx.y * ARGMAX_CHUNK, hi = min(V, lo + ARGMAX_CHUNK);
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = lo + threadIdx.x; i < hi; i += 256) {
+    const float v = row[i];
+    if (v > best) {
+      best = v;
+      bi = i;
+    }
+  }
+  argmax_block_reduce(best, bi, sval, sidx);
+  if (threadIdx.x == 0) {
+    pval[blockIdx.x * nchunks + blockIdx.y] = best;
+    pidx[blockIdx.x * nchunks + blockIdx.y] = bi;
+  }
+}
+
+__global__ __launch_bounds__(256) void argmax_final_kernel(const float* __restrict__ pval,
+                                                           const int* __restrict__ pidx,
+                                                           int* __restrict__ out, int nchunks) {
+  __shared__ float sval[256];
+  __shared__ int sidx[256];
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = threadIdx.x; i < nchunks; i += 256) {
+    const float v = pval[blockIdx.x * nchunks + i];
+    const int id = pidx[blockIdx.x * nchunks + i];
+    if (v > best || (v == best && id < bi)) {
+      best = v;
+      bi = id;
+    }
+  }
+  argmax_block_reduce(best, bi, sval, sidx);
+  if (threadIdx.x == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+}
+
+// ws: (float + int) * n * ceil(V / 4096) of scratch
+extern "C" int zf_argmax(const float* logits, int* out, void* ws, int n, int V,
+                         hipStream_t stream) {
   if (n <= 0) return 0;
-  hipLaunchKernelGGL(argmax_kernel, dim3(n), dim3(256), 0, stream, logits, out, V);
+  const int nchunks = (V + ARGMAX_CHUNK - 1) / ARGMAX_CHUNK;
+  float* pval = (float*)ws;
+  int* pidx = (int*)(pval + (size_t)n * nchunks);
+  hipLaunchKernelGGL(argmax_chunk_kernel, dim3(n, nchunks), dim3(256), 0, stream, logits, pval,
+                     pidx, V, nchunks);
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(n), dim3(256), 0, stream, pval, pidx, out,
+                     nchunks);
   ZF_CHECK_LAUNCH();
 }

@@ -31,6 +31,7 @@ class Scratch:
     def __init__(self, device):
         self.device = device
         self._bufs: Dict[str, torch.Tensor] = {}
+        self.generation = 0            # goes up whenever a buffer moves (captured graphs die)
 
     def get(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
         n = 1
@@ -41,6 +42,7 @@ class Scratch:
         if buf is None or buf.numel() < nbytes:
             buf = torch.empty(((nbytes + 255) // 256 * 256,), dtype=torch.uint8, device=self.device)
             self._bufs[name] = buf
+            self.generation += 1
         return buf[:n * torch.empty((), dtype=dtype).element_size()].view(dtype).view(*shape)
 
 
@@ -64,6 +66,7 @@ class StepContext:
     ctx_lens: List[int]
     slots: List[int]
     n_single: int = 0             # sequences with exactly one token in this step
+    meta_offset: int = 0          # address of the packed metadata (part of a graph's key)
     _scratch: Scratch = None
 
     def scratch(self, name: str, shape, dtype) -> torch.Tensor:

@@ -26,9 +26,12 @@ def _pad4(n: int) -> int:
 class Engine:
     """Owns a model, its cache and work buffers; ``step`` is the only way tokens run."""
 
+    GRAPH_PAGE_BUCKET = 64      # decode graphs are captured for block tables this many pages wide
+    MAX_GRAPHS = 16
+
     def __init__(self, model: DecoderModel, *, page_size: int = 16, num_pages: int = 256,
                  max_requests: int = 64, kv_dtype: Optional[torch.dtype] = None,
-                 poison_freed: bool = False):
+                 poison_freed: bool = False, use_graphs: bool = True):
         self.model = model
         self.device = model.ctx.device
         spec = model.spec
@@ -42,7 +45,13 @@ class Engine:
         self._scratch = Scratch(self.device)
         self._meta_host: Optional[torch.Tensor] = None
         self._meta_dev: Optional[torch.Tensor] = None
+        self._meta_generation = 0
         self.steps_run = 0
+        # decode-only steps (one token per request) are launch-bound: they are captured once
+        # per batch shape into a HIP graph and replayed
+        self.use_graphs = use_graphs and self.device.type == "cuda"
+        self._graphs: Dict[tuple, tuple] = {}
+        self.graph_replays = 0
 
     # ------------------------------------------------------------------ requests
     def has_request(self, rid) -> bool:
@@ -94,8 +103,10 @@ class Engine:
                 if not self.cache.has_request(rid):
                     self.cache.add_request(rid)
                 self.cache.reserve(rid, new_len)
-            ctx = self._build_context(entries)
-            logits = self.model.forward(ctx, self.views)
+            decode_only = self.use_graphs and all(len(e.tokens) == 1 for e in entries)
+            ctx = self._build_context(entries, bucket_pages=decode_only)
+            logits = self._forward_graphed(ctx) if decode_only \
+                else self.model.forward(ctx, self.views)
             for rid, new_len in wanted_len:
                 self.cache.commit(rid, new_len)
             self.steps_run += 1
@@ -103,6 +114,33 @@ class Engine:
             logits = torch.empty((0, spec.vocab_size), dtype=torch.float32, device=self.device)
         for rid in end:
             self.cache.release(rid)
+        return logits
+
+    def _generations(self) -> tuple:
+        from .. import ops
+        return (self._scratch.generation, ops.workspace_generation(), self._meta_generation)
+
+    def _forward_graphed(self, ctx: StepContext) -> torch.Tensor:
+        """A decode-only step through a captured graph.  The graph holds the addresses of the
+        metadata views, work buffers and pools: it is keyed by everything that fixes them
+        (sequences, wanted rows, width of the block tables) and dropped when a buffer moves."""
+        key = (ctx.n_seqs, ctx.n_want, tuple(t.max_pages for t in ctx.kv), ctx.meta_offset)
+        held = self._graphs.get(key)
+        if held is not None and held[2] == self._generations():
+            held[0].replay()
+            self.graph_replays += 1
+            return held[1]
+        # first time: an eager run settles the sizes of every work buffer (it writes the same
+        # keys and values the replay will write again), then capture and replay
+        logits = self.model.forward(ctx, self.views)
+        if len(self._graphs) >= self.MAX_GRAPHS:
+            self._graphs.clear()
+        torch.cuda.current_stream(self.device).synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.model.forward(ctx, self.views)
+        self._graphs[key] = (graph, logits, self._generations())
+        graph.replay()
         return logits
 
     def argmax(self, logits: torch.Tensor) -> List[int]:
@@ -116,7 +154,7 @@ class Engine:
         return out.tolist()
 
     # ------------------------------------------------------------------ metadata
-    def _build_context(self, entries: Sequence[StepEntry]) -> StepContext:
+    def _build_context(self, entries: Sequence[StepEntry], bucket_pages: bool = False) -> StepContext:
         ps = self.page_size
         n_seqs = len(entries)
         q_lens = [len(e.tokens) for e in entries]
@@ -132,6 +170,11 @@ class Engine:
         n_want = len(want_rows)
         n_groups = len(self.cache.groups)
         max_pages = max((c + ps - 1) // ps for c in ctx_lens)
+        max_ctx = max(ctx_lens)
+        if bucket_pages:      # a fixed table width (and context bound) per captured graph
+            b = self.GRAPH_PAGE_BUCKET
+            max_pages = (max_pages + b - 1) // b * b
+            max_ctx = max_pages * ps
 
         # one packed int32 buffer, one copy to the device
         sizes = [("token_ids", T), ("positions", T), ("seq_index", T), ("q_start", n_seqs + 1),
@@ -182,7 +225,8 @@ class Engine:
             positions=view("positions"), seq_index=view("seq_index"), q_start=view("q_start"),
             ctx_len=view("ctx_len"), state_slots=view("state_slots"),
             want_rows=view("want_rows")[:n_want], kv=kv, max_q_len=max(q_lens),
-            max_ctx_len=max(ctx_lens), q_lens=q_lens, ctx_lens=ctx_lens, slots=slots,
+            max_ctx_len=max_ctx, q_lens=q_lens, ctx_lens=ctx_lens, slots=slots,
+            meta_offset=self._meta_dev.data_ptr() if self._meta_dev is not None else 0,
             n_single=sum(1 for n in q_lens if n == 1),
             _scratch=self._scratch)
 
@@ -191,9 +235,10 @@ class Engine:
         if self.device.type == "cpu":
             return torch.from_numpy(host.copy())
         if self._meta_host is None or self._meta_host.numel() < n:
-            cap = max(n * 2, 4096)
+            cap = max(n * 2, 1 << 18)
             self._meta_host = torch.empty((cap,), dtype=torch.int32, pin_memory=True)
             self._meta_dev = torch.empty((cap,), dtype=torch.int32, device=self.device)
+            self._meta_generation += 1
         # the previous step's copy must have left the pinned buffer before it is rewritten
         torch.cuda.current_stream(self.device).synchronize()
         self._meta_host[:n].numpy()[:] = host

@@ -141,21 +141,31 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     if logits.dtype != torch.float32 or out.shape != (n,):
         raise KernelUnavailable("argmax: float32 [n, V] -> int32 [n]")
     lib = build.load("elementwise")
-    _check(lib.zf_argmax(_ptr(logits), _ptr(out), n, V, _stream()), "argmax")
+    ws = _workspace("argmax", 2 * n * ((V + 4095) // 4096), torch.float32, logits.device)
+    _check(lib.zf_argmax(_ptr(logits), _ptr(out), _ptr(ws), n, V, _stream()), "argmax")
 
 
 # ------------------------------------------------------------------------- work buffers
 _workspaces = {}
+_workspace_generation = 0
+
+
+def workspace_generation() -> int:
+    """Goes up whenever a work buffer is (re)allocated: a captured graph that used the old
+    buffer must not be replayed."""
+    return _workspace_generation
 
 
 def _workspace(name: str, numel: int, dtype: torch.dtype, device) -> torch.Tensor:
     """A persistent device buffer of at least ``numel`` elements (grown when needed, never
     inside a stream capture once sizes have settled)."""
+    global _workspace_generation
     key = (name, str(device), dtype)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < numel:
         buf = torch.empty((max(numel, 1),), dtype=dtype, device=device)
         _workspaces[key] = buf
+        _workspace_generation += 1
     return buf
 
 
