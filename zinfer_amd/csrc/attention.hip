@@ -142,29 +142,54 @@ __device__ __forceinline__ u32x2_t keep_range4(u32x2_t v, int n_lo, int n_hi) {
 }
 
 // ---------------------------------------------------------------- decode: one query token
-// Grid (sequence, kv head, split).  A split covers the keys [split * split_keys,
-// (split + 1) * split_keys) of the context, so which keys a split holds depends on the
-// context length only.  One wave per workgroup: the G query heads of the kv head are the
-// columns of 16x16x32 MFMAs (G <= 16).  Each split writes an un-normalised partial
-// (max, sum, O[G, hd]); attn_decode_merge_kernel combines the splits in split order.
+// Grid (sequence, kv head, split).  A split is the 64 keys [64 * split, 64 * split + 64) of
+// the context, so which keys a split holds depends on the context length only.  One wave
+// per workgroup takes its 64 keys in one go: all key loads are issued together, then all
+// value loads, the soft-max over the 64 scores needs no running rescale.  The G query heads
+// of the kv head are the columns of 16x16x32 MFMAs (G <= 16).  Each split writes an
+// un-normalised partial (max, sum, O[G, hd]); attn_decode_merge_kernel combines the splits
+// in split order.
+#define DEC_SPLIT 64
+
 template <int HD>
 __global__ __launch_bounds__(64) void attn_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int* __restrict__ block_table,
     const int* __restrict__ q_start, const int* __restrict__ ctx_len, float* __restrict__ ws_o,
     float* __restrict__ ws_ml, float scale_log2e, int window, int nH, int nKV, int ps,
-    int max_pages, int max_splits, int split_keys) {
+    int max_pages, int max_splits) {
   const int s = blockIdx.x, kvh = blockIdx.y, sp = blockIdx.z;
   if (q_start[s + 1] - q_start[s] != 1) return;
   const int ctx = ctx_len[s], pos = ctx - 1;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int k_begin = max(lo, sp * split_keys), k_end = min(ctx, (sp + 1) * split_keys);
+  const int kb = sp * DEC_SPLIT;
+  const int k_begin = max(lo, kb), k_end = min(ctx, kb + DEC_SPLIT);
   if (k_begin >= k_end) return;
   const int G = nH / nKV;
   const int lane = threadIdx.x, j = lane % 16, qd = lane / 16;
   const int t = q_start[s];
   const int* table = block_table + (size_t)s * max_pages;
 
+  // pages of the four 16-key groups; a group outside [k_begin, k_end) may have no page at
+  // all: it reads the page of a key that certainly exists and is masked
+  int page[4];
+  bool any[4];
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    const int base = kb + 16 * h;
+    any[h] = base < k_end && base + 16 > k_begin;
+    page[h] = table[(any[h] ? max(base, k_begin) : k_begin) / ps];
+  }
+  // keys: row i = lane % 16 of group h, head elements 32 step + 8 qd ..
+  u32x4_t kf[4][HD / 32];
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    const int key = min(max(kb + 16 * h + j, k_begin), k_end - 1);
+    const int kpage = any[h] ? page[h] : table[key / ps];
+    const bf16_t* krow = k_pool + (((size_t)kpage * nKV + kvh) * ps + key % ps) * HD + 8 * qd;
+#pragma unroll
+    for (int stp = 0; stp < HD / 32; ++stp) kf[h][stp] = *(const u32x4_t*)(krow + stp * 32);
+  }
   bf16x8_t qf[HD / 32];
   {
     const bf16_t* qrow = q + ((size_t)t * nH + kvh * G + min(j, G - 1)) * HD + 8 * qd;
@@ -175,83 +200,63 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
       qf[st] = *(bf16x8_t*)&v;
     }
   }
+  // values (transposed in the pool): row d = 16 dt + j, keys kb + 16 h + 4 qd .. + 3
+  u32x2_t vf[4][HD / 16];
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    const int off = (kb + 16 * h) % ps + 4 * qd;
+    const bf16_t* vb = v_pool + ((size_t)page[h] * nKV + kvh) * ps * HD + (size_t)j * ps + off;
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt) vf[h][dt] = *(const u32x2_t*)(vb + (size_t)dt * 16 * ps);
+  }
+  f32x4_t st[4];
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    st[h] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int stp = 0; stp < HD / 32; ++stp)
+      st[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&kf[h][stp], qf[stp],
+                                                      st[h], 0, 0, 0);
+  }
+  // st[h][r]: key kb + 16 h + 4 qd + r, query column j
+  float sc[16];
+  float m = -INFINITY;
+#pragma unroll
+  for (int h = 0; h < 4; ++h)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int key = kb + 16 * h + 4 * qd + r;
+      const float v = (key >= k_begin && key < k_end) ? st[h][r] * scale_log2e : -INFINITY;
+      sc[h * 4 + r] = v;
+      m = fmaxf(m, v);
+    }
+  m = fmaxf(m, __shfl_xor(m, 16, 64));
+  m = fmaxf(m, __shfl_xor(m, 32, 64));
+  float l = 0.f;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    sc[e] = exp2f(sc[e] - m);
+    l += sc[e];
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
   f32x4_t o[HD / 16];
 #pragma unroll
   for (int dt = 0; dt < HD / 16; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
-
-  for (int kb = (k_begin / 32) * 32; kb < k_end; kb += 32) {
-    f32x4_t st[2];
-    int page[2];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      // the 16 keys kb + 16 h .. + 15 lie in one page; a half outside [k_begin, k_end) may have
-      // no page at all: read the page of a key that certainly exists and mask everything
-      const int base = kb + 16 * h;
-      const bool any = base < k_end && base + 16 > k_begin;
-      const int safe = any ? max(base, k_begin) : k_begin;
-      page[h] = table[safe / ps];
-      const int key = min(max(base + j, k_begin), k_end - 1);
-      const int kpage = any ? page[h] : table[key / ps];
-      const bf16_t* krow = k_pool + (((size_t)kpage * nKV + kvh) * ps + key % ps) * HD + 8 * qd;
-      st[h] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int stp = 0; stp < HD / 32; ++stp) {
-        const u32x4_t kv = *(const u32x4_t*)(krow + stp * 32);
-        st[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&kv, qf[stp], st[h], 0,
-                                                        0, 0);
-      }
-    }
-    // st[h][r]: key kb + 16 h + 4 qd + r, query column j
-    float sc[8];
-    float tmax = -INFINITY;
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int key = kb + 16 * h + 4 * qd + r;
-        const float v = (key >= k_begin && key < k_end) ? st[h][r] * scale_log2e : -INFINITY;
-        sc[h * 4 + r] = v;
-        tmax = fmaxf(tmax, v);
-      }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float m_new = fmaxf(m, tmax);
-    const float corr = exp2f(m - m_new);
-    float psum = 0.f;
-    float p[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      p[e] = exp2f(sc[e] - m_new);
-      psum += p[e];
-    }
-    psum += __shfl_xor(psum, 16, 64);
-    psum += __shfl_xor(psum, 32, 64);
-    l = l * corr + psum;
-    m = m_new;
-    u32x4_t pk = u32x4_t{pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]),
-                         pack_bf16(p[6], p[7])};
+  for (int hh = 0; hh < 2; ++hh) {     // two MFMAs of 32 keys: groups 2 hh and 2 hh + 1
+    u32x4_t pk = u32x4_t{pack_bf16(sc[8 * hh + 0], sc[8 * hh + 1]),
+                         pack_bf16(sc[8 * hh + 2], sc[8 * hh + 3]),
+                         pack_bf16(sc[8 * hh + 4], sc[8 * hh + 5]),
+                         pack_bf16(sc[8 * hh + 6], sc[8 * hh + 7])};
     const bf16x8_t pf = *(bf16x8_t*)&pk;
-    // V^T operand: row d = 16 dt + j, keys kb + 16 h + 4 qd .. + 3 for h = 0, 1
-    const bf16_t* vb[2];
-    int n_lo[2], n_hi[2];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int base = kb + 16 * h + 4 * qd;
-      n_lo[h] = k_begin - base;
-      n_hi[h] = k_end - base;
-      const int off = (kb + 16 * h) % ps + 4 * qd;
-      vb[h] = v_pool + ((size_t)page[h] * nKV + kvh) * ps * HD + (size_t)j * ps + off;
-    }
+    const int b0 = kb + 32 * hh + 4 * qd, b1 = b0 + 16;
 #pragma unroll
     for (int dt = 0; dt < HD / 16; ++dt) {
-      u32x2_t v0 = *(const u32x2_t*)(vb[0] + (size_t)dt * 16 * ps);
-      u32x2_t v1 = *(const u32x2_t*)(vb[1] + (size_t)dt * 16 * ps);
-      v0 = keep_range4(v0, n_lo[0], n_hi[0]);
-      v1 = keep_range4(v1, n_lo[1], n_hi[1]);
+      // stale or poisoned rows outside [k_begin, k_end) are zeroed: 0 * NaN would spoil the sum
+      const u32x2_t v0 = keep_range4(vf[2 * hh][dt], k_begin - b0, k_end - b0);
+      const u32x2_t v1 = keep_range4(vf[2 * hh + 1][dt], k_begin - b1, k_end - b1);
       u32x4_t vv = u32x4_t{v0[0], v0[1], v1[0], v1[1]};
-#pragma unroll
-      for (int r = 0; r < 4; ++r) o[dt][r] *= corr;
       o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8_t*)&vv, pf, o[dt], 0, 0, 0);
     }
   }
@@ -261,8 +266,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
     float* dst = ws_o + slot * HD;
 #pragma unroll
     for (int dt = 0; dt < HD / 16; ++dt)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) dst[dt * 16 + 4 * qd + r] = o[dt][r];
+      *(f32x4_t*)(dst + dt * 16 + 4 * qd) = o[dt];
     if (qd == 0) {
       ws_ml[slot * 2] = m;
       ws_ml[slot * 2 + 1] = l;
@@ -270,50 +274,83 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
   }
 }
 
-// Combines the splits of one (sequence, head) in split order and writes bfloat16.
-__global__ void attn_decode_merge_kernel(const float* __restrict__ ws_o,
-                                         const float* __restrict__ ws_ml,
-                                         const int* __restrict__ q_start,
-                                         const int* __restrict__ ctx_len, bf16_t* __restrict__ out,
-                                         int window, int nH, int hd, int max_splits,
-                                         int split_keys) {
-  const int s = blockIdx.x, head = blockIdx.y;
+// Combines the splits of one (sequence, head) in split order and writes bfloat16.  One wave:
+// every lane first takes one split's (max, sum) of a chunk of 64 splits, so that the weights
+// exp2(m - max) are formed side by side; then the lanes, each owning hd / 64 output elements,
+// add the partial outputs with eight loads in flight.
+__global__ __launch_bounds__(64) void attn_decode_merge_kernel(
+    const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+    const int* __restrict__ q_start, const int* __restrict__ ctx_len, bf16_t* __restrict__ out,
+    int window, int nH, int hd, int max_splits) {
+  const int s = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   if (q_start[s + 1] - q_start[s] != 1) return;
   const int ctx = ctx_len[s], pos = ctx - 1;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int first = lo / split_keys, last = pos / split_keys;
+  const int first = lo / DEC_SPLIT, last = pos / DEC_SPLIT;
   const size_t base = ((size_t)s * nH + head) * max_splits;
   float mx = -INFINITY;
-  for (int sp = first; sp <= last; ++sp) mx = fmaxf(mx, ws_ml[(base + sp) * 2]);
+  for (int sp = first + lane; sp <= last; sp += 64) mx = fmaxf(mx, ws_ml[(base + sp) * 2]);
+  mx = wave_max(mx);
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
   float denom = 0.f;
-  for (int sp = first; sp <= last; ++sp)
-    denom += exp2f(ws_ml[(base + sp) * 2] - mx) * ws_ml[(base + sp) * 2 + 1];
+  for (int chunk = first; chunk <= last; chunk += 64) {
+    const int mine = chunk + lane;
+    float w_l = 0.f, l_l = 0.f;
+    if (mine <= last) {
+      const float2 ml = *(const float2*)(ws_ml + (base + mine) * 2);
+      w_l = exp2f(ml.x - mx);
+      l_l = ml.y;
+    }
+    denom += wave_sum(w_l * l_l);
+    const int n = min(64, last - chunk + 1);
+    for (int i0 = 0; i0 < n; i0 += 8) {
+      float v[8][8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int sp = min(chunk + i0 + u, last);
+        const float* src = ws_o + (base + sp) * hd;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int d = lane + 64 * i;
+          v[u][i] = (d < hd) ? src[d] : 0.f;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const float w = (i0 + u < n) ? __shfl(w_l, i0 + u, 64) : 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = fmaf(w, v[u][i], acc[i]);
+      }
+    }
+  }
   const float inv = 1.0f / denom;
   bf16_t* orow = out + ((size_t)q_start[s] * nH + head) * hd;
-  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-    float acc = 0.f;
-    for (int sp = first; sp <= last; ++sp)
-      acc += exp2f(ws_ml[(base + sp) * 2] - mx) * ws_o[(base + sp) * hd + d];
-    orow[d] = float_to_bf16(acc * inv);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int d = lane + 64 * i;
+    if (d < hd) orow[d] = float_to_bf16(acc[i] * inv);
   }
 }
 
+// ws_o: n_seqs * nH * max_splits * hd floats, ws_ml: n_seqs * nH * max_splits * 2 floats,
+// max_splits >= ceil(longest context / 64).
 extern "C" int zf_attn_decode_bf16(const void* q, const void* k_pool, const void* v_pool,
                                    const int* block_table, const int* q_start,
                                    const int* ctx_len, void* out, float* ws_o, float* ws_ml,
                                    float scale, int window, int n_seqs, int nH, int nKV, int hd,
-                                   int page_size, int max_pages, int max_splits, int split_keys,
+                                   int page_size, int max_pages, int max_splits,
                                    hipStream_t stream) {
   if (n_seqs <= 0) return 0;
-  if (page_size % 16 != 0 || nKV <= 0 || nH % nKV != 0 || nH / nKV > 16 || split_keys % 32 != 0)
-    return -2;
+  if (page_size % 16 != 0 || nKV <= 0 || nH % nKV != 0 || nH / nKV > 16) return -2;
   const float scale_log2e = scale * 1.4426950408889634f;
   dim3 grid(n_seqs, nKV, max_splits);
 #define ZF_DEC(HD)                                                                              \
   hipLaunchKernelGGL(attn_decode_kernel<HD>, grid, dim3(64), 0, stream, (const bf16_t*)q,       \
                      (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, q_start,        \
                      ctx_len, ws_o, ws_ml, scale_log2e, window, nH, nKV, page_size, max_pages,  \
-                     max_splits, split_keys)
+                     max_splits)
   if (hd == 32) ZF_DEC(32);
   else if (hd == 64) ZF_DEC(64);
   else if (hd == 128) ZF_DEC(128);
@@ -321,7 +358,7 @@ extern "C" int zf_attn_decode_bf16(const void* q, const void* k_pool, const void
   else return -2;
 #undef ZF_DEC
   hipLaunchKernelGGL(attn_decode_merge_kernel, dim3(n_seqs, nH), dim3(64), 0, stream, ws_o, ws_ml,
-                     q_start, ctx_len, (bf16_t*)out, window, nH, hd, max_splits, split_keys);
+                     q_start, ctx_len, (bf16_t*)out, window, nH, hd, max_splits);
   ZF_CHECK_LAUNCH();
 }
 

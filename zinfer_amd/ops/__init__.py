@@ -226,7 +226,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
 
 
 # ------------------------------------------------------------------------- attention
-DECODE_SPLIT_KEYS = 256
+DECODE_SPLIT_KEYS = 64      # keys per split of the decode kernel (DEC_SPLIT in attention.hip)
 
 
 def mfma_attention_covers(dtype, n_heads, n_kv_heads, head_dim, page_size) -> bool:
@@ -277,7 +277,7 @@ def paged_attention(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index,
                 _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), _ptr(q_start),
                 _ptr(ctx_len), _ptr(out), _ptr(ws_o), _ptr(ws_ml), ctypes.c_float(scale),
                 int(window), n_seqs, n_heads, n_kv_heads, head_dim, page_size, max_pages,
-                max_splits, DECODE_SPLIT_KEYS, _stream()), "paged_attention (decode)")
+                max_splits, _stream()), "paged_attention (decode)")
         if n_single != n_seqs and max_q_len > 1:
             _check(lib.zf_attn_prefill_bf16(
                 _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), _ptr(q_start),
