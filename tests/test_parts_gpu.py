@@ -1,0 +1,373 @@
+"""Each part alone on the GPU against the plain functions, the entry point's greedy
+generation, and (c)'s generality: parts defined here, in the test, are registered, built
+from a model folder and stepped without a change to the framework's files: a mixer with
+state of its own, and a model whose layers differ (full and windowed attention), run in an
+order that names layers twice and lets a run read another run's cache."""
+import json
+import os
+from dataclasses import dataclass
+from typing import Optional
+
+import numpy as np
+import pytest
+import torch
+
+import plain
+import tiny
+import traces
+from gpu_util import DEV, rel_err
+
+pytestmark = pytest.mark.gpu
+F64 = torch.float64
+
+
+# ----------------------------------------------------------------------------- harness
+class _StubModel:
+    """Just enough of a model for an Engine to hand out pages and build step contexts."""
+
+    def __init__(self, needs, dtype):
+        from zinfer_amd.config.specs import ModelSpec, ScheduleEntry
+        from zinfer_amd.parts import BuildContext
+        self.ctx = BuildContext(dtype, torch.device(DEV))
+        self._needs = needs
+        self.spec = ModelSpec(vocab_size=100, hidden_size=8, max_positions=4096, layers=(),
+                              schedule=tuple(ScheduleEntry(0) for _ in needs), final_norm=None,
+                              tie_word_embeddings=True)
+
+    def cache_needs(self):
+        return self._needs
+
+
+class _context:
+    """Step context for {request: n_tokens}: pages are reserved on entry, lengths are
+    committed (and pages a window has passed given back) on exit, as Engine.step does."""
+
+    def __init__(self, eng, cuts):
+        self.eng, self.cuts = eng, cuts
+
+    def __enter__(self):
+        from zinfer_amd.engine import StepEntry
+        entries = []
+        for rid, n in self.cuts.items():
+            if not self.eng.cache.has_request(rid):
+                self.eng.cache.add_request(rid)
+            self.eng.cache.reserve(rid, self.eng.cache.length(rid) + n)
+            entries.append(StepEntry(rid, [0] * n, []))
+        return self.eng._build_context(entries)
+
+    def __exit__(self, *exc):
+        for rid, n in self.cuts.items():
+            self.eng.cache.commit(rid, self.eng.cache.length(rid) + n)
+
+
+def _rand(shape, seed, scale=1.0, dtype=torch.float32):
+    return (torch.randn(shape, generator=torch.Generator().manual_seed(seed)) * scale).to(dtype)
+
+
+# ----------------------------------------------------------------------------- parts alone
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rms_norm_part(dtype):
+    from zinfer_amd.config.specs import RmsNormSpec
+    from zinfer_amd.parts import BuildContext, build_part
+    part = build_part("norm", RmsNormSpec(80, 3e-6), BuildContext(dtype, torch.device(DEV)), "n.")
+    assert list(part.declare()) == ["n.weight"] and part.declare()["n.weight"].shape == (80,)
+    g = 1 + 0.1 * _rand((80,), 1)
+    part.bind({"n.weight": g.to(dtype)})
+    x = _rand((7, 80), 2, 3.0)
+    out = torch.empty((7, 80), dtype=dtype, device=DEV)
+    part.forward(x.to(DEV), out)
+    want = plain.rms_norm(x, g.to(dtype), 3e-6)
+    assert rel_err(out, want) <= (2e-5 if dtype == torch.float32 else 2 ** -8)
+
+
+def test_rotary_tables_follow_the_plain_angles():
+    from zinfer_amd.parts.position import rotary_tables
+    for hd, theta in ((16, 1e4), (128, 1e6), (48, 5e4)):
+        cos, sin = rotary_tables(hd, theta, 300)
+        for p in (0, 1, 2, 77, 299):
+            c, s = plain.rope_cos_sin(p, hd, theta)
+            assert torch.allclose(cos[p].double(), c, atol=1e-7)
+            assert torch.allclose(sin[p].double(), s, atol=1e-7)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu_part(dtype):
+    from zinfer_amd.config.specs import SwiGluSpec
+    from zinfer_amd.engine import Engine
+    from zinfer_amd.parts import build_part
+    stub = _StubModel([], dtype)
+    eng = Engine(stub, num_pages=4, max_requests=2)
+    part = build_part("feed_forward", SwiGluSpec(96, 200), stub.ctx, "mlp.")
+    w = {"mlp.gate_proj.weight": _rand((200, 96), 3, 0.1, dtype),
+         "mlp.up_proj.weight": _rand((200, 96), 4, 0.1, dtype),
+         "mlp.down_proj.weight": _rand((96, 200), 5, 0.1, dtype)}
+    part.bind(w)
+    h = _rand((5, 96), 6, 1.0, dtype)
+    residual = _rand((5, 96), 7)
+    res = residual.clone().to(DEV)
+    with _context(eng, {"a": 5}) as ctx:
+        part.forward(h.to(DEV), res, ctx)
+    want = residual.double() + plain.linear(
+        plain.swiglu(plain.linear(h, w["mlp.gate_proj.weight"]),
+                     plain.linear(h, w["mlp.up_proj.weight"])), w["mlp.down_proj.weight"])
+    assert rel_err(res, want) <= (2e-5 if dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("qk_norm,window,rope", [(True, None, True), (False, 9, True),
+                                                 (True, None, False)])
+def test_attention_part(dtype, qk_norm, window, rope):
+    """The attention mixer alone over two steps (a portion, then single tokens) against the
+    plain single-query attention with the same projections."""
+    from zinfer_amd.config.specs import GqaAttentionSpec, NoPositionSpec, RotaryHalfSplitSpec
+    from zinfer_amd.engine import Engine
+    from zinfer_amd.parts import build_part
+    H, nH, nKV, hd, eps, theta = 96, 6, 2, 32, 1e-5, 1e4
+    pos_spec = RotaryHalfSplitSpec(hd, theta, 256) if rope else NoPositionSpec()
+    spec = GqaAttentionSpec(H, nH, nKV, hd, eps if qk_norm else None, pos_spec, window)
+    stub = _StubModel([None], dtype)
+    part = build_part("mixer", spec, stub.ctx, "a.")
+    stub._needs = [part.cache_need()]
+    eng = Engine(stub, page_size=16, num_pages=8, max_requests=2, poison_freed=True)
+    w = {"a.q_proj.weight": _rand((nH * hd, H), 1, 0.1, dtype),
+         "a.k_proj.weight": _rand((nKV * hd, H), 2, 0.1, dtype),
+         "a.v_proj.weight": _rand((nKV * hd, H), 3, 0.1, dtype),
+         "a.o_proj.weight": _rand((H, nH * hd), 4, 0.1, dtype)}
+    if qk_norm:
+        w["a.q_norm.weight"] = (1 + 0.1 * _rand((hd,), 5)).to(dtype)
+        w["a.k_norm.weight"] = (1 + 0.1 * _rand((hd,), 6)).to(dtype)
+    assert set(part.declare()) == set(w)
+    part.bind(w)
+    T = 40
+    h = _rand((T, H), 7, 1.0, dtype)
+    # plain: token after token
+    ks, vs, want = [], [], []
+    for p in range(T):
+        q = plain.linear(h[p], w["a.q_proj.weight"])
+        k = plain.linear(h[p], w["a.k_proj.weight"])
+        v = plain.linear(h[p], w["a.v_proj.weight"])
+        if qk_norm:
+            q = plain.per_head_rms_norm(q, nH, hd, w["a.q_norm.weight"], eps)
+            k = plain.per_head_rms_norm(k, nKV, hd, w["a.k_norm.weight"], eps)
+        if rope:
+            q, k = plain.rope_heads(q, nH, hd, p, theta), plain.rope_heads(k, nKV, hd, p, theta)
+        ks.append(k.reshape(nKV, hd)); vs.append(v.reshape(nKV, hd))
+        o = plain.attention_single_query(q, torch.stack(ks), torch.stack(vs), nH, nKV, hd, window)
+        want.append(plain.linear(o, w["a.o_proj.weight"]))
+    want = torch.stack(want)
+    got = torch.zeros((T, H), device=DEV)
+    done = 0
+    for n in (23, 1, 1, 13, 2):
+        with _context(eng, {"r": n}) as ctx:
+            part.forward(h[done:done + n].to(DEV).contiguous(), got[done:done + n], ctx,
+                         eng.views[0])
+        done += n
+    assert rel_err(got, want) <= (2e-5 if dtype == torch.float32 else 1.5e-2)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_entry_point(dtype, tmp_path):
+    from zinfer_amd.entrypoints import LLM
+    from zinfer_amd.sampling import SamplingParams
+    name = "D" if dtype == "bfloat16" else "B"
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    path = tiny.model_dir_of(name, str(tmp_path), store)
+    cfg, w = tiny.CONFIGS[name], tiny.weights_of(name, store)
+    prompts = [tiny.random_tokens(n, cfg["vocab_size"], 40 + n) for n in (1, 9, 33, 64, 130)]
+    llm = LLM(path, dtype=dtype, device=DEV, page_size=tiny.PAGE_SIZE[name], max_tokens=448,
+              max_step_tokens=48, chunk_size=24)
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=12,
+                                                ignore_eos=True))
+    assert not llm.engine.cache.requests
+    for p, got in zip(prompts, outs):
+        if dtype == "float32":
+            assert got == plain.greedy_generate(cfg, w, p, 12)
+        else:       # a near-tie may flip in bfloat16: every token must be a near-best one
+            toks = list(p)
+            for g in got:
+                logits = plain.model_forward_batched(cfg, w, toks)[-1]
+                assert logits[g] >= logits.max() - 0.04 * logits.abs().max()
+                toks.append(g)
+    # seeded sampling: the same seed gives the same tokens, alone or in a batch
+    sp = SamplingParams(temperature=0.8, top_k=50, seed=3, max_new_tokens=10, ignore_eos=True)
+    alone = llm.generate([prompts[2]], sp)[0]
+    again = llm.generate([prompts[2]], sp)[0]
+    assert alone == again and len(alone) == 10
+
+
+# ----------------------------------------------------------------------------- toy parts
+@dataclass(frozen=True)
+class ToyStateSpec:
+    """A mixer with state of its own: s <- decay * s + W_in h_t ; out_t = W_out s."""
+    hidden_size: int
+    state_size: int
+    decay: float
+
+
+def _register_toy_state():
+    from zinfer_amd.parts import Mixer, StateNeed, TensorDecl, register_part
+
+    class ToyStateMixer(Mixer):
+        def declare(self):
+            s = self.spec
+            return {self.prefix + "in.weight": TensorDecl((s.state_size, s.hidden_size)),
+                    self.prefix + "out.weight": TensorDecl((s.hidden_size, s.state_size))}
+
+        def bind(self, tensors):
+            self.w_in = tensors[self.prefix + "in.weight"].float().to(self.ctx.device)
+            self.w_out = tensors[self.prefix + "out.weight"].float().to(self.ctx.device)
+
+        def cache_need(self):
+            return StateNeed((self.spec.state_size,), torch.float32)
+
+        def forward(self, h, residual, step, cache):
+            u = h.float() @ self.w_in.T                      # [T, S]
+            start = 0
+            for n, slot in zip(step.q_lens, step.slots):     # each request's tokens in order
+                s = cache.state[slot]
+                for t in range(start, start + n):
+                    s = self.spec.decay * s + u[t]
+                    residual[t] += s @ self.w_out.T
+                cache.state[slot] = s
+                start += n
+
+    register_part("mixer", ToyStateSpec, ToyStateMixer)
+
+
+@dataclass(frozen=True)
+class ToyConfig:
+    hidden_size: int
+    state_size: int
+    decay: float
+    window: int
+    vocab_size: int
+    kind: str                  # "state" or "mixed"
+    model_type: str = "toy"
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(**{k: raw[k] for k in ("hidden_size", "state_size", "decay", "window",
+                                          "vocab_size", "kind")})
+
+    def to_dict(self):
+        return dict(architectures=["ToyForCausalLM"], model_type="toy",
+                    hidden_size=self.hidden_size, state_size=self.state_size, decay=self.decay,
+                    window=self.window, vocab_size=self.vocab_size, kind=self.kind)
+
+    def model_spec(self):
+        from zinfer_amd.config.specs import (GqaAttentionSpec, ModelSpec, PreNormBlockSpec,
+                                             RmsNormSpec, RotaryHalfSplitSpec, ScheduleEntry,
+                                             SwiGluSpec)
+        H = self.hidden_size
+        norm = RmsNormSpec(H, 1e-5)
+        ff = SwiGluSpec(H, 2 * H)
+        rope = RotaryHalfSplitSpec(32, 1e4, 512)
+        full = GqaAttentionSpec(H, 4, 2, 32, 1e-5, rope, None)
+        win = GqaAttentionSpec(H, 4, 2, 32, None, rope, self.window)
+        state = ToyStateSpec(H, self.state_size, self.decay)
+        blk = lambda m: PreNormBlockSpec(mixer=m, feed_forward=ff, mixer_norm=norm, ff_norm=norm)
+        if self.kind == "state":
+            layers = (blk(state), blk(full), blk(state))
+            schedule = (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2))
+        else:   # layers differ; 0 and 1 run twice; the last run reads the cache of run 1
+            layers = (blk(full), blk(win))
+            schedule = (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0),
+                        ScheduleEntry(1, cache_of=1))
+        return ModelSpec(vocab_size=self.vocab_size, hidden_size=H, max_positions=512,
+                         layers=layers, schedule=schedule, final_norm=norm,
+                         tie_word_embeddings=True)
+
+
+def _toy_plain(cfg: ToyConfig, w, toks):
+    """Whole sequence, token after token, from the plain part functions."""
+    spec = cfg.model_spec()
+    H = cfg.hidden_size
+    caches = [([], []) for _ in spec.schedule]
+    states = [torch.zeros(cfg.state_size, dtype=F64) for _ in spec.schedule]
+    rows = []
+    for p, tok in enumerate(toks):
+        x = w["model.embed_tokens.weight"][tok].to(F64)
+        for pos, e in enumerate(spec.schedule):
+            pre = f"model.layers.{e.layer}."
+            blk = spec.layers[e.layer]
+            n = plain.rms_norm(x, w[pre + "input_layernorm.weight"], 1e-5)
+            m = blk.mixer
+            if isinstance(m, ToyStateSpec):
+                states[pos] = m.decay * states[pos] + plain.linear(n, w[pre + "self_attn.in.weight"])
+                x = x + plain.linear(states[pos], w[pre + "self_attn.out.weight"])
+            else:
+                q = plain.linear(n, w[pre + "self_attn.q_proj.weight"])
+                k = plain.linear(n, w[pre + "self_attn.k_proj.weight"])
+                v = plain.linear(n, w[pre + "self_attn.v_proj.weight"])
+                if m.qk_norm_eps is not None:
+                    q = plain.per_head_rms_norm(q, 4, 32, w[pre + "self_attn.q_norm.weight"], 1e-5)
+                    k = plain.per_head_rms_norm(k, 2, 32, w[pre + "self_attn.k_norm.weight"], 1e-5)
+                q, k = plain.rope_heads(q, 4, 32, p, 1e4), plain.rope_heads(k, 2, 32, p, 1e4)
+                src = pos if e.cache_of is None else e.cache_of
+                if e.cache_of is None:
+                    caches[pos][0].append(k.reshape(2, 32)); caches[pos][1].append(v.reshape(2, 32))
+                o = plain.attention_single_query(q, torch.stack(caches[src][0]),
+                                                 torch.stack(caches[src][1]), 4, 2, 32, m.window)
+                x = x + plain.linear(o, w[pre + "self_attn.o_proj.weight"])
+            mm = plain.rms_norm(x, w[pre + "post_attention_layernorm.weight"], 1e-5)
+            x = x + plain.linear(plain.swiglu(plain.linear(mm, w[pre + "mlp.gate_proj.weight"]),
+                                              plain.linear(mm, w[pre + "mlp.up_proj.weight"])),
+                                 w[pre + "mlp.down_proj.weight"])
+        rows.append(plain.linear(plain.rms_norm(x, w["model.norm.weight"], 1e-5),
+                                 w["model.embed_tokens.weight"]))
+    return torch.stack(rows).numpy()
+
+
+@pytest.mark.parametrize("kind", ["state", "mixed"])
+def test_toy_architecture_registered_built_and_stepped(kind, tmp_path):
+    """A model folder of an architecture that exists only in this test: config.json names
+    it, the registry finds it, the loader binds its tensors, the cache manager gives it
+    state slots / windowed pages, the engine steps it under every cutting."""
+    from zinfer_amd.config import register_architecture, unregister_architecture
+    from zinfer_amd.engine import StepEntry
+    from zinfer_amd.engine.replay import make_engine
+    from zinfer_amd.parts import unregister_part
+    from zinfer_amd.weights import SafetensorsFile, write_model_dir
+    _register_toy_state()
+    register_architecture("ToyForCausalLM", ToyConfig, model_type="toy")
+    try:
+        cfg = ToyConfig(hidden_size=64, state_size=24, decay=0.9, window=19, vocab_size=300,
+                        kind=kind)
+        path = write_model_dir(str(tmp_path / "toy"), cfg, seed=5, dtype=torch.float32)
+        with SafetensorsFile(os.path.join(path, "model.safetensors")) as f:
+            w = {n: f.tensor(n) for n in f.names()}
+        requests = {f"q{i}": tiny.random_tokens(n, 300, 70 + i) for i, n in enumerate((50, 7, 90, 33))}
+        ref = {rid: _toy_plain(cfg, w, t) for rid, t in requests.items()}
+        outs = {}
+        for mode in ("whole", "portions", "mixed", "prefill_then_32"):
+            steps = {"whole": traces.whole, "portions": traces.changing_portions,
+                     "mixed": traces.mixed, "prefill_then_32": traces.prefill_then_single}[mode](requests)
+            eng = make_engine(path, "float32", traces.peak_tokens(steps, 64), DEV, poison_freed=True)
+            if kind == "state":
+                assert len(eng.cache.state_pools) == 2 and len(eng.cache.groups) == 1
+            else:
+                assert len(eng.cache.groups) == 2      # full and windowed pages apart
+                assert eng.views[3].k_pool.data_ptr() == eng.views[1].k_pool.data_ptr()
+                assert not eng.views[3].writes
+            got_steps = {}
+            for st in steps:
+                lg = eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]],
+                              end=st["end"])
+                if lg.shape[0]:
+                    got_steps[st["step"]] = lg.cpu().numpy()
+            eng.cache.check()
+            outs[mode] = traces.collect(steps, got_steps, 300)
+            for rid in requests:
+                err = np.abs(outs[mode][rid] - ref[rid]).max() / np.abs(ref[rid]).max()
+                assert err <= 2e-5, f"{kind} {mode} {rid}: {err:.3g}"
+        if kind == "mixed":
+            # the windowed group gave pages back while requests were still running
+            steps = traces.changing_portions({"w": requests["q2"]})
+            eng = make_engine(path, "float32", 128, DEV)
+            for st in steps:
+                eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]])
+            held = [g.pages.num_held for g in eng.cache.groups]
+            assert held[0] == 6 and held[1] <= 3       # 90 tokens: 6 pages; window 19: <= 3
+    finally:
+        unregister_architecture("ToyForCausalLM")
+        unregister_part("mixer", ToyStateSpec)

@@ -49,7 +49,8 @@ class Engine:
         self.steps_run = 0
         # decode-only steps (one token per request) are launch-bound: they are captured once
         # per batch shape into a HIP graph and replayed
-        self.use_graphs = use_graphs and self.device.type == "cuda"
+        self.use_graphs = use_graphs and self.device.type == "cuda" \
+            and getattr(model, "graph_safe", False)
         self._graphs: Dict[tuple, tuple] = {}
         self.graph_replays = 0
 

@@ -22,6 +22,7 @@ class DecoderModel:
         self.blocks = [build_part("block", b, ctx, spec.layer_prefix.format(i))
                        for i, b in enumerate(spec.layers)]
         self.final_norm = build_part("norm", spec.final_norm, ctx, spec.final_norm_prefix)
+        self.graph_safe = self.final_norm.graph_safe and all(b.graph_safe for b in self.blocks)
         for pos, e in enumerate(spec.schedule):
             if not (0 <= e.layer < len(self.blocks)):
                 raise ConfigError(f"schedule[{pos}] names layer {e.layer} of {len(self.blocks)}")

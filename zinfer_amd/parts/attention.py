@@ -18,6 +18,8 @@ class GqaAttention(Mixer):
     optional per-head RMSNorm of q and k, position encoding of q and k, append (k, v) at the
     token's position, softmax(q K^T / sqrt(hd)) V over the positions up to the token's own
     (query head h reads kv head h // G), output projection added to the residual."""
+    graph_safe = True
+
 
     def __init__(self, spec: GqaAttentionSpec, ctx, prefix):
         super().__init__(spec, ctx, prefix)
@@ -32,6 +34,7 @@ class GqaAttention(Mixer):
         self.kv_width = s.n_kv_heads * s.head_dim
         self.scale = s.scale if s.scale is not None else 1.0 / math.sqrt(float(s.head_dim))
         self.position = build_part("position", s.position, ctx, prefix)
+        self.graph_safe = self.position.graph_safe
 
     def declare(self) -> Dict[str, TensorDecl]:
         s, p = self.spec, self.prefix

@@ -67,7 +67,11 @@ class BuildContext:
 
 
 class Part:
+    """``graph_safe`` says that ``forward`` only launches work on the current stream whose
+    arguments depend on the step's device tensors and sizes, never on its host-side lists
+    (``q_lens``, ``slots``, ...): only then may a decode step be captured once and replayed."""
     role = ""
+    graph_safe = False
 
     def __init__(self, spec, ctx: BuildContext, prefix: str):
         self.spec = spec

@@ -19,6 +19,7 @@ class PreNormBlock(Block):
         self.feed_forward = build_part("feed_forward", spec.feed_forward, ctx,
                                        prefix + spec.ff_prefix)
         self.parts = (self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward)
+        self.graph_safe = all(p.graph_safe for p in self.parts)
 
     def declare(self) -> Dict[str, TensorDecl]:
         d: Dict[str, TensorDecl] = {}

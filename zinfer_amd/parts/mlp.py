@@ -15,6 +15,8 @@ class SwiGluMlp(FeedForward):
     (`src/model/runtime/optimized_decoder/layer.zig:194-201`, `src/kernel/core/cpu.zig:130-147`).
     gate and up rows are stacked into one matrix at load: each output keeps its own dot
     product."""
+    graph_safe = True
+
 
     def declare(self) -> Dict[str, TensorDecl]:
         s, p = self.spec, self.prefix

@@ -13,6 +13,8 @@ from .linear import place_gain
 class RmsNorm(Norm):
     """n = x * w / sqrt(mean(x^2) + eps) (`src/kernel/core/cpu.zig:38-48,73-110`); reads the
     float32 residual stream, writes the activation dtype."""
+    graph_safe = True
+
 
     def declare(self) -> Dict[str, TensorDecl]:
         return {self.prefix + "weight": TensorDecl((self.spec.width,), init="gain")}

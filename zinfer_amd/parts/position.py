@@ -27,6 +27,8 @@ def rotary_tables(head_dim: int, theta: float, max_positions: int):
 class RotaryHalfSplit(PositionEncoding):
     """Half-split rotation over the full head (`src/kernel/attention/rope.zig:92-109`); the
     attention kernel applies it from the tables."""
+    graph_safe = True
+
 
     def __init__(self, spec, ctx, prefix):
         super().__init__(spec, ctx, prefix)
@@ -40,6 +42,8 @@ class RotaryHalfSplit(PositionEncoding):
 
 class NoPosition(PositionEncoding):
     """q and k go into the attention as they are."""
+    graph_safe = True
+
 
 
 register_part("position", RotaryHalfSplitSpec, RotaryHalfSplit)
