@@ -34,6 +34,10 @@ class Engine:
                  poison_freed: bool = False, use_graphs: bool = True):
         self.model = model
         self.device = model.ctx.device
+        if self.device.type == "cuda":
+            # what this model needs is built now, side by side, if it is not built yet
+            from ..ops import build
+            build.prepare(getattr(model, "kernel_modules", ()))
         spec = model.spec
         needs = model.cache_needs()
         reads = [e.cache_of for e in spec.schedule]

@@ -23,6 +23,9 @@ class DecoderModel:
                        for i, b in enumerate(spec.layers)]
         self.final_norm = build_part("norm", spec.final_norm, ctx, spec.final_norm_prefix)
         self.graph_safe = self.final_norm.graph_safe and all(b.graph_safe for b in self.blocks)
+        # embedding, row gather and head are the model's own launches
+        self.kernel_modules = tuple(sorted(
+            {"elementwise", "gemm"} | {m for b in self.blocks for m in b.kernel_modules}))
         for pos, e in enumerate(spec.schedule):
             if not (0 <= e.layer < len(self.blocks)):
                 raise ConfigError(f"schedule[{pos}] names layer {e.layer} of {len(self.blocks)}")

@@ -19,6 +19,7 @@ class GqaAttention(Mixer):
     token's position, softmax(q K^T / sqrt(hd)) V over the positions up to the token's own
     (query head h reads kv head h // G), output projection added to the residual."""
     graph_safe = True
+    kernel_modules = ("elementwise", "gemm", "attention")
 
 
     def __init__(self, spec: GqaAttentionSpec, ctx, prefix):

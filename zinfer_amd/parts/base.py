@@ -72,6 +72,7 @@ class Part:
     (``q_lens``, ``slots``, ...): only then may a decode step be captured once and replayed."""
     role = ""
     graph_safe = False
+    kernel_modules = ()        # names of the HIP kernel libraries the part launches
 
     def __init__(self, spec, ctx: BuildContext, prefix: str):
         self.spec = spec

@@ -20,6 +20,7 @@ class PreNormBlock(Block):
                                        prefix + spec.ff_prefix)
         self.parts = (self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward)
         self.graph_safe = all(p.graph_safe for p in self.parts)
+        self.kernel_modules = tuple(sorted({m for p in self.parts for m in p.kernel_modules}))
 
     def declare(self) -> Dict[str, TensorDecl]:
         d: Dict[str, TensorDecl] = {}

@@ -16,6 +16,7 @@ class SwiGluMlp(FeedForward):
     gate and up rows are stacked into one matrix at load: each output keeps its own dot
     product."""
     graph_safe = True
+    kernel_modules = ("elementwise", "gemm")
 
 
     def declare(self) -> Dict[str, TensorDecl]:

@@ -14,6 +14,7 @@ class RmsNorm(Norm):
     """n = x * w / sqrt(mean(x^2) + eps) (`src/kernel/core/cpu.zig:38-48,73-110`); reads the
     float32 residual stream, writes the activation dtype."""
     graph_safe = True
+    kernel_modules = ("elementwise",)
 
 
     def declare(self) -> Dict[str, TensorDecl]:
