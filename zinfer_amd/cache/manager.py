@@ -58,6 +58,8 @@ class KVGroup:
     def pages_missing(self, rid, length: int, new_len: int) -> int:
         table = self.tables[rid]
         last = (new_len + self.page_size - 1) // self.page_size
+        if self.need.window is None:       # no holes: every page up to len(table) is held
+            return max(0, last - len(table))
         first = self.first_needed_page(length)
         return sum(1 for i in range(first, last) if i >= len(table) or table[i] == NO_PAGE)
 
@@ -208,6 +210,9 @@ class CacheManager:
         return self.groups[group].tables[rid]
 
     # ------------------------------------------------------------------ accounting
+    def num_free_slots(self) -> int:
+        return self._slots.num_free
+
     def num_free_pages(self) -> List[int]:
         return [g.pages.num_free for g in self.groups]
 

@@ -196,10 +196,17 @@ class Engine:
             o, n = offs[name]
             host[o:o + len(values)] = values
 
-        put("token_ids", np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries]))
-        put("positions", np.concatenate([np.arange(s, s + n, dtype=np.int32)
-                                         for s, n in zip(starts, q_lens)]))
-        put("seq_index", np.repeat(np.arange(n_seqs, dtype=np.int32), q_lens))
+        single = max(q_lens) == 1
+        if single:
+            put("token_ids", np.fromiter((e.tokens[0] for e in entries), np.int32, n_seqs))
+            put("positions", np.asarray(starts, dtype=np.int32))
+            put("seq_index", np.arange(n_seqs, dtype=np.int32))
+        else:
+            put("token_ids", np.concatenate([np.asarray(e.tokens, dtype=np.int32)
+                                             for e in entries]))
+            put("positions", np.concatenate([np.arange(s, s + n, dtype=np.int32)
+                                             for s, n in zip(starts, q_lens)]))
+            put("seq_index", np.repeat(np.arange(n_seqs, dtype=np.int32), q_lens))
         put("q_start", np.asarray(q_start, dtype=np.int32))
         put("ctx_len", np.asarray(ctx_lens, dtype=np.int32))
         put("state_slots", np.asarray(slots, dtype=np.int32))
@@ -208,10 +215,14 @@ class Engine:
             bt = np.full((n_seqs, max_pages), NO_PAGE, dtype=np.int32)
             sm = np.empty((T,), dtype=np.int32)
             for i, e in enumerate(entries):
-                table = np.asarray(self.cache.table(g, e.request_id), dtype=np.int32)
-                bt[i, :len(table)] = table[:max_pages]
-                pos = np.arange(starts[i], ctx_lens[i])
-                sm[q_start[i]:q_start[i + 1]] = table[pos // ps] * ps + pos % ps
+                table = self.cache.table(g, e.request_id)
+                bt[i, :len(table)] = table
+                if q_lens[i] == 1:
+                    p = starts[i]
+                    sm[q_start[i]] = table[p // ps] * ps + p % ps
+                else:
+                    pos = np.arange(starts[i], ctx_lens[i])
+                    sm[q_start[i]:q_start[i + 1]] = bt[i, pos // ps] * ps + pos % ps
             if (sm < 0).any():
                 raise StepError("a token would be written to a page that is not held")
             put(f"slot_mapping{g}", sm)

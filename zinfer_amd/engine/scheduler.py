@@ -98,13 +98,20 @@ class Scheduler:
         while True:
             planned: List[PlannedEntry] = []
             budget = self.max_step_tokens
-            wanted: List[Tuple[object, int]] = []
+            # pages and request slots the entries planned so far will take
+            taken = [0] * len(self.cache.groups)
+            free = self.cache.num_free_pages()
+            new_slots = [0]
 
             def try_add(req: Request, n: int) -> bool:
-                trial = wanted + [(req.id, req.n_computed + n)]
-                if not self.cache.can_reserve(trial):
+                need = self.cache.pages_missing(req.id, req.n_computed + n)
+                slot = 0 if self.cache.has_request(req.id) else 1
+                if new_slots[0] + slot > self.cache.num_free_slots() or \
+                        any(t + m > f for t, m, f in zip(taken, need, free)):
                     return False
-                wanted.append(trial[-1])
+                for g, m in enumerate(need):
+                    taken[g] += m
+                new_slots[0] += slot
                 planned.append(PlannedEntry(req, n, n == req.pending))
                 return True
 
@@ -117,8 +124,9 @@ class Scheduler:
                     elif starved is None:
                         starved = req
             # 2. running requests still in their prompt (or recomputing)
+            in_plan = {id(p.request) for p in planned}
             for req in self.running:
-                if any(p.request is req for p in planned) or req is starved:
+                if id(req) in in_plan or req is starved:
                     continue
                 if req.pending == 1 and req.generated:
                     continue
