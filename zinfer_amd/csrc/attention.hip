@@ -363,7 +363,7 @@ extern "C" int zf_attn_decode_bf16(const void* q, const void* k_pool, const void
 }
 
 // ---------------------------------------------------------------- prefill: portions of prompts
-// Grid (sequence, tile of 32 queries, kv head); wave w of a workgroup takes the query heads
+// One workgroup per (sequence, tile of 32 queries, kv head); wave w takes the query heads
 // w, w + waves, ... of the kv head.  32x32x16 MFMAs: S^T tile of 32 keys x 32 queries,
 // O^T tiles of 32 head elements x 32 queries.  A query at position p reads keys lo..p; a
 // portion may start anywhere in the context (earlier pages plus its own tokens).
@@ -373,8 +373,14 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int* __restrict__ block_table,
     const int* __restrict__ q_start, const int* __restrict__ ctx_len, bf16_t* __restrict__ out,
-    float scale_log2e, int window, int nH, int nKV, int ps, int max_pages, int skip_single) {
-  const int s = blockIdx.x, qt = blockIdx.y, kvh = blockIdx.z;
+    float scale_log2e, int window, int nH, int nKV, int ps, int max_pages, int skip_single,
+    int q_tiles) {
+  // workgroups are handed out in the order of blockIdx.x: kv heads vary fastest and the
+  // last query tiles (the longest key ranges under the causal bound) come first, so the
+  // heavy tiles do not end up as the tail
+  const int kvh = blockIdx.x % nKV;
+  const int qt = q_tiles - 1 - (blockIdx.x / nKV) % q_tiles;
+  const int s = blockIdx.x / (nKV * q_tiles);
   const int q_len = q_start[s + 1] - q_start[s];
   if (q_len == 1 && skip_single) return;
   const int qbase = qt * 32;
@@ -412,21 +418,45 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
       for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
     float m = -INFINITY, l = 0.f;
 
-    for (int kb = (lo_min / 32) * 32; kb <= p_max; kb += 32) {
+    // The loop is software-pipelined: the key rows of the next tile and the value rows of
+    // this tile are requested before this tile's scores are computed, so that two rounds of
+    // memory latency overlap the MFMAs and the soft-max.
+    auto load_keys = [&](int kb, u32x4_t* dst) {
+      const int key = min(max(kb + j, lo_min), p_max);
+      const int kpage = table[key / ps];
+      const bf16_t* krow = k_pool + (((size_t)kpage * nKV + kvh) * ps + key % ps) * HD + 8 * hf;
+#pragma unroll
+      for (int stp = 0; stp < HD / 16; ++stp) dst[stp] = *(const u32x4_t*)(krow + stp * 16);
+    };
+    const int kb0 = (lo_min / 32) * 32;
+    u32x4_t kf[HD / 16];
+    load_keys(kb0, kf);
+    for (int kb = kb0; kb <= p_max; kb += 32) {
+      // values of this tile: keys kb + 16 u .. + 15 (one page) for u = 0, 1
+      u32x2_t vf[2][HD / 32][2];
+      bool any[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int base = kb + 16 * u;
+        any[u] = base <= p_max && base + 16 > lo_min;
+        const int safe = any[u] ? max(base, lo_min) : p_max;
+        const int vpage = table[safe / ps];
+        const int off = base % ps + 4 * hf;
+        const bf16_t* vb = v_pool + ((size_t)vpage * nKV + kvh) * ps * HD + (size_t)j * ps + off;
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt) {
+          vf[u][dt][0] = *(const u32x2_t*)(vb + (size_t)dt * 32 * ps);
+          vf[u][dt][1] = *(const u32x2_t*)(vb + (size_t)dt * 32 * ps + 8);
+        }
+      }
       // S^T: rows are the keys kb + (lane % 32), clamped into the keys that exist
       f32x16_t st;
 #pragma unroll
       for (int r = 0; r < 16; ++r) st[r] = 0.f;
-      {
-        const int key = min(max(kb + j, lo_min), p_max);
-        const int kpage = table[key / ps];
-        const bf16_t* krow = k_pool + (((size_t)kpage * nKV + kvh) * ps + key % ps) * HD + 8 * hf;
 #pragma unroll
-        for (int stp = 0; stp < HD / 16; ++stp) {
-          const u32x4_t kv = *(const u32x4_t*)(krow + stp * 16);
-          st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&kv, qf[stp], st, 0, 0, 0);
-        }
-      }
+      for (int stp = 0; stp < HD / 16; ++stp)
+        st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&kf[stp], qf[stp], st, 0, 0, 0);
+      if (kb + 32 <= p_max) load_keys(kb + 32, kf);      // next tile's keys, in flight from here
       // st[r]: key kb + 8 (r / 4) + 4 hf + r % 4, query column j
       float tmax = -INFINITY;
 #pragma unroll
@@ -456,29 +486,25 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
         for (int r = 0; r < 16; ++r) o[dt][r] *= corr;
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        // keys kb + 16 u .. + 15 (one page); slots e = 0..7 <-> st[8 u + e]:
-        // keys kb + 16 u + 4 hf + e (e < 4) and kb + 16 u + 8 + 4 hf + (e - 4)
+        // slots e = 0..7 <-> st[8 u + e]: keys kb + 16 u + 4 hf + e (e < 4) and
+        // kb + 16 u + 8 + 4 hf + (e - 4)
         u32x4_t pk = u32x4_t{pack_bf16(st[8 * u + 0], st[8 * u + 1]),
                              pack_bf16(st[8 * u + 2], st[8 * u + 3]),
                              pack_bf16(st[8 * u + 4], st[8 * u + 5]),
                              pack_bf16(st[8 * u + 6], st[8 * u + 7])};
         const bf16x8_t pf = *(bf16x8_t*)&pk;
-        const int base = kb + 16 * u;
-        const bool any = base <= p_max && base + 16 > lo_min;
-        const int safe = any ? max(base, lo_min) : p_max;
-        const int vpage = table[safe / ps];
-        const int off = base % ps + 4 * hf;
-        const bf16_t* vb = v_pool + ((size_t)vpage * nKV + kvh) * ps * HD + (size_t)j * ps + off;
         // keys at or beyond ctx hold nothing of this request; keys below lo_min may lie in
         // a page that was given back: both are zeroed (0 * NaN would poison the sum)
-        const int a0 = base + 4 * hf, a1 = a0 + 8;
-        const int hi_lim = any ? ctx : 0;
+        const int a0 = kb + 16 * u + 4 * hf, a1 = a0 + 8;
+        const int hi_lim = any[u] ? ctx : 0;
+        const bool edge = !any[u] || a0 < lo_min || a1 + 4 > ctx;
 #pragma unroll
         for (int dt = 0; dt < HD / 32; ++dt) {
-          u32x2_t v0 = *(const u32x2_t*)(vb + (size_t)dt * 32 * ps);
-          u32x2_t v1 = *(const u32x2_t*)(vb + (size_t)dt * 32 * ps + 8);
-          v0 = keep_range4(v0, lo_min - a0, hi_lim - a0);
-          v1 = keep_range4(v1, lo_min - a1, hi_lim - a1);
+          u32x2_t v0 = vf[u][dt][0], v1 = vf[u][dt][1];
+          if (edge) {
+            v0 = keep_range4(v0, lo_min - a0, hi_lim - a0);
+            v1 = keep_range4(v1, lo_min - a1, hi_lim - a1);
+          }
           u32x4_t vv = u32x4_t{v0[0], v0[1], v1[0], v1[1]};
           o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8_t*)&vv, pf, o[dt], 0, 0, 0);
         }
@@ -510,13 +536,14 @@ extern "C" int zf_attn_prefill_bf16(const void* q, const void* k_pool, const voi
   if (page_size % 16 != 0 || nKV <= 0 || nH % nKV != 0) return -2;
   const float scale_log2e = scale * 1.4426950408889634f;
   const int G = nH / nKV;
-  dim3 grid(n_seqs, (max_q_len + 31) / 32, nKV);
+  const int q_tiles = (max_q_len + 31) / 32;
+  dim3 grid((unsigned)n_seqs * q_tiles * nKV);
   dim3 block(64 * (G < 8 ? G : 8));
 #define ZF_PRE(HD)                                                                              \
   hipLaunchKernelGGL(attn_prefill_kernel<HD>, grid, block, 0, stream, (const bf16_t*)q,         \
                      (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, q_start,        \
                      ctx_len, (bf16_t*)out, scale_log2e, window, nH, nKV, page_size, max_pages, \
-                     skip_single)
+                     skip_single, q_tiles)
   if (hd == 32) ZF_PRE(32);
   else if (hd == 64) ZF_PRE(64);
   else if (hd == 128) ZF_PRE(128);
