@@ -358,3 +358,68 @@ def test_cpu_tensor_is_refused():
     from zinfer_amd.errors import KernelUnavailable
     with pytest.raises(KernelUnavailable):
         _ops().rmsnorm(torch.zeros((1, 4)), torch.ones(4), 1e-6, torch.zeros((1, 4)))
+
+
+@pytest.mark.parametrize("V", [1000, 151936, 7])
+def test_sample_topk_against_the_host_sampler(V):
+    """The device sampler draws the token the host sampler (the reference's semantics) draws
+    for the same uniform number.  Device and host exponentials may differ in the last bit,
+    which can only matter when u * sum falls within that rounding of a boundary between two
+    candidates: then the neighbouring candidate is accepted."""
+    import numpy as np
+    import zinfer_amd.ops as ops
+    from zinfer_amd.sampling import SamplingParams, Xoshiro256pp, adjust_logits, count_history, \
+        sample_token, top_k_candidates
+
+    class FixedU:
+        def __init__(self, u):
+            self.u = u
+
+        def float64(self):
+            return self.u
+    rs = np.random.RandomState(5)
+    cases = []
+    for trial in range(40):
+        sp = SamplingParams(temperature=float(rs.choice([0.6, 0.8, 1.0, 1.7])),
+                            top_k=int(rs.choice([1, 2, 20, 50, 1024])) if V > 7 else int(rs.choice([1, 3, 7])),
+                            top_p=float(rs.choice([1.0, 0.95, 0.8, 0.3])),
+                            min_p=float(rs.choice([0.0, 0.05, 0.5])),
+                            repetition_penalty=float(rs.choice([1.0, 1.1, 2.0])),
+                            presence_penalty=float(rs.choice([0.0, 0.7])),
+                            frequency_penalty=float(rs.choice([0.0, 0.2])))
+        logits = (rs.randn(V) * 2.5).astype(np.float32)
+        if trial % 5 == 0:
+            logits[rs.randint(0, V, 4)] = logits.max() + 1.0      # exact ties at the top
+        history = rs.randint(0, V, size=rs.randint(0, 60)).tolist()
+        cases.append((sp, logits, history, float(rs.rand())))
+    n = len(cases)
+    lg = torch.from_numpy(np.stack([c[1] for c in cases])).to(DEV)
+    rec = np.zeros((n,), dtype=ops.SAMPLE_ROW_DTYPE)
+    rows, toks, cnts = [], [], []
+    params = np.zeros((n, 3), np.float32)
+    for i, (sp, logits, history, u) in enumerate(cases):
+        rec[i] = (sp.temperature, sp.top_p, sp.min_p, sp.top_k, u)
+        counts = count_history(history, V)
+        rows += [i] * len(counts); toks += list(counts.keys()); cnts += list(counts.values())
+        params[i] = (sp.repetition_penalty, sp.presence_penalty, sp.frequency_penalty)
+    t = lambda a: torch.from_numpy(np.asarray(a, np.int32)).to(DEV)
+    if rows:
+        ops.apply_penalties(lg, t(rows), t(toks), t(cnts), torch.from_numpy(params).to(DEV))
+    for i, (sp, logits, history, u) in enumerate(cases):      # the penalties alone
+        adj = adjust_logits(logits, count_history(history, V), sp)
+        assert np.allclose(lg[i].cpu().numpy(), adj, rtol=1e-6, atol=1e-6)
+    out = torch.empty((n,), dtype=torch.int32, device=DEV)
+    ops.sample_topk(lg, torch.from_numpy(rec.view(np.uint8).reshape(-1).copy()).to(DEV), out)
+    got = out.cpu().tolist()
+    exact = 0
+    for i, (sp, logits, history, u) in enumerate(cases):
+        want = sample_token(logits, history, sp, FixedU(u))
+        if got[i] == want:
+            exact += 1
+            continue
+        adj = adjust_logits(logits, count_history(history, V), sp)
+        ids, _ = top_k_candidates(adj, min(sp.top_k, V))
+        pos = {int(t): j for j, t in enumerate(ids)}
+        assert got[i] in pos and abs(pos[got[i]] - pos[want]) == 1, \
+            f"case {i}: device {got[i]}, host {want}"
+    assert exact >= n - 2

@@ -193,6 +193,19 @@ def test_greedy_generation_through_the_entry_point(dtype, tmp_path):
     alone = llm.generate([prompts[2]], sp)[0]
     again = llm.generate([prompts[2]], sp)[0]
     assert alone == again and len(alone) == 10
+    # the device sampler (top_k 50) and the host sampler (whole vocabulary: top_k 0 with the
+    # same cut made by top_k) see the same stream: with penalties and top-p as well
+    sp2 = SamplingParams(temperature=0.7, top_k=20, top_p=0.8, repetition_penalty=1.1, seed=11,
+                         max_new_tokens=8, ignore_eos=True)
+    batch = llm.generate([prompts[1], prompts[3]], sp2)
+    assert [len(b) for b in batch] == [8, 8]
+    if dtype == "float32":
+        from zinfer_amd.sampling import Xoshiro256pp, sample_token
+        toks, rng = list(prompts[1]), Xoshiro256pp(11)      # request index 0: seed ^ 0
+        for g in batch[0]:
+            logits = plain.model_forward_batched(cfg, w, toks)[-1].float().numpy()
+            assert g == sample_token(logits, toks, sp2, rng)
+            toks.append(g)
 
 
 # ----------------------------------------------------------------------------- toy parts

@@ -158,6 +158,25 @@ class Engine:
         ops.argmax(logits, out)
         return out.tolist()
 
+    def sample(self, logits: torch.Tensor, records, penalties=None) -> List[int]:
+        """Draws one token per row on the device.  ``records`` is a numpy array of
+        ``ops.SAMPLE_ROW_DTYPE`` (temperature, top_p, min_p, top_k in 1..1024, u);
+        ``penalties`` = (rows, tokens, counts, params[n, 3]) numpy arrays or None."""
+        from .. import ops
+        n = logits.shape[0]
+        if n == 0:
+            return []
+        dev = self.device
+        if penalties is not None and len(penalties[0]):
+            rows, tokens, counts, params = penalties
+            ops.apply_penalties(logits, torch.from_numpy(rows).to(dev),
+                                torch.from_numpy(tokens).to(dev), torch.from_numpy(counts).to(dev),
+                                torch.from_numpy(params).to(dev))
+        rec = torch.from_numpy(records.view(np.uint8).reshape(-1).copy()).to(dev)
+        out = self._scratch.get("sampled", (n,), torch.int32)
+        ops.sample_topk(logits, rec, out)
+        return out.tolist()
+
     # ------------------------------------------------------------------ metadata
     def _build_context(self, entries: Sequence[StepEntry], bucket_pages: bool = False) -> StepContext:
         ps = self.page_size

@@ -39,6 +39,7 @@ class Request:
     finished: bool = False
     finish_reason: Optional[str] = None
     preemptions: int = 0
+    counts: Optional[Dict[int, int]] = None    # occurrences of each token so far (penalties)
 
     @property
     def tokens(self) -> List[int]:
@@ -212,16 +213,56 @@ class Scheduler:
         self.finished[req.id] = req
 
     def _sample(self, logits: torch.Tensor, sampling: List[PlannedEntry]) -> List[int]:
+        """Greedy rows without penalties: the device arg-max.  Rows whose top_k is 1..1024:
+        the device sampler (penalties applied on the device too), with the uniform number
+        taken from the request's own stream.  Anything else (the whole vocabulary as
+        candidates): the host sampler on a copy of the row."""
         if not sampling:
             return []
-        if all(p.request.params.greedy and not p.request.params.has_penalties for p in sampling):
+        params = [p.request.params for p in sampling]
+        if all(sp.greedy and not sp.has_penalties for sp in params):
             return self.engine.argmax(logits)
+        if hasattr(self.engine, "sample") and all(
+                sp.greedy or 1 <= sp.top_k <= 1024 for sp in params):
+            return self._sample_on_device(logits, sampling)
         rows = logits.detach().to("cpu", torch.float32).numpy()
         out = []
         for i, p in enumerate(sampling):
             req = p.request
             out.append(sample_token(rows[i], req.tokens, req.params, req.rng))
         return out
+
+    def _sample_on_device(self, logits: torch.Tensor, sampling: List[PlannedEntry]) -> List[int]:
+        from ..ops import SAMPLE_ROW_DTYPE
+        V = logits.shape[1]
+        rec = np.zeros((len(sampling),), dtype=SAMPLE_ROW_DTYPE)
+        pen_rows, pen_tok, pen_cnt = [], [], []
+        pen_params = np.zeros((len(sampling), 3), dtype=np.float32)
+        pen_params[:, 0] = 1.0
+        for i, p in enumerate(sampling):
+            req, sp = p.request, p.request.params
+            if sp.greedy:          # the arg-max is the draw among the single best candidate
+                rec[i] = (1.0, 1.0, 0.0, 1, 0.0)
+            else:
+                rec[i] = (sp.temperature, sp.top_p, sp.min_p, sp.top_k, req.rng.float64())
+            if sp.has_penalties:
+                if req.counts is None:
+                    req.counts = {}
+                    req._counted = 0
+                toks = req.tokens
+                for t in toks[req._counted:]:
+                    if t < V:
+                        req.counts[t] = req.counts.get(t, 0) + 1
+                req._counted = len(toks)
+                pen_rows.extend([i] * len(req.counts))
+                pen_tok.extend(req.counts.keys())
+                pen_cnt.extend(req.counts.values())
+                pen_params[i] = (sp.repetition_penalty, sp.presence_penalty, sp.frequency_penalty)
+        pen = None
+        if pen_rows:
+            pen = (np.asarray(pen_rows, np.int32), np.asarray(pen_tok, np.int32),
+                   np.asarray(pen_cnt, np.int32), pen_params)
+        return self.engine.sample(logits, rec, pen)
 
     def run(self) -> Dict[object, Request]:
         """Steps until every request has finished."""

@@ -290,3 +290,39 @@ def paged_attention(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index,
         _ptr(ctx_len), _ptr(seq_index), _ptr(out), ctypes.c_float(scale), int(window), T,
         n_heads, n_kv_heads, head_dim, page_size, max_pages, _stream()),
         "paged_attention")
+
+
+# ------------------------------------------------------------------------- sampling
+SAMPLE_MAX_TOP_K = 1024
+SAMPLE_ROW_DTYPE = [("temperature", "<f4"), ("top_p", "<f4"), ("min_p", "<f4"), ("top_k", "<i4"),
+                    ("u", "<f8")]
+
+
+def apply_penalties(logits, rows, tokens, counts, params) -> None:
+    """In place, for every triple (rows[i], tokens[i], counts[i]): the repetition, presence
+    and frequency penalties of ``params[row] = (repetition, presence, frequency)``."""
+    _need_gpu(logits, rows, tokens, counts, params)
+    for t, name in ((rows, "rows"), (tokens, "tokens"), (counts, "counts")):
+        _i32(t, name)
+    n, V = rows.shape[0], logits.shape[1]
+    if logits.dtype != torch.float32 or params.dtype != torch.float32 \
+            or params.shape != (logits.shape[0], 3) or tokens.shape[0] != n or counts.shape[0] != n:
+        raise KernelUnavailable("apply_penalties: float32 logits [n, V], params [n, 3], int32 triples")
+    lib = build.load("sampling")
+    _check(lib.zf_apply_penalties(_ptr(logits), _ptr(rows), _ptr(tokens), _ptr(counts),
+                                  _ptr(params), n, V, _stream()), "apply_penalties")
+
+
+def sample_topk(logits: torch.Tensor, params: torch.Tensor, out: torch.Tensor) -> None:
+    """out[r] = a token of row r drawn as the reference's sampler draws it: the top_k
+    (1..1024) largest logits, temperature, min-p, top-p, and the uniform number u of the
+    row.  ``params`` is a uint8 tensor holding one SAMPLE_ROW_DTYPE record per row."""
+    _need_gpu(logits, params, out)
+    _i32(out, "out")
+    n, V = logits.shape
+    if logits.dtype != torch.float32 or params.dtype != torch.uint8 \
+            or params.numel() != n * 24 or out.shape != (n,):
+        raise KernelUnavailable("sample_topk: float32 logits [n, V], 24-byte records, int32 out [n]")
+    lib = build.load("sampling")
+    _check(lib.zf_sample_topk(_ptr(logits), _ptr(params), _ptr(out), n, V, _stream()),
+           "sample_topk")
