@@ -21,7 +21,11 @@ def rmsnorm(x, gain, eps, out):
     out.copy_((x64 * inv * gain.to(F64)).to(out.dtype))
 
 
-def gemm(a, w, out, accumulate=False):
+def can_pretile(w):
+    return False
+
+
+def gemm(a, w, out, accumulate=False, w_tiled=False):
     r = a.to(F64) @ w.to(F64).T
     if accumulate:
         r = r + out.to(F64)
@@ -110,7 +114,7 @@ def argmax(logits, out):
     out.copy_(torch.argmax(logits, dim=-1).to(torch.int32))
 
 
-ALL = ("embed", "rmsnorm", "gemm", "qk_norm_rope_kv_write", "paged_attention", "swiglu",
+ALL = ("embed", "rmsnorm", "gemm", "can_pretile", "qk_norm_rope_kv_write", "paged_attention", "swiglu",
        "gather_rows", "argmax")
 
 

@@ -110,6 +110,26 @@ def test_gemm_bf16_mfma_paths(M, N, K, o_dtype, accumulate):
     assert rel_err(got, want) <= (tol(o_dtype) if not accumulate else 2e-5)
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 48, 64, 65, 200, 300])
+@pytest.mark.parametrize("N,K", [(64, 64), (4160, 1088), (192, 4096), (1024, 320)])
+@pytest.mark.parametrize("o_dtype,accumulate", [(torch.bfloat16, False), (torch.float32, True)])
+def test_gemm_pretiled_weights(M, N, K, o_dtype, accumulate):
+    """The kernels' own weight layout (made once at load) gives the same product."""
+    a = _rand((M, K), torch.bfloat16, 30)
+    w = _rand((N, K), torch.bfloat16, 31, 0.05)
+    base = _rand((M, N), torch.float32, 32).to(o_dtype)
+    want = base.clone()
+    ref.gemm(a, w, want, accumulate)
+    wt = _ops().pretile_weight(w.to(DEV))
+    assert wt.shape == w.shape and not torch.equal(wt.cpu(), w)
+    got = base.clone().to(DEV)
+    _ops().gemm(a.to(DEV), wt, got, accumulate, w_tiled=True)
+    assert rel_err(got, want) <= (tol(o_dtype) if not accumulate else 2e-5)
+    plain_out = base.clone().to(DEV)
+    _ops().gemm(a.to(DEV), w.to(DEV), plain_out, accumulate)
+    assert rel_err(got, plain_out) <= (tol(o_dtype) if not accumulate else 2e-5)
+
+
 @pytest.mark.parametrize("a_dtype", DTYPES)
 def test_gemm_accumulate_and_one_hot(a_dtype):
     """out += a w^T in 32-bit; a one-hot row picks a column of W (the reference's

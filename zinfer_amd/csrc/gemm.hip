@@ -122,7 +122,18 @@ typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 #define TK 64
 #define LDS_ROW 72
 
-template <int BM, int BN, int WM, int WN, int EPI>
+// Pre-tiled weights (WT): W is stored as [N / 16][K / 64][2][64][8]: the 16 rows x 64 k of a
+// tile lie together (2 KB) in the order in which the lanes of a 16x16x32 MFMA pair consume
+// them (chunk c of lane l = 16 g + r holds row r, k = 16 g + 8 c .. + 8), so that one wave
+// load of the weight-streaming kernel is 1 KB of consecutive memory.  This kernel reads the
+// same layout 16 bytes at a time.
+__device__ __forceinline__ size_t tiled_offset(int n, int k, int K) {
+  const int kk = k % 64;
+  return ((size_t)(n / 16) * (K / 64) + k / 64) * 1024 + ((kk % 16) / 8) * 512 +
+         ((kk / 16) * 16 + n % 16) * 8 + kk % 8;
+}
+
+template <int BM, int BN, int WM, int WN, int EPI, bool WT>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
     int N, int K, int tiles_m, int tiles_n) {
@@ -187,7 +198,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_ker
       const int row = chunk / 8, kc = (chunk % 8) * 8;
       const int n = min(n0 + row, N - 1);
       if (k0 + kc < K)
-        breg[c] = *(const u32x4_t*)(W + (size_t)n * K + k0 + kc);
+        breg[c] = *(const u32x4_t*)(W + (WT ? tiled_offset(n, k0 + kc, K)
+                                            : (size_t)n * K + k0 + kc));
       else
         breg[c] = u32x4_t{0, 0, 0, 0};
     }
@@ -260,7 +272,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_ker
     }
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, bool WT>
 static int launch_tile(const void* A, const void* W, void* C, int M, int N, int K, int epi,
                        hipStream_t stream) {
   constexpr int NT = (BM / WM) * (BN / WN) * 64;
@@ -269,7 +281,7 @@ static int launch_tile(const void* A, const void* W, void* C, int M, int N, int 
   const size_t smem = (size_t)2 * (BM + BN) * LDS_ROW * sizeof(bf16_t);
 #define ZF_TILE_LAUNCH(E)                                                                      \
   do {                                                                                         \
-    auto kern = gemm_bf16_tile_kernel<BM, BN, WM, WN, E>;                                      \
+    auto kern = gemm_bf16_tile_kernel<BM, BN, WM, WN, E, WT>;                                  \
     if (smem > 64 * 1024) {                                                                    \
       hipError_t e = hipFuncSetAttribute((const void*)kern,                                    \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
@@ -287,16 +299,25 @@ static int launch_tile(const void* A, const void* W, void* C, int M, int N, int 
 
 // variant: 0 = 128x128 (waves 64x64), 1 = 256x128 (waves 128x64), 2 = 256x256 (waves 128x128),
 //          3 = 128x128 (waves 64x32, 8 waves), 4 = 256x256 (waves 128x64, 8 waves)
+//          w_tiled: W is in the pre-tiled layout (needs N % 16 == 0 and K % 64 == 0)
 extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, int N, int K,
-                                 int epi, int variant, hipStream_t stream) {
+                                 int epi, int variant, int w_tiled, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K % 8 != 0) return -3;
+  if (w_tiled) {
+    if (N % 16 != 0 || K % 64 != 0) return -3;
+    switch (variant) {
+      case 0: return launch_tile<128, 128, 64, 64, true>(A, W, C, M, N, K, epi, stream);
+      case 4: return launch_tile<256, 256, 128, 64, true>(A, W, C, M, N, K, epi, stream);
+      default: return -4;
+    }
+  }
   switch (variant) {
-    case 0: return launch_tile<128, 128, 64, 64>(A, W, C, M, N, K, epi, stream);
-    case 1: return launch_tile<256, 128, 128, 64>(A, W, C, M, N, K, epi, stream);
-    case 2: return launch_tile<256, 256, 128, 128>(A, W, C, M, N, K, epi, stream);
-    case 3: return launch_tile<128, 128, 64, 32>(A, W, C, M, N, K, epi, stream);
-    case 4: return launch_tile<256, 256, 128, 64>(A, W, C, M, N, K, epi, stream);
+    case 0: return launch_tile<128, 128, 64, 64, false>(A, W, C, M, N, K, epi, stream);
+    case 1: return launch_tile<256, 128, 128, 64, false>(A, W, C, M, N, K, epi, stream);
+    case 2: return launch_tile<256, 256, 128, 128, false>(A, W, C, M, N, K, epi, stream);
+    case 3: return launch_tile<128, 128, 64, 32, false>(A, W, C, M, N, K, epi, stream);
+    case 4: return launch_tile<256, 256, 128, 64, false>(A, W, C, M, N, K, epi, stream);
     default: return -4;
   }
 }
@@ -311,7 +332,7 @@ extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, i
 // workgroups write float32 partials to a workspace [KSPLIT, M, N] that
 // skinny_reduce_kernel adds in split order.  Nothing depends on timing.  No LDS staging of W:
 // nothing of it is reused.
-template <int MT, int RG, int EPI>
+template <int MT, int RG, int EPI, bool WT>
 __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
     int N, int K) {
@@ -319,9 +340,13 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int n0 = blockIdx.x * (16 * RG);
   const int g = lane / 16;
+  // plain layout: row pointer, k added later; pre-tiled: the lane's 16 bytes of chunk 0 of
+  // the row group's first tile, tiles of 64 k are 1024 elements apart, chunk 1 is 512 on
   const bf16_t* wrow[RG];
 #pragma unroll
-  for (int r = 0; r < RG; ++r) wrow[r] = W + (size_t)min(n0 + r * 16 + lane % 16, N - 1) * K;
+  for (int r = 0; r < RG; ++r)
+    wrow[r] = WT ? W + (size_t)(n0 / 16 + r) * (K / 64) * 1024 + lane * 8
+                 : W + (size_t)min(n0 + r * 16 + lane % 16, N - 1) * K;
   const bf16_t* arow[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) arow[t] = A + (size_t)min(t * 16 + lane % 16, M - 1) * K;
@@ -340,8 +365,14 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
     u32x4_t w0[RG], w1[RG];
 #pragma unroll
     for (int r = 0; r < RG; ++r) {
-      w0[r] = (k < K) ? __builtin_nontemporal_load((const u32x4_t*)(wrow[r] + k)) : zero;
-      w1[r] = (k + 8 < K) ? __builtin_nontemporal_load((const u32x4_t*)(wrow[r] + k + 8)) : zero;
+      if (WT) {       // N % 16 == 0 and K % 64 == 0: nothing to clamp, nothing to zero-fill
+        const bf16_t* tile = wrow[r] + (size_t)(k0 / 64) * 1024;
+        w0[r] = __builtin_nontemporal_load((const u32x4_t*)tile);
+        w1[r] = __builtin_nontemporal_load((const u32x4_t*)(tile + 512));
+      } else {
+        w0[r] = (k < K) ? __builtin_nontemporal_load((const u32x4_t*)(wrow[r] + k)) : zero;
+        w1[r] = (k + 8 < K) ? __builtin_nontemporal_load((const u32x4_t*)(wrow[r] + k + 8)) : zero;
+      }
     }
     u32x4_t a0[MT], a1[MT];
 #pragma unroll
@@ -413,19 +444,19 @@ __global__ void skinny_reduce_kernel(const float* __restrict__ ws, void* __restr
     ((float*)Cv)[i] += s;
 }
 
-template <int MT, int RG>
+template <int MT, int RG, bool WT>
 static int launch_skinny(const void* A, const void* W, void* C, void* ws, int M, int N, int K,
                          int epi, int ksplit, hipStream_t stream) {
   const dim3 grid((N + 16 * RG - 1) / (16 * RG), ksplit), block(512);
   void* dst = ksplit > 1 ? ws : C;
   if (epi == EPI_STORE_BF16)
-    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_STORE_BF16>), grid, block, 0, stream,
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_STORE_BF16, WT>), grid, block, 0, stream,
                        (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K);
   else if (epi == EPI_STORE_F32)
-    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_STORE_F32>), grid, block, 0, stream,
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_STORE_F32, WT>), grid, block, 0, stream,
                        (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K);
   else
-    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_ACC_F32>), grid, block, 0, stream,
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_ACC_F32, WT>), grid, block, 0, stream,
                        (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K);
   if (ksplit > 1) {
     const size_t mn = (size_t)M * N;
@@ -444,14 +475,19 @@ static int launch_skinny(const void* A, const void* W, void* C, void* ws, int M,
 }
 
 // rg: row groups of 16 per workgroup (1, 2 or 4); ksplit: workgroups along K (1..16), which
-// needs a float32 workspace of ksplit * M * N elements when > 1.
+// needs a float32 workspace of ksplit * M * N elements when > 1; w_tiled: W is pre-tiled
+// (N % 16 == 0, K % 64 == 0, N a multiple of 16 * rg).
 extern "C" int zf_gemm_bf16_skinny(const void* A, const void* W, void* C, void* ws, int M, int N,
-                                   int K, int epi, int rg, int ksplit, hipStream_t stream) {
+                                   int K, int epi, int rg, int ksplit, int w_tiled,
+                                   hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K % 8 != 0 || M > 64 || ksplit < 1 || ksplit > 16 || (ksplit > 1 && ws == nullptr))
     return -3;
+  if (w_tiled && (N % (16 * rg) != 0 || K % 64 != 0)) return -3;
   const int mt = (M + 15) / 16;
-#define ZF_SK(MT, RG) return launch_skinny<MT, RG>(A, W, C, ws, M, N, K, epi, ksplit, stream)
+#define ZF_SK(MT, RG)                                                                         \
+  return w_tiled ? launch_skinny<MT, RG, true>(A, W, C, ws, M, N, K, epi, ksplit, stream)     \
+                 : launch_skinny<MT, RG, false>(A, W, C, ws, M, N, K, epi, ksplit, stream)
   if (rg == 1) { if (mt == 1) ZF_SK(1, 1); if (mt == 2) ZF_SK(2, 1); if (mt == 3) ZF_SK(3, 1); ZF_SK(4, 1); }
   if (rg == 2) { if (mt == 1) ZF_SK(1, 2); if (mt == 2) ZF_SK(2, 2); if (mt == 3) ZF_SK(3, 2); ZF_SK(4, 2); }
   if (rg == 4) { if (mt == 1) ZF_SK(1, 4); if (mt == 2) ZF_SK(2, 4); if (mt == 3) ZF_SK(3, 4); ZF_SK(4, 4); }

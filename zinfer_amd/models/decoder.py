@@ -58,7 +58,7 @@ class DecoderModel:
         if s.head_name in tensors:
             self.head = Linear(place_matrix(tensors[s.head_name], self.ctx))
         else:  # tied: the embedding stands in for the head
-            self.head = Linear(self.embedding)
+            self.head = Linear(self.embedding, pretile=False)
 
     # ---------------------------------------------------------------- cache needs
     def cache_needs(self) -> List[Optional[object]]:

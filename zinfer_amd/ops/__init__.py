@@ -174,10 +174,18 @@ _EPI_STORE_BF16, _EPI_STORE_F32, _EPI_ACC_F32 = 0, 1, 2
 SKINNY_MAX_M = 64
 
 
-def _skinny_plan(M: int, N: int):
+def _skinny_plan(M: int, N: int, K: int, tiled: bool):
     """Row groups of 16 per workgroup and workgroups along K for the weight-streaming kernel:
     enough workgroups to fill 256 CUs, as many rows per workgroup as that allows (the tokens
-    are re-read once per workgroup)."""
+    are re-read once per workgroup).  Measured on MI355X at the Qwen3-8B sizes."""
+    if tiled:
+        if M <= 16:
+            return (2 if N >= 6144 else 1), 1
+        if N >= 16384:
+            return 4, 1
+        if N >= 6144:
+            return 2, 1
+        return (4, 4) if K >= 8192 else (2, 2)
     if M <= 16:
         rg = 4 if N // 64 >= 256 else 1
         ks = 2 if (rg == 4 and N // 64 < 1024) else 1
@@ -194,8 +202,28 @@ def _tile_variant(M: int, N: int) -> int:
     return 4 if tiles >= 160 else 0
 
 
-def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
-    """out = a w^T (w is [N, K]); with ``accumulate`` out += a w^T, in 32-bit.
+def can_pretile(w: torch.Tensor) -> bool:
+    return w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[0] % 64 == 0 \
+        and w.shape[1] % 64 == 0
+
+
+def pretile_weight(w: torch.Tensor) -> torch.Tensor:
+    """The bfloat16 kernels' own weight layout, made once at load: [N / 16][K / 64][2][64][8],
+    the 16 rows x 64 k of a tile together (2 KB) in the order the lanes of the 16x16x32 MFMA
+    pair consume them, so that the weight-streaming kernel reads 1 KB of consecutive memory
+    per wave load.  Returned with shape [N, K]; only the kernels know what lies where."""
+    N, K = w.shape
+    if not can_pretile(w):
+        raise KernelUnavailable(f"pretile_weight: bfloat16 [N % 64 == 0, K % 64 == 0], got "
+                                f"{tuple(w.shape)} {w.dtype}")
+    t = w.view(N // 16, 16, K // 64, 4, 2, 8).permute(0, 2, 4, 3, 1, 5).contiguous()
+    return t.view(N, K)
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
+         w_tiled: bool = False) -> None:
+    """out = a w^T (w is [N, K]); with ``accumulate`` out += a w^T, in 32-bit.  ``w_tiled``:
+    ``w`` went through ``pretile_weight``.
 
     bfloat16 operands with K a multiple of 8 go to the MFMA kernels (weight streaming for up
     to 64 rows of ``a``, LDS-tiled above); everything else, the whole 32-bit path included,
@@ -209,17 +237,21 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     if accumulate and out.dtype != torch.float32:
         raise KernelUnavailable("gemm: accumulation needs a float32 output")
     lib = build.load("gemm")
+    if w_tiled and not (a.dtype == torch.bfloat16 and can_pretile(w)):
+        raise KernelUnavailable("gemm: a pre-tiled weight needs bfloat16 operands")
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and K % 8 == 0 and M > 0:
         epi = _EPI_ACC_F32 if accumulate else \
             (_EPI_STORE_BF16 if out.dtype == torch.bfloat16 else _EPI_STORE_F32)
         if M <= SKINNY_MAX_M:
-            rg, ks = _skinny_plan(M, N)
+            rg, ks = _skinny_plan(M, N, K, w_tiled)
             ws = _workspace("gemm_splitk", ks * M * N, torch.float32, a.device) if ks > 1 else None
             _check(lib.zf_gemm_bf16_skinny(_ptr(a), _ptr(w), _ptr(out), _ptr(ws), M, N, K, epi,
-                                           rg, ks, _stream()), "gemm (weight streaming)")
+                                           rg, ks, 1 if w_tiled else 0, _stream()),
+                   "gemm (weight streaming)")
         else:
             _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, epi,
-                                         _tile_variant(M, N), _stream()), "gemm (tiled)")
+                                         _tile_variant(M, N), 1 if w_tiled else 0, _stream()),
+                   "gemm (tiled)")
         return
     _check(lib.zf_gemm_fma(_ptr(a), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), M, N, K,
                            1 if accumulate else 0, _stream()), "gemm")

@@ -8,14 +8,19 @@ from .. import ops
 
 
 class Linear:
-    def __init__(self, weight: torch.Tensor):
+    """``pretile``: a bfloat16 matrix on the GPU whose sizes allow it is re-laid once into the
+    MFMA kernels' own order (the plain copy is dropped); pass False for a matrix that is also
+    read by rows (a tied embedding)."""
+
+    def __init__(self, weight: torch.Tensor, pretile: bool = True):
         assert weight.dim() == 2
-        self.weight = weight.contiguous()
         self.out_features, self.in_features = weight.shape
+        self.tiled = bool(pretile and weight.is_cuda and ops.can_pretile(weight))
+        self.weight = ops.pretile_weight(weight) if self.tiled else weight.contiguous()
 
     def forward(self, x: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
         """out = x W^T, or out += x W^T (``out`` float32) when ``accumulate``."""
-        ops.gemm(x, self.weight, out, accumulate)
+        ops.gemm(x, self.weight, out, accumulate, w_tiled=self.tiled)
         return out
 
 
