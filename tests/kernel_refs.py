@@ -25,6 +25,19 @@ def can_pretile(w):
     return False
 
 
+def can_fuse_swiglu(w):
+    return False
+
+
+def gemm_swiglu(a, w, out, w_tiled=False):
+    """``w`` rows alternate in groups of 16 between gate and up."""
+    N, K = w.shape
+    wv = w.to(F64).view(N // 32, 2, 16, K)
+    g = a.to(F64) @ wv[:, 0].reshape(N // 2, K).T
+    u = a.to(F64) @ wv[:, 1].reshape(N // 2, K).T
+    out.copy_((g / (1.0 + torch.exp(-g)) * u).to(out.dtype))
+
+
 def gemm(a, w, out, accumulate=False, w_tiled=False):
     r = a.to(F64) @ w.to(F64).T
     if accumulate:
@@ -114,7 +127,7 @@ def argmax(logits, out):
     out.copy_(torch.argmax(logits, dim=-1).to(torch.int32))
 
 
-ALL = ("embed", "rmsnorm", "gemm", "can_pretile", "qk_norm_rope_kv_write", "paged_attention", "swiglu",
+ALL = ("embed", "rmsnorm", "gemm", "can_pretile", "can_fuse_swiglu", "gemm_swiglu", "qk_norm_rope_kv_write", "paged_attention", "swiglu",
        "gather_rows", "argmax")
 
 

@@ -130,6 +130,28 @@ def test_gemm_pretiled_weights(M, N, K, o_dtype, accumulate):
     assert rel_err(got, plain_out) <= (tol(o_dtype) if not accumulate else 2e-5)
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64, 65, 200, 300])
+@pytest.mark.parametrize("I,K,tiled", [(32, 64, True), (12288 // 8, 320, True), (96, 136, False),
+                                       (352, 4096, True), (8192, 192, True)])
+def test_gemm_swiglu(M, I, K, tiled):
+    """silu(a Wg^T) * (a Wu^T) in the product's epilogue, against the plain reference, with
+    gate and up rows interleaved in groups of 16 (and the result of the separate kernels)."""
+    ops = _ops()
+    a = _rand((M, K), torch.bfloat16, 40)
+    g = _rand((I, K), torch.bfloat16, 41, 0.08)
+    u = _rand((I, K), torch.bfloat16, 42, 0.08)
+    w = ops.interleave_gate_up(g.to(DEV), u.to(DEV))
+    want = torch.empty((M, I), dtype=torch.bfloat16)
+    ref.gemm_swiglu(a, w.cpu(), want)
+    plain_gu = a.double() @ torch.cat([g, u]).double().T
+    assert rel_err(want, (torch.nn.functional.silu(plain_gu[:, :I]) * plain_gu[:, I:])) <= tol(torch.bfloat16)
+    if tiled:
+        w = ops.pretile_weight(w)
+    got = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_swiglu(a.to(DEV), w, got, w_tiled=tiled)
+    assert rel_err(got, want) <= tol(torch.bfloat16)
+
+
 @pytest.mark.parametrize("a_dtype", DTYPES)
 def test_gemm_accumulate_and_one_hot(a_dtype):
     """out += a w^T in 32-bit; a one-hot row picks a column of W (the reference's

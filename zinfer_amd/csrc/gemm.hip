@@ -113,6 +113,12 @@ typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 #define EPI_STORE_BF16 0
 #define EPI_STORE_F32 1
 #define EPI_ACC_F32 2
+// SwiGLU fused into the product: the rows of W alternate in groups of 16 between the gate
+// and the up projection (gate 0..15, up 0..15, gate 16..31, ...); the output is
+// silu(gate) * up as bfloat16 [M, N / 2]  (a_j = g_j / (1 + exp(-g_j)) * u_j, cpu.zig:130-147)
+#define EPI_SWIGLU 3
+
+__device__ __forceinline__ float swiglu_f(float g, float u) { return g / (1.0f + expf(-g)) * u; }
 
 // ---------------------------------------------------------------- large M: LDS-tiled
 // Block tile BM x BN x 64, waves laid out (BM/WM) x (BN/WN), each wave WM x WN through
@@ -181,6 +187,21 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_ker
 
   u32x4_t areg[A_CHUNKS], breg[B_CHUNKS];
 
+  // which 16 bytes of the W tile a thread moves: (row of the tile, k offset).  Plain layout:
+  // 8 consecutive threads take the 8 chunks of a row.  Pre-tiled: 128 consecutive threads
+  // take the 128 chunks of a 16-row group in the order they lie in memory (chunk p = 64 c +
+  // 16 g + r holds row r, k = 16 g + 8 c), so their loads are consecutive 16-byte pieces.
+  auto b_chunk = [&](int chunk, int& row, int& kc) {
+    if (WT) {
+      const int p = chunk % 128;
+      row = (chunk / 128) * 16 + p % 16;
+      kc = ((p % 64) / 16) * 16 + (p / 64) * 8;
+    } else {
+      row = chunk / 8;
+      kc = (chunk % 8) * 8;
+    }
+  };
+
   auto gload = [&](int k0) {
 #pragma unroll
     for (int c = 0; c < A_CHUNKS; ++c) {
@@ -194,8 +215,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_ker
     }
 #pragma unroll
     for (int c = 0; c < B_CHUNKS; ++c) {
-      const int chunk = tid + c * NT;
-      const int row = chunk / 8, kc = (chunk % 8) * 8;
+      int row, kc;
+      b_chunk(tid + c * NT, row, kc);
       const int n = min(n0 + row, N - 1);
       if (k0 + kc < K)
         breg[c] = *(const u32x4_t*)(W + (WT ? tiled_offset(n, k0 + kc, K)
@@ -215,8 +236,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_ker
     }
 #pragma unroll
     for (int c = 0; c < B_CHUNKS; ++c) {
-      const int chunk = tid + c * NT;
-      const int row = chunk / 8, kc = (chunk % 8) * 8;
+      int row, kc;
+      b_chunk(tid + c * NT, row, kc);
       *(u32x4_t*)(b_s + row * LDS_ROW + kc) = breg[c];
     }
   };
@@ -259,6 +280,14 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_ker
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
+        if (EPI == EPI_SWIGLU) {
+          // columns 0..15 of the 32-wide block are gate, 16..31 the matching up columns
+          const float other = __shfl_xor(acc[i][j][r], 16, 64);
+          if (lane % 32 < 16 && m < M && n < N)
+            ((bf16_t*)Cv)[(size_t)m * (N / 2) + (n / 32) * 16 + n % 16] =
+                float_to_bf16(swiglu_f(acc[i][j][r], other));
+          continue;
+        }
         if (m < M && n < N) {
           const size_t off = (size_t)m * N + n;
           if (EPI == EPI_STORE_BF16)
@@ -292,6 +321,7 @@ static int launch_tile(const void* A, const void* W, void* C, int M, int N, int 
   } while (0)
   if (epi == EPI_STORE_BF16) ZF_TILE_LAUNCH(EPI_STORE_BF16);
   else if (epi == EPI_STORE_F32) ZF_TILE_LAUNCH(EPI_STORE_F32);
+  else if (epi == EPI_SWIGLU) ZF_TILE_LAUNCH(EPI_SWIGLU);
   else ZF_TILE_LAUNCH(EPI_ACC_F32);
 #undef ZF_TILE_LAUNCH
   return (int)hipGetLastError();
@@ -303,7 +333,7 @@ static int launch_tile(const void* A, const void* W, void* C, int M, int N, int 
 extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, int N, int K,
                                  int epi, int variant, int w_tiled, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K % 8 != 0) return -3;
+  if (K % 8 != 0 || (epi == EPI_SWIGLU && N % 32 != 0)) return -3;
   if (w_tiled) {
     if (N % 16 != 0 || K % 64 != 0) return -3;
     switch (variant) {
@@ -359,7 +389,6 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
 
   const u32x4_t zero = u32x4_t{0, 0, 0, 0};
   const int kstride = 512 * gridDim.y;
-#pragma unroll 2
   for (int k0 = (blockIdx.y * 8 + wave) * 64; k0 < K; k0 += kstride) {
     const int k = k0 + g * 16;
     u32x4_t w0[RG], w1[RG];
@@ -397,6 +426,31 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
 #pragma unroll
       for (int e = 0; e < 4; ++e) part[wave][r * MT + t][lane][e] = acc[r][t][e];
   __syncthreads();
+  if (EPI == EPI_SWIGLU) {
+    // row groups alternate gate / up: the pair (2 p, 2 p + 1) gives 16 outputs per token
+    for (int item = tid; item < (RG / 2) * MT * 64; item += 512) {
+      const int pt = item / 64, l = item % 64;
+      const int p = pt / MT, t = pt % MT;
+      float g[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < 8; ++w)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          g[e] += part[w][(2 * p) * MT + t][l][e];
+          u[e] += part[w][(2 * p + 1) * MT + t][l][e];
+        }
+      const int token = t * 16 + l % 16;
+      if (token < M) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int n = n0 / 2 + p * 16 + 4 * (l / 16) + e;      // column of the [M, N / 2] output
+          if (2 * n < N)
+            ((bf16_t*)Cv)[(size_t)token * (N / 2) + n] = float_to_bf16(swiglu_f(g[e], u[e]));
+        }
+      }
+    }
+    return;
+  }
   for (int item = tid; item < RG * MT * 64; item += 512) {
     const int rt = item / 64, l = item % 64;
     const int r = rt / MT, t = rt % MT;
@@ -449,6 +503,12 @@ static int launch_skinny(const void* A, const void* W, void* C, void* ws, int M,
                          int epi, int ksplit, hipStream_t stream) {
   const dim3 grid((N + 16 * RG - 1) / (16 * RG), ksplit), block(512);
   void* dst = ksplit > 1 ? ws : C;
+  if (epi == EPI_SWIGLU) {
+    if (RG < 2 || ksplit != 1 || N % 32 != 0) return -3;
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, (RG < 2 ? 2 : RG), EPI_SWIGLU, WT>), grid, block,
+                       0, stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K);
+    return (int)hipGetLastError();
+  }
   if (epi == EPI_STORE_BF16)
     hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_STORE_BF16, WT>), grid, block, 0, stream,
                        (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K);

@@ -170,7 +170,7 @@ def _workspace(name: str, numel: int, dtype: torch.dtype, device) -> torch.Tenso
 
 
 # ------------------------------------------------------------------------- matrix product
-_EPI_STORE_BF16, _EPI_STORE_F32, _EPI_ACC_F32 = 0, 1, 2
+_EPI_STORE_BF16, _EPI_STORE_F32, _EPI_ACC_F32, _EPI_SWIGLU = 0, 1, 2, 3
 SKINNY_MAX_M = 64
 
 
@@ -255,6 +255,43 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         return
     _check(lib.zf_gemm_fma(_ptr(a), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), M, N, K,
                            1 if accumulate else 0, _stream()), "gemm")
+
+
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """Rows of the gate and the up projection alternating in groups of 16 (gate 0..15, up
+    0..15, gate 16..31, ...): the order ``gemm_swiglu`` wants.  Needs I % 16 == 0."""
+    I, K = gate.shape
+    return torch.stack([gate.view(I // 16, 16, K), up.view(I // 16, 16, K)], dim=1) \
+        .reshape(2 * I, K).contiguous()
+
+
+def can_fuse_swiglu(w: torch.Tensor) -> bool:
+    return w.is_cuda and w.dtype == torch.bfloat16 and w.shape[0] % 64 == 0 and w.shape[1] % 8 == 0
+
+
+def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bool = False) -> None:
+    """out[M, I] = silu(a Wg^T) * (a Wu^T) as bfloat16, with ``w`` [2 I, K] from
+    ``interleave_gate_up`` (then possibly ``pretile_weight``): the activation is applied to
+    the 32-bit sums in the product's epilogue, nothing of width 2 I is written."""
+    _need_gpu(a, w, out)
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K or out.shape != (M, N // 2) or out.dtype != torch.bfloat16 \
+            or a.dtype != torch.bfloat16 or not can_fuse_swiglu(w):
+        raise KernelUnavailable(f"gemm_swiglu: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} "
+                                f"{w.dtype}, out {tuple(out.shape)} {out.dtype}")
+    if M == 0:
+        return
+    lib = build.load("gemm")
+    if M <= SKINNY_MAX_M:
+        rg = 4 if (M > 16 and N >= 16384) else 2
+        _check(lib.zf_gemm_bf16_skinny(_ptr(a), _ptr(w), _ptr(out), _ptr(None), M, N, K,
+                                       _EPI_SWIGLU, rg, 1, 1 if w_tiled else 0, _stream()),
+               "gemm_swiglu (weight streaming)")
+    else:
+        _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, _EPI_SWIGLU,
+                                     _tile_variant(M, N), 1 if w_tiled else 0, _stream()),
+               "gemm_swiglu (tiled)")
 
 
 # ------------------------------------------------------------------------- attention

@@ -30,18 +30,35 @@ class SwiGluMlp(FeedForward):
         g, u = tensors[p + "gate_proj.weight"], tensors[p + "up_proj.weight"]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
-        self.gate_up = Linear(place_matrix(torch.cat([g, u], dim=0), self.ctx))
+        g, u = place_matrix(g, self.ctx), place_matrix(u, self.ctx)
+        # bfloat16 on the GPU with sizes the MFMA kernels take: gate and up rows alternate in
+        # groups of 16 and the activation runs in the product's epilogue
+        self.fused = self.ctx.compute_dtype == torch.bfloat16 and g.shape[0] % 32 == 0 \
+            and ops.can_fuse_swiglu(_probe(g))
+        stacked = ops.interleave_gate_up(g, u) if self.fused else torch.cat([g, u], dim=0)
+        del g, u
+        self.gate_up = Linear(stacked)
         self.down = Linear(place_matrix(tensors[p + "down_proj.weight"], self.ctx))
 
     def forward(self, h, residual, step) -> None:
         T = h.shape[0]
         I = self.spec.intermediate_size
         act = self.ctx.act_dtype
-        gu = step.scratch("gate_up", (T, 2 * I), act)
-        self.gate_up.forward(h, gu)
         a = step.scratch("ff_act", (T, I), act)
-        ops.swiglu(gu, a)
+        if self.fused and h.dtype == torch.bfloat16:
+            ops.gemm_swiglu(h, self.gate_up.weight, a, w_tiled=self.gate_up.tiled)
+        else:
+            gu = step.scratch("gate_up", (T, 2 * I), act)
+            self.gate_up.forward(h, gu)
+            ops.swiglu(gu, a)
         self.down.forward(a, residual, accumulate=True)
+
+
+class _probe:
+    """Shape and placement of the stacked gate/up matrix, without building it."""
+
+    def __init__(self, g: torch.Tensor):
+        self.is_cuda, self.dtype, self.shape = g.is_cuda, g.dtype, (2 * g.shape[0], g.shape[1])
 
 
 register_part("feed_forward", SwiGluSpec, SwiGluMlp)
