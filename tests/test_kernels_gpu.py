@@ -152,6 +152,37 @@ def test_gemm_swiglu(M, I, K, tiled):
     assert rel_err(got, want) <= tol(torch.bfloat16)
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(6144, 4096), (4160, 1088), (64, 64), (24576, 320)])
+@pytest.mark.parametrize("kind", ["bf16", "f32", "swiglu"])
+def test_norm_gemm(M, N, K, kind):
+    """The RMSNorm folded into the weight-streaming product against norm-then-product in
+    64-bit: 32-bit sum of squares and scale, bfloat16 operands."""
+    ops = _ops()
+    x = _rand((M, K), torch.float32, 50, 2.0)
+    gain = 1 + 0.1 * _rand((K,), torch.float32, 51)
+    w = _rand((N, K), torch.bfloat16, 52, 0.05)
+    eps = 1e-5
+    normed = torch.empty((M, K), dtype=torch.float64)
+    ref.rmsnorm(x, gain, eps, normed)
+    if ops.norm_gemm_plan(M, N, K, w.to(DEV), True) is None and kind != "swiglu":
+        pytest.skip("this size uses a split over workgroups: the norm runs on its own")
+    if kind == "swiglu":
+        I = N // 2
+        wi = ops.interleave_gate_up(w[:I].to(DEV), w[I:].to(DEV))
+        want = torch.empty((M, I), dtype=torch.float64)
+        ref.gemm_swiglu(normed, wi.cpu(), want)
+        got = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.norm_gemm(x.to(DEV), gain.to(DEV), eps, ops.pretile_weight(wi), got, swiglu=True)
+    else:
+        o_dtype = torch.bfloat16 if kind == "bf16" else torch.float32
+        want = normed @ w.double().T
+        got = torch.full((M, N), float("nan"), dtype=o_dtype, device=DEV)
+        ops.norm_gemm(x.to(DEV), gain.to(DEV), eps, ops.pretile_weight(w.to(DEV)), got)
+    # the operands are rounded to bfloat16 once (2^-9 each), the sums are 32-bit
+    assert rel_err(got, want) <= 2.0 ** -7
+
+
 @pytest.mark.parametrize("a_dtype", DTYPES)
 def test_gemm_accumulate_and_one_hot(a_dtype):
     """out += a w^T in 32-bit; a one-hot row picks a column of W (the reference's

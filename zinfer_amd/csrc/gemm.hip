@@ -362,11 +362,19 @@ extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, i
 // workgroups write float32 partials to a workspace [KSPLIT, M, N] that
 // skinny_reduce_kernel adds in split order.  Nothing depends on timing.  No LDS staging of W:
 // nothing of it is reused.
-template <int MT, int RG, int EPI, bool WT>
+//
+// NORM: the tokens come as the float32 residual stream and the RMSNorm before the product is
+// folded in.  The product is linear, so  W (x * gain * inv) = inv * W (x * gain): the lanes
+// feed bfloat16(x * gain) to the MFMAs, add up x^2 on the way (the workgroup sees all of K
+// when there is no split over workgroups), and the epilogue scales each token's sums by
+// inv = 1 / sqrt(mean(x^2) + eps), all in 32-bit  (n = x w / sqrt(mean(x^2) + eps),
+// src/kernel/core/cpu.zig:38-48 of the reference).
+template <int MT, int RG, int EPI, bool WT, bool NORM>
 __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
-    int N, int K) {
+    int N, int K, const float* __restrict__ gain, float eps) {
   __shared__ float part[8][RG * MT][64][4];
+  __shared__ float ssum[8][MT][16];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int n0 = blockIdx.x * (16 * RG);
   const int g = lane / 16;
@@ -378,8 +386,15 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
     wrow[r] = WT ? W + (size_t)(n0 / 16 + r) * (K / 64) * 1024 + lane * 8
                  : W + (size_t)min(n0 + r * 16 + lane % 16, N - 1) * K;
   const bf16_t* arow[MT];
+  const float* xrow[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) arow[t] = A + (size_t)min(t * 16 + lane % 16, M - 1) * K;
+  for (int t = 0; t < MT; ++t) {
+    arow[t] = A + (size_t)min(t * 16 + lane % 16, M - 1) * K;
+    xrow[t] = (const float*)A + (size_t)min(t * 16 + lane % 16, M - 1) * K;
+  }
+  float ss[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) ss[t] = 0.f;
 
   f32x4_t acc[RG][MT];
 #pragma unroll
@@ -404,10 +419,33 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
       }
     }
     u32x4_t a0[MT], a1[MT];
+    if (NORM) {       // K % 64 == 0 here: 16 floats of x and of the gain per lane
+      float4 gv[4];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      a0[t] = (k < K) ? *(const u32x4_t*)(arow[t] + k) : zero;
-      a1[t] = (k + 8 < K) ? *(const u32x4_t*)(arow[t] + k + 8) : zero;
+      for (int c = 0; c < 4; ++c) gv[c] = *(const float4*)(gain + k + 4 * c);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        float4 xv[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) xv[c] = *(const float4*)(xrow[t] + k + 4 * c);
+        uint32_t pk[8];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          ss[t] += xv[c].x * xv[c].x + xv[c].y * xv[c].y + xv[c].z * xv[c].z + xv[c].w * xv[c].w;
+          pk[2 * c] = (uint32_t)float_to_bf16(xv[c].x * gv[c].x) |
+                      ((uint32_t)float_to_bf16(xv[c].y * gv[c].y) << 16);
+          pk[2 * c + 1] = (uint32_t)float_to_bf16(xv[c].z * gv[c].z) |
+                          ((uint32_t)float_to_bf16(xv[c].w * gv[c].w) << 16);
+        }
+        a0[t] = u32x4_t{pk[0], pk[1], pk[2], pk[3]};
+        a1[t] = u32x4_t{pk[4], pk[5], pk[6], pk[7]};
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        a0[t] = (k < K) ? *(const u32x4_t*)(arow[t] + k) : zero;
+        a1[t] = (k + 8 < K) ? *(const u32x4_t*)(arow[t] + k + 8) : zero;
+      }
     }
 #pragma unroll
     for (int r = 0; r < RG; ++r)
@@ -425,7 +463,24 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
     for (int t = 0; t < MT; ++t)
 #pragma unroll
       for (int e = 0; e < 4; ++e) part[wave][r * MT + t][lane][e] = acc[r][t][e];
+  if (NORM) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      float v = ss[t];
+      v += __shfl_xor(v, 16, 64);
+      v += __shfl_xor(v, 32, 64);
+      if (lane < 16) ssum[wave][t][lane] = v;
+    }
+  }
   __syncthreads();
+  // the token's 1 / sqrt(mean(x^2) + eps): the waves' partial sums in wave order
+  auto inv_rms = [&](int t, int j) {
+    if (!NORM) return 1.0f;
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) tot += ssum[w][t][j];
+    return 1.0f / sqrtf(tot / (float)K + eps);
+  };
   if (EPI == EPI_SWIGLU) {
     // row groups alternate gate / up: the pair (2 p, 2 p + 1) gives 16 outputs per token
     for (int item = tid; item < (RG / 2) * MT * 64; item += 512) {
@@ -441,11 +496,13 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
         }
       const int token = t * 16 + l % 16;
       if (token < M) {
+        const float inv = inv_rms(t, l % 16);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int n = n0 / 2 + p * 16 + 4 * (l / 16) + e;      // column of the [M, N / 2] output
           if (2 * n < N)
-            ((bf16_t*)Cv)[(size_t)token * (N / 2) + n] = float_to_bf16(swiglu_f(g[e], u[e]));
+            ((bf16_t*)Cv)[(size_t)token * (N / 2) + n] =
+                float_to_bf16(swiglu_f(g[e] * inv, u[e] * inv));
         }
       }
     }
@@ -462,6 +519,9 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
     // D[i][j]: i = 4 * (l / 16) + e is the W row (output feature), j = l % 16 the token
     const int token = t * 16 + l % 16;
     if (token < M) {
+      const float inv = inv_rms(t, l % 16);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[e] *= inv;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int n = n0 + r * 16 + 4 * (l / 16) + e;
@@ -498,26 +558,28 @@ __global__ void skinny_reduce_kernel(const float* __restrict__ ws, void* __restr
     ((float*)Cv)[i] += s;
 }
 
-template <int MT, int RG, bool WT>
+template <int MT, int RG, bool WT, bool NORM = false>
 static int launch_skinny(const void* A, const void* W, void* C, void* ws, int M, int N, int K,
-                         int epi, int ksplit, hipStream_t stream) {
+                         int epi, int ksplit, hipStream_t stream, const float* gain = nullptr,
+                         float eps = 0.f) {
   const dim3 grid((N + 16 * RG - 1) / (16 * RG), ksplit), block(512);
   void* dst = ksplit > 1 ? ws : C;
+  if (NORM && (ksplit != 1 || epi == EPI_ACC_F32)) return -3;
   if (epi == EPI_SWIGLU) {
     if (RG < 2 || ksplit != 1 || N % 32 != 0) return -3;
-    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, (RG < 2 ? 2 : RG), EPI_SWIGLU, WT>), grid, block,
-                       0, stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K);
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, (RG < 2 ? 2 : RG), EPI_SWIGLU, WT, NORM>), grid,
+                       block, 0, stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K, gain, eps);
     return (int)hipGetLastError();
   }
   if (epi == EPI_STORE_BF16)
-    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_STORE_BF16, WT>), grid, block, 0, stream,
-                       (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K);
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_STORE_BF16, WT, NORM>), grid, block, 0,
+                       stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K, gain, eps);
   else if (epi == EPI_STORE_F32)
-    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_STORE_F32, WT>), grid, block, 0, stream,
-                       (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K);
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_STORE_F32, WT, NORM>), grid, block, 0,
+                       stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K, gain, eps);
   else
-    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_ACC_F32, WT>), grid, block, 0, stream,
-                       (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K);
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_ACC_F32, WT, false>), grid, block, 0,
+                       stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K, gain, eps);
   if (ksplit > 1) {
     const size_t mn = (size_t)M * N;
     const unsigned blocks = (unsigned)((mn + 255) / 256);
@@ -552,5 +614,23 @@ extern "C" int zf_gemm_bf16_skinny(const void* A, const void* W, void* C, void* 
   if (rg == 2) { if (mt == 1) ZF_SK(1, 2); if (mt == 2) ZF_SK(2, 2); if (mt == 3) ZF_SK(3, 2); ZF_SK(4, 2); }
   if (rg == 4) { if (mt == 1) ZF_SK(1, 4); if (mt == 2) ZF_SK(2, 4); if (mt == 3) ZF_SK(3, 4); ZF_SK(4, 4); }
 #undef ZF_SK
+  return -4;
+}
+
+// The same product with the RMSNorm before it folded in: X is the float32 residual stream
+// [M, K], gain float32 [K]; W must be pre-tiled, M <= 64, no split over workgroups; epi is
+// store-bf16, store-f32 or SwiGLU.
+extern "C" int zf_norm_gemm_bf16_skinny(const float* X, const float* gain, float eps, const void* W,
+                                        void* C, int M, int N, int K, int epi, int rg,
+                                        hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K % 64 != 0 || N % (16 * rg) != 0 || epi == EPI_ACC_F32) return -3;
+  const int mt = (M + 15) / 16;
+#define ZF_NSK(MT, RG) \
+  return launch_skinny<MT, RG, true, true>(X, W, C, nullptr, M, N, K, epi, 1, stream, gain, eps)
+  if (rg == 1) { if (mt == 1) ZF_NSK(1, 1); if (mt == 2) ZF_NSK(2, 1); if (mt == 3) ZF_NSK(3, 1); ZF_NSK(4, 1); }
+  if (rg == 2) { if (mt == 1) ZF_NSK(1, 2); if (mt == 2) ZF_NSK(2, 2); if (mt == 3) ZF_NSK(3, 2); ZF_NSK(4, 2); }
+  if (rg == 4) { if (mt == 1) ZF_NSK(1, 4); if (mt == 2) ZF_NSK(2, 4); if (mt == 3) ZF_NSK(3, 4); ZF_NSK(4, 4); }
+#undef ZF_NSK
   return -4;
 }

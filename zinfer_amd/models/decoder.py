@@ -13,6 +13,7 @@ from ..config.specs import ModelSpec
 from ..errors import ConfigError
 from ..parts import BuildContext, TensorDecl, build_part
 from ..parts.linear import Linear, place_matrix
+from ..parts.norm import LazyRmsNorm, RmsNorm
 
 
 class DecoderModel:
@@ -83,7 +84,10 @@ class DecoderModel:
             return logits
         rows = step.scratch("want_rows", (n_rows, s.hidden_size), torch.float32)
         ops.gather_rows(x, step.want_rows, rows)
-        normed = step.scratch("final_normed", (n_rows, s.hidden_size), self.ctx.act_dtype)
-        self.final_norm.forward(rows, normed)
-        self.head.forward(normed, logits)
+        make = lambda: step.scratch("final_normed", (n_rows, s.hidden_size), self.ctx.act_dtype)
+        if isinstance(self.final_norm, RmsNorm) and rows.is_cuda \
+                and self.ctx.compute_dtype == torch.bfloat16:
+            self.head.forward(LazyRmsNorm(self.final_norm, rows, make), logits)   # folded if it can be
+        else:
+            self.head.forward(self.final_norm.forward(rows, make()), logits)
         return logits

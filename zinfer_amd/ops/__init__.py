@@ -172,6 +172,7 @@ def _workspace(name: str, numel: int, dtype: torch.dtype, device) -> torch.Tenso
 # ------------------------------------------------------------------------- matrix product
 _EPI_STORE_BF16, _EPI_STORE_F32, _EPI_ACC_F32, _EPI_SWIGLU = 0, 1, 2, 3
 SKINNY_MAX_M = 64
+NORM_FOLD_MAX_M = 16
 
 
 def _skinny_plan(M: int, N: int, K: int, tiled: bool):
@@ -255,6 +256,42 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         return
     _check(lib.zf_gemm_fma(_ptr(a), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), M, N, K,
                            1 if accumulate else 0, _stream()), "gemm")
+
+
+def norm_gemm_plan(M: int, N: int, K: int, w: torch.Tensor, w_tiled: bool):
+    """Row groups per workgroup if ``norm_gemm`` covers the product (the weight-streaming
+    kernel without a split over workgroups on a pre-tiled bfloat16 weight), else None."""
+    # beyond 16 tokens the lanes' extra work (32-bit rows, gains, conversions for every group
+    # of 16 tokens) costs more than the norm kernel it saves (measured)
+    if not (w_tiled and 0 < M <= NORM_FOLD_MAX_M and w.dtype == torch.bfloat16):
+        return None
+    rg, ks = _skinny_plan(M, N, K, True)
+    return rg if ks == 1 else None
+
+
+def norm_gemm(x: torch.Tensor, gain: torch.Tensor, eps: float, w: torch.Tensor,
+              out: torch.Tensor, swiglu: bool = False) -> None:
+    """out = rmsnorm(x, gain, eps) w^T with the norm folded into the weight-streaming product
+    (``w`` pre-tiled; with ``swiglu`` the rows of ``w`` alternate gate / up as for
+    ``gemm_swiglu`` and out is [M, N / 2]).  x float32 [M <= 64, K]; the sum of squares, the
+    scale and the product's sums are 32-bit, the MFMA operands bfloat16(x * gain)."""
+    _need_gpu(x, gain, w, out)
+    M, K = x.shape
+    N = w.shape[0]
+    rg = norm_gemm_plan(M, N, K, w, True)
+    if swiglu and 0 < M <= SKINNY_MAX_M:
+        rg = 4 if (M > 16 and N >= 16384) else 2
+    if rg is None or x.dtype != torch.float32 or gain.dtype != torch.float32 \
+            or gain.shape != (K,) or w.shape[1] != K or not can_pretile(w) \
+            or out.shape != (M, N // 2 if swiglu else N) \
+            or (swiglu and out.dtype != torch.bfloat16):
+        raise KernelUnavailable(f"norm_gemm: x {tuple(x.shape)} {x.dtype}, w {tuple(w.shape)}, "
+                                f"out {tuple(out.shape)} {out.dtype}")
+    epi = _EPI_SWIGLU if swiglu else \
+        (_EPI_STORE_BF16 if out.dtype == torch.bfloat16 else _EPI_STORE_F32)
+    lib = build.load("gemm")
+    _check(lib.zf_norm_gemm_bf16_skinny(_ptr(x), _ptr(gain), ctypes.c_float(eps), _ptr(w),
+                                        _ptr(out), M, N, K, epi, rg, _stream()), "norm_gemm")
 
 
 def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:

@@ -19,6 +19,7 @@ class GqaAttention(Mixer):
     token's position, softmax(q K^T / sqrt(hd)) V over the positions up to the token's own
     (query head h reads kv head h // G), output projection added to the residual."""
     graph_safe = True
+    accepts_lazy_norm = True       # h is only ever handed to the q/k/v product
     kernel_modules = ("elementwise", "gemm", "attention")
 
 

@@ -2,8 +2,11 @@ from __future__ import annotations
 
 from typing import Dict
 
+import torch
+
 from ..config.specs import PreNormBlockSpec
 from .base import Block, TensorDecl, build_part, register_part
+from .norm import LazyRmsNorm, RmsNorm
 
 
 class PreNormBlock(Block):
@@ -35,12 +38,18 @@ class PreNormBlock(Block):
     def cache_need(self):
         return self.mixer.cache_need()
 
+    def _normed(self, norm, consumer, x, step):
+        """The consumer's input: the normed activations, or, for a consumer that says it can
+        fold an RMSNorm into its first product, the norm still to be run."""
+        make = lambda: step.scratch("normed", x.shape, self.ctx.act_dtype)
+        if isinstance(norm, RmsNorm) and getattr(consumer, "accepts_lazy_norm", False) \
+                and x.is_cuda and self.ctx.compute_dtype == torch.bfloat16:
+            return LazyRmsNorm(norm, x, make)
+        return norm.forward(x, make())
+
     def forward(self, x, step, cache) -> None:
-        h = step.scratch("normed", x.shape, self.ctx.act_dtype)
-        self.mixer_norm.forward(x, h)
-        self.mixer.forward(h, x, step, cache)
-        self.ff_norm.forward(x, h)
-        self.feed_forward.forward(h, x, step)
+        self.mixer.forward(self._normed(self.mixer_norm, self.mixer, x, step), x, step, cache)
+        self.feed_forward.forward(self._normed(self.ff_norm, self.feed_forward, x, step), x, step)
 
 
 register_part("block", PreNormBlockSpec, PreNormBlock)

@@ -18,8 +18,17 @@ class Linear:
         self.tiled = bool(pretile and weight.is_cuda and ops.can_pretile(weight))
         self.weight = ops.pretile_weight(weight) if self.tiled else weight.contiguous()
 
-    def forward(self, x: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
-        """out = x W^T, or out += x W^T (``out`` float32) when ``accumulate``."""
+    def forward(self, x, out: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
+        """out = x W^T, or out += x W^T (``out`` float32) when ``accumulate``.  ``x`` may be a
+        norm that has not run yet (``LazyRmsNorm``): it is folded into the product when the
+        weight-streaming kernel covers it, else it runs first."""
+        if hasattr(x, "materialize"):
+            M, K = x.shape
+            if not accumulate and \
+                    ops.norm_gemm_plan(M, self.out_features, K, self.weight, self.tiled) is not None:
+                ops.norm_gemm(x.x, x.gain, x.eps, self.weight, out)
+                return out
+            x = x.materialize()
         ops.gemm(x, self.weight, out, accumulate, w_tiled=self.tiled)
         return out
 

@@ -16,6 +16,7 @@ class SwiGluMlp(FeedForward):
     gate and up rows are stacked into one matrix at load: each output keeps its own dot
     product."""
     graph_safe = True
+    accepts_lazy_norm = True
     kernel_modules = ("elementwise", "gemm")
 
 
@@ -45,6 +46,13 @@ class SwiGluMlp(FeedForward):
         I = self.spec.intermediate_size
         act = self.ctx.act_dtype
         a = step.scratch("ff_act", (T, I), act)
+        if self.fused and hasattr(h, "materialize") and self.gate_up.tiled \
+                and T <= ops.NORM_FOLD_MAX_M:
+            ops.norm_gemm(h.x, h.gain, h.eps, self.gate_up.weight, a, swiglu=True)
+            self.down.forward(a, residual, accumulate=True)
+            return
+        if hasattr(h, "materialize"):
+            h = h.materialize()
         if self.fused and h.dtype == torch.bfloat16:
             ops.gemm_swiglu(h, self.gate_up.weight, a, w_tiled=self.gate_up.tiled)
         else:

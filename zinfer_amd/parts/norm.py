@@ -28,4 +28,21 @@ class RmsNorm(Norm):
         return out
 
 
+class LazyRmsNorm:
+    """A norm that has not run yet: the residual rows and the norm's parameters.  A consumer
+    whose first matrix product can fold the norm in (``Linear.forward``) takes it apart;
+    anyone else calls ``materialize()`` and gets the normed activations (computed once)."""
+
+    def __init__(self, norm: "RmsNorm", x: torch.Tensor, make_out):
+        self.x, self.gain, self.eps = x, norm.gain, float(norm.spec.eps)
+        self.shape = x.shape
+        self._norm, self._make_out, self._out = norm, make_out, None
+
+    def materialize(self) -> torch.Tensor:
+        if self._out is None:
+            self._out = self._make_out()
+            self._norm.forward(self.x, self._out)
+        return self._out
+
+
 register_part("norm", RmsNormSpec, RmsNorm)
