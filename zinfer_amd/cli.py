@@ -24,6 +24,7 @@ USAGE = """Usage:
   zinfer bench [model_dir] <ids_csv> [max_new_tokens]
   zinfer bench-batch [model_dir] <ids_csv> <batch_size> [max_new_tokens]
   zinfer bench-continuous [model_dir] <ids_csv> <batch_size> <total_requests> [max_new_tokens]
+  zinfer bench-ops [model_dir] [--shape 8b|14b|32b] [--tokens 1,8,64,2048] [--iters N]
   zinfer random-model <config.json> <out_dir> [--seed <u64>] [--dtype bfloat16|float32]
 
 Defaults:
@@ -473,8 +474,11 @@ def main(argv: Optional[List[str]] = None) -> int:
             return cmd_bench(args, cmd)
         if cmd == "random-model":
             return cmd_random_model(args)
+        if cmd == "bench-ops":
+            from .bench_ops import main as bench_ops_main
+            return bench_ops_main(args)
         if cmd in ("quantize", "tokenize", "decode-ids", "generate-chat", "chat", "probe-linear",
-                   "probe-block", "probe-model", "bench-ops", "bench-suite"):
+                   "probe-block", "probe-model", "bench-suite"):
             print(f"zinfer: {cmd!r} belongs to what this engine does not build (text front "
                   "end, quantisation, CPU probes)", file=sys.stderr)
             return 2
