@@ -404,7 +404,43 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
 
   const u32x4_t zero = u32x4_t{0, 0, 0, 0};
   const int kstride = 512 * gridDim.y;
-  for (int k0 = (blockIdx.y * 8 + wave) * 64; k0 < K; k0 += kstride) {
+  int k0 = (blockIdx.y * 8 + wave) * 64;
+  if (WT && !NORM && RG * MT == 1) {
+    // one row group and up to 16 tokens per wave: take 4 k-steps at once so that more loads
+    // are in flight (pre-tiled weights need no bounds checks; K % 64 == 0); measured to help
+    // only in this case
+    constexpr int UNR = 4;
+    for (; k0 + (UNR - 1) * kstride < K; k0 += UNR * kstride) {
+      u32x4_t w0[UNR][RG], w1[UNR][RG], a0[UNR][MT], a1[UNR][MT];
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) {
+        const int kk = k0 + u * kstride;
+#pragma unroll
+        for (int r = 0; r < RG; ++r) {
+          const bf16_t* tile = wrow[r] + (size_t)(kk / 64) * 1024;
+          w0[u][r] = __builtin_nontemporal_load((const u32x4_t*)tile);
+          w1[u][r] = __builtin_nontemporal_load((const u32x4_t*)(tile + 512));
+        }
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          a0[u][t] = *(const u32x4_t*)(arow[t] + kk + g * 16);
+          a1[u][t] = *(const u32x4_t*)(arow[t] + kk + g * 16 + 8);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < UNR; ++u)
+#pragma unroll
+        for (int r = 0; r < RG; ++r)
+#pragma unroll
+          for (int t = 0; t < MT; ++t) {
+            acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                *(bf16x8_t*)&w0[u][r], *(bf16x8_t*)&a0[u][t], acc[r][t], 0, 0, 0);
+            acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                *(bf16x8_t*)&w1[u][r], *(bf16x8_t*)&a1[u][t], acc[r][t], 0, 0, 0);
+          }
+    }
+  }
+  for (; k0 < K; k0 += kstride) {
     const int k = k0 + g * 16;
     u32x4_t w0[RG], w1[RG];
 #pragma unroll
