@@ -136,3 +136,18 @@ def install(monkeypatch):
     import zinfer_amd.ops as ops
     for name in ALL:
         monkeypatch.setattr(ops, name, globals()[name])
+
+
+# ------------------------------------------------------------------- pool layouts
+def tile_k_pool(k_pool, n_kv_heads, page_size, hd):
+    """[page, kv head, row, hd] -> the MFMA attention kernels' order: every group of 16 rows
+    as [hd / 32][16 * ((d % 32) / 8) + row][d % 8]."""
+    p = k_pool.view(-1, n_kv_heads, page_size // 16, 16, hd // 32, 4, 8)
+    return p.permute(0, 1, 2, 4, 5, 3, 6).contiguous().view(k_pool.shape)
+
+
+def tile_v_pool(v_pool, n_kv_heads, page_size, hd):
+    """[page, kv head, hd, row] -> every group of 16 rows as
+    [hd / 16][16 * (row / 4) + d % 16][row % 4]."""
+    p = v_pool.view(-1, n_kv_heads, hd // 16, 16, page_size // 16, 4, 4)
+    return p.permute(0, 1, 4, 2, 5, 3, 6).contiguous().view(v_pool.shape)

@@ -263,6 +263,10 @@ def _run_attention(s, dtype, nH, nKV, hd, page_size, window, q_lens, ctx_lens):
                         page_size, max(q_lens), max(ctx_lens))
     got = torch.full((T, nH * hd), float("nan"), dtype=dtype, device=DEV)
     d = {k: v.to(DEV) for k, v in s.items() if isinstance(v, torch.Tensor)}
+    if _ops().mfma_attention_covers(dtype, nH, nKV, hd, page_size):
+        # the MFMA kernels read pools in their own order (what qk_norm_rope_kv_write writes)
+        d["k_pool"] = ref.tile_k_pool(d["k_pool"], nKV, page_size, hd)
+        d["v_pool"] = ref.tile_v_pool(d["v_pool"], nKV, page_size, hd)
     _ops().paged_attention(d["q"], d["k_pool"], d["v_pool"], d["block_table"], d["q_start"],
                            d["ctx_len"], d["seq_index"], got, scale, window, nH, nKV, hd,
                            page_size, max(q_lens), max(ctx_lens),
@@ -377,6 +381,9 @@ def test_qk_norm_rope_kv_write(dtype, nH, nKV, hd, page_size, use_norm, use_rope
                                  positions.to(DEV), slots.to(DEV), kp, vp, q_got, nH, nKV, hd,
                                  page_size)
     assert rel_err(q_got, q_want) <= tol(dtype)
+    if _ops().mfma_attention_covers(dtype, nH, nKV, hd, page_size):
+        pools[0] = ref.tile_k_pool(pools[0], nKV, page_size, hd)
+        pools[1] = ref.tile_v_pool(pools[1], nKV, page_size, hd)
     assert rel_err(kp, pools[0]) <= tol(dtype)
     assert torch.equal(vp.cpu(), pools[1])
     # in place, nothing stored: q and k come back in the qkv buffer, v is untouched

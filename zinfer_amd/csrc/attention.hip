@@ -111,10 +111,16 @@ extern "C" int zf_paged_attention_wave(const void* q, const void* k_pool, const 
 //  lane's score registers all belong to one query (its column): the soft-max runs in
 //  registers, the probabilities are already in the operand order of the second product
 //  O^T = V^T P^T, and the output accumulators of a lane belong to that same query, so the
-//  running rescale is a per-lane factor.  V^T is what the value pool stores
-//  ([page, kv head, hd, row]).  No LDS is used; K, V and Q go from global memory (L2) straight
-//  into MFMA operands.  page_size must be a multiple of 16, hd one of 32, 64, 128, 256.
-//  Soft-max in 32-bit with exp2 and the scale folded into the exponent.
+//  running rescale is a per-lane factor.  K, V and Q go from global memory straight into MFMA
+//  operands.  page_size must be a multiple of 16, hd one of 32, 64, 128, 256.  Soft-max in
+//  32-bit with exp2 and the scale folded into the exponent.
+//
+//  Pools these kernels read are in the MFMA operand order ("tiled", written so by
+//  qk_norm_rope_kv_write when it is told to): inside the block of one (page, kv head) every
+//  group of 16 rows (positions) is stored as the lanes of the decode kernel consume it,
+//    keys:    [hd / 32][lane = 16 * ((d % 32) / 8) + row][d % 8]        (1 KB per wave load)
+//    values:  [hd / 16][lane = 16 * (row / 4) + d % 16][row % 4]        (512 B per wave load)
+//  so that one wave load is consecutive memory instead of 16 pieces of 64 or 32 bytes.
 // =====================================================================================
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
@@ -141,135 +147,157 @@ __device__ __forceinline__ u32x2_t keep_range4(u32x2_t v, int n_lo, int n_hi) {
   return u32x2_t{(uint32_t)x, (uint32_t)(x >> 32)};
 }
 
+// offsets inside the block of one (page, kv head) of a tiled pool, group of 16 rows `grp`
+__device__ __forceinline__ size_t tiled_k_offset(int grp, int r16, int d, int hd) {
+  return (size_t)grp * 16 * hd + (d / 32) * 512 + (((d % 32) / 8) * 16 + r16) * 8 + d % 8;
+}
+__device__ __forceinline__ size_t tiled_v_offset(int grp, int r16, int d, int hd) {
+  return (size_t)grp * 16 * hd + (d / 16) * 256 + ((r16 / 4) * 16 + d % 16) * 4 + r16 % 4;
+}
+
 // ---------------------------------------------------------------- decode: one query token
-// Grid (sequence, kv head, split).  A split is the 64 keys [64 * split, 64 * split + 64) of
-// the context, so which keys a split holds depends on the context length only.  One wave
-// per workgroup takes its 64 keys in one go: all key loads are issued together, then all
-// value loads, the soft-max over the 64 scores needs no running rescale.  The G query heads
-// of the kv head are the columns of 16x16x32 MFMAs (G <= 16).  Each split writes an
-// un-normalised partial (max, sum, O[G, hd]); attn_decode_merge_kernel combines the splits
-// in split order.
-#define DEC_SPLIT 64
+// Grid (sequence, kv head, split).  A split is the 256 keys [256 * split, 256 * split + 256)
+// of the context, so which keys a split holds depends on the context length only.  Each of
+// the workgroup's 4 waves takes 64 of them in one go: all key loads are issued together,
+// then all value loads; the soft-max over a wave's 64 scores needs no running rescale.  The
+// G query heads of the kv head are the columns of 16x16x32 MFMAs (G <= 16).  The waves'
+// partials are combined through LDS in wave order; the workgroup writes one un-normalised
+// partial (max, sum, O[G, hd]) that attn_decode_merge_kernel combines in split order.
+#define DEC_SPLIT 256
+#define DEC_WAVE_KEYS 64
 
 template <int HD>
-__global__ __launch_bounds__(64) void attn_decode_kernel(
+__global__ __launch_bounds__(256) void attn_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int* __restrict__ block_table,
     const int* __restrict__ q_start, const int* __restrict__ ctx_len, float* __restrict__ ws_o,
     float* __restrict__ ws_ml, float scale_log2e, int window, int nH, int nKV, int ps,
     int max_pages, int max_splits) {
+  __shared__ __attribute__((aligned(16))) float s_o[4][16][HD];
+  __shared__ float s_m[4][16], s_l[4][16];
   const int s = blockIdx.x, kvh = blockIdx.y, sp = blockIdx.z;
   if (q_start[s + 1] - q_start[s] != 1) return;
   const int ctx = ctx_len[s], pos = ctx - 1;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int kb = sp * DEC_SPLIT;
-  const int k_begin = max(lo, kb), k_end = min(ctx, kb + DEC_SPLIT);
-  if (k_begin >= k_end) return;
+  if (max(lo, sp * DEC_SPLIT) >= min(ctx, (sp + 1) * DEC_SPLIT)) return;   // whole workgroup
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, j = lane % 16, qd = lane / 16;
+  const int kb = sp * DEC_SPLIT + wave * DEC_WAVE_KEYS;
+  const int k_begin = max(lo, kb), k_end = min(ctx, kb + DEC_WAVE_KEYS);
   const int G = nH / nKV;
-  const int lane = threadIdx.x, j = lane % 16, qd = lane / 16;
   const int t = q_start[s];
   const int* table = block_table + (size_t)s * max_pages;
-
-  // pages of the four 16-key groups; a group outside [k_begin, k_end) may have no page at
-  // all: it reads the page of a key that certainly exists and is masked
-  int page[4];
-  bool any[4];
-#pragma unroll
-  for (int h = 0; h < 4; ++h) {
-    const int base = kb + 16 * h;
-    any[h] = base < k_end && base + 16 > k_begin;
-    page[h] = table[(any[h] ? max(base, k_begin) : k_begin) / ps];
-  }
-  // keys: row i = lane % 16 of group h, head elements 32 step + 8 qd ..
-  u32x4_t kf[4][HD / 32];
-#pragma unroll
-  for (int h = 0; h < 4; ++h) {
-    const int key = min(max(kb + 16 * h + j, k_begin), k_end - 1);
-    const int kpage = any[h] ? page[h] : table[key / ps];
-    const bf16_t* krow = k_pool + (((size_t)kpage * nKV + kvh) * ps + key % ps) * HD + 8 * qd;
-#pragma unroll
-    for (int stp = 0; stp < HD / 32; ++stp) kf[h][stp] = *(const u32x4_t*)(krow + stp * 32);
-  }
-  bf16x8_t qf[HD / 32];
-  {
-    const bf16_t* qrow = q + ((size_t)t * nH + kvh * G + min(j, G - 1)) * HD + 8 * qd;
-#pragma unroll
-    for (int st = 0; st < HD / 32; ++st) {
-      u32x4_t v = *(const u32x4_t*)(qrow + st * 32);
-      if (j >= G) v = u32x4_t{0, 0, 0, 0};
-      qf[st] = *(bf16x8_t*)&v;
-    }
-  }
-  // values (transposed in the pool): row d = 16 dt + j, keys kb + 16 h + 4 qd .. + 3
-  u32x2_t vf[4][HD / 16];
-#pragma unroll
-  for (int h = 0; h < 4; ++h) {
-    const int off = (kb + 16 * h) % ps + 4 * qd;
-    const bf16_t* vb = v_pool + ((size_t)page[h] * nKV + kvh) * ps * HD + (size_t)j * ps + off;
-#pragma unroll
-    for (int dt = 0; dt < HD / 16; ++dt) vf[h][dt] = *(const u32x2_t*)(vb + (size_t)dt * 16 * ps);
-  }
-  f32x4_t st[4];
-#pragma unroll
-  for (int h = 0; h < 4; ++h) {
-    st[h] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int stp = 0; stp < HD / 32; ++stp)
-      st[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&kf[h][stp], qf[stp],
-                                                      st[h], 0, 0, 0);
-  }
-  // st[h][r]: key kb + 16 h + 4 qd + r, query column j
-  float sc[16];
-  float m = -INFINITY;
-#pragma unroll
-  for (int h = 0; h < 4; ++h)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int key = kb + 16 * h + 4 * qd + r;
-      const float v = (key >= k_begin && key < k_end) ? st[h][r] * scale_log2e : -INFINITY;
-      sc[h * 4 + r] = v;
-      m = fmaxf(m, v);
-    }
-  m = fmaxf(m, __shfl_xor(m, 16, 64));
-  m = fmaxf(m, __shfl_xor(m, 32, 64));
-  float l = 0.f;
-#pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    sc[e] = exp2f(sc[e] - m);
-    l += sc[e];
-  }
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
+  float m = -INFINITY, l = 0.f;
   f32x4_t o[HD / 16];
 #pragma unroll
   for (int dt = 0; dt < HD / 16; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  if (k_begin < k_end) {
+    // the four 16-key groups of this wave; a group outside [k_begin, k_end) may have no page
+    // at all: it reads the group of a key that certainly exists and is masked
+    const bf16_t* kg[4];
+    const bf16_t* vg[4];
 #pragma unroll
-  for (int hh = 0; hh < 2; ++hh) {     // two MFMAs of 32 keys: groups 2 hh and 2 hh + 1
-    u32x4_t pk = u32x4_t{pack_bf16(sc[8 * hh + 0], sc[8 * hh + 1]),
-                         pack_bf16(sc[8 * hh + 2], sc[8 * hh + 3]),
-                         pack_bf16(sc[8 * hh + 4], sc[8 * hh + 5]),
-                         pack_bf16(sc[8 * hh + 6], sc[8 * hh + 7])};
-    const bf16x8_t pf = *(bf16x8_t*)&pk;
-    const int b0 = kb + 32 * hh + 4 * qd, b1 = b0 + 16;
+    for (int h = 0; h < 4; ++h) {
+      const int base = kb + 16 * h;
+      const bool any = base < k_end && base + 16 > k_begin;
+      const int key = any ? base : (k_begin / 16) * 16;
+      const size_t blk = (((size_t)table[key / ps] * nKV + kvh) * ps + (key % ps)) * HD;
+      kg[h] = k_pool + blk + lane * 8;
+      vg[h] = v_pool + blk + lane * 4;
+    }
+    u32x4_t kf[4][HD / 32];
 #pragma unroll
-    for (int dt = 0; dt < HD / 16; ++dt) {
-      // stale or poisoned rows outside [k_begin, k_end) are zeroed: 0 * NaN would spoil the sum
-      const u32x2_t v0 = keep_range4(vf[2 * hh][dt], k_begin - b0, k_end - b0);
-      const u32x2_t v1 = keep_range4(vf[2 * hh + 1][dt], k_begin - b1, k_end - b1);
-      u32x4_t vv = u32x4_t{v0[0], v0[1], v1[0], v1[1]};
-      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8_t*)&vv, pf, o[dt], 0, 0, 0);
+    for (int h = 0; h < 4; ++h)
+#pragma unroll
+      for (int stp = 0; stp < HD / 32; ++stp) kf[h][stp] = *(const u32x4_t*)(kg[h] + stp * 512);
+    bf16x8_t qf[HD / 32];
+    {
+      const bf16_t* qrow = q + ((size_t)t * nH + kvh * G + min(j, G - 1)) * HD + 8 * qd;
+#pragma unroll
+      for (int st = 0; st < HD / 32; ++st) {
+        u32x4_t v = *(const u32x4_t*)(qrow + st * 32);
+        if (j >= G) v = u32x4_t{0, 0, 0, 0};
+        qf[st] = *(bf16x8_t*)&v;
+      }
+    }
+    // values: lane (d % 16 = j, keys 4 qd .. 4 qd + 3) of head-element tile dt
+    u32x2_t vf[4][HD / 16];
+#pragma unroll
+    for (int h = 0; h < 4; ++h)
+#pragma unroll
+      for (int dt = 0; dt < HD / 16; ++dt) vf[h][dt] = *(const u32x2_t*)(vg[h] + dt * 256);
+    f32x4_t st[4];
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+      st[h] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int stp = 0; stp < HD / 32; ++stp)
+        st[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&kf[h][stp], qf[stp],
+                                                        st[h], 0, 0, 0);
+    }
+    // st[h][r]: key kb + 16 h + 4 qd + r, query column j
+    float sc[16];
+#pragma unroll
+    for (int h = 0; h < 4; ++h)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int key = kb + 16 * h + 4 * qd + r;
+        const float v = (key >= k_begin && key < k_end) ? st[h][r] * scale_log2e : -INFINITY;
+        sc[h * 4 + r] = v;
+        m = fmaxf(m, v);
+      }
+    m = fmaxf(m, __shfl_xor(m, 16, 64));
+    m = fmaxf(m, __shfl_xor(m, 32, 64));
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      sc[e] = exp2f(sc[e] - m);
+      l += sc[e];
+    }
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {     // two MFMAs of 32 keys: groups 2 hh and 2 hh + 1
+      u32x4_t pk = u32x4_t{pack_bf16(sc[8 * hh + 0], sc[8 * hh + 1]),
+                           pack_bf16(sc[8 * hh + 2], sc[8 * hh + 3]),
+                           pack_bf16(sc[8 * hh + 4], sc[8 * hh + 5]),
+                           pack_bf16(sc[8 * hh + 6], sc[8 * hh + 7])};
+      const bf16x8_t pf = *(bf16x8_t*)&pk;
+      const int b0 = kb + 32 * hh + 4 * qd, b1 = b0 + 16;
+#pragma unroll
+      for (int dt = 0; dt < HD / 16; ++dt) {
+        // stale or poisoned rows outside [k_begin, k_end) are zeroed: 0 * NaN would spoil the sum
+        const u32x2_t v0 = keep_range4(vf[2 * hh][dt], k_begin - b0, k_end - b0);
+        const u32x2_t v1 = keep_range4(vf[2 * hh + 1][dt], k_begin - b1, k_end - b1);
+        u32x4_t vv = u32x4_t{v0[0], v0[1], v1[0], v1[1]};
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8_t*)&vv, pf, o[dt], 0, 0, 0);
+      }
     }
   }
-  if (j < G) {
-    const int head = kvh * G + j;
-    const size_t slot = ((size_t)s * nH + head) * max_splits + sp;
-    float* dst = ws_o + slot * HD;
+  // this wave's partial for query column j: rows d = 16 dt + 4 qd + r
 #pragma unroll
-    for (int dt = 0; dt < HD / 16; ++dt)
-      *(f32x4_t*)(dst + dt * 16 + 4 * qd) = o[dt];
-    if (qd == 0) {
-      ws_ml[slot * 2] = m;
-      ws_ml[slot * 2 + 1] = l;
+  for (int dt = 0; dt < HD / 16; ++dt) *(f32x4_t*)&s_o[wave][j][dt * 16 + 4 * qd] = o[dt];
+  if (qd == 0) {
+    s_m[wave][j] = m;
+    s_l[wave][j] = l;
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < G * HD; idx += 256) {
+    const int col = idx / HD, d = idx % HD;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) mx = fmaxf(mx, s_m[w][col]);
+    float acc = 0.f, den = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = exp2f(s_m[w][col] - mx);     // a wave without keys has max -inf: weight 0
+      acc += f * s_o[w][col][d];
+      den += f * s_l[w][col];
+    }
+    const size_t slot = ((size_t)s * nH + kvh * G + col) * max_splits + sp;
+    ws_o[slot * HD + d] = acc;
+    if (d == 0) {
+      ws_ml[slot * 2] = mx;
+      ws_ml[slot * 2 + 1] = den;
     }
   }
 }
@@ -335,7 +363,7 @@ __global__ __launch_bounds__(64) void attn_decode_merge_kernel(
 }
 
 // ws_o: n_seqs * nH * max_splits * hd floats, ws_ml: n_seqs * nH * max_splits * 2 floats,
-// max_splits >= ceil(longest context / 64).
+// max_splits >= ceil(longest context / 256); the pools are tiled.
 extern "C" int zf_attn_decode_bf16(const void* q, const void* k_pool, const void* v_pool,
                                    const int* block_table, const int* q_start,
                                    const int* ctx_len, void* out, float* ws_o, float* ws_ml,
@@ -347,7 +375,7 @@ extern "C" int zf_attn_decode_bf16(const void* q, const void* k_pool, const void
   const float scale_log2e = scale * 1.4426950408889634f;
   dim3 grid(n_seqs, nKV, max_splits);
 #define ZF_DEC(HD)                                                                              \
-  hipLaunchKernelGGL(attn_decode_kernel<HD>, grid, dim3(64), 0, stream, (const bf16_t*)q,       \
+  hipLaunchKernelGGL(attn_decode_kernel<HD>, grid, dim3(256), 0, stream, (const bf16_t*)q,      \
                      (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, q_start,        \
                      ctx_len, ws_o, ws_ml, scale_log2e, window, nH, nKV, page_size, max_pages,  \
                      max_splits)
@@ -424,9 +452,12 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
     auto load_keys = [&](int kb, u32x4_t* dst) {
       const int key = min(max(kb + j, lo_min), p_max);
       const int kpage = table[key / ps];
-      const bf16_t* krow = k_pool + (((size_t)kpage * nKV + kvh) * ps + key % ps) * HD + 8 * hf;
+      // tiled pool: head elements 16 stp + 8 hf .. + 8 of row key % 16 of its 16-row group
+      const bf16_t* kblk = k_pool + ((size_t)kpage * nKV + kvh) * ps * HD +
+                           (size_t)((key % ps) / 16) * 16 * HD + (hf * 16 + key % 16) * 8;
 #pragma unroll
-      for (int stp = 0; stp < HD / 16; ++stp) dst[stp] = *(const u32x4_t*)(krow + stp * 16);
+      for (int stp = 0; stp < HD / 16; ++stp)
+        dst[stp] = *(const u32x4_t*)(kblk + (stp / 2) * 512 + (stp % 2) * 256);
     };
     const int kb0 = (lo_min / 32) * 32;
     u32x4_t kf[HD / 16];
@@ -441,12 +472,14 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
         any[u] = base <= p_max && base + 16 > lo_min;
         const int safe = any[u] ? max(base, lo_min) : p_max;
         const int vpage = table[safe / ps];
-        const int off = base % ps + 4 * hf;
-        const bf16_t* vb = v_pool + ((size_t)vpage * nKV + kvh) * ps * HD + (size_t)j * ps + off;
+        // tiled pool: head element 32 dt + j, rows 4 hf .. + 3 and 8 + 4 hf .. + 3 of the group
+        const bf16_t* vb = v_pool + ((size_t)vpage * nKV + kvh) * ps * HD +
+                           (size_t)((base % ps) / 16) * 16 * HD + (j / 16) * 256 +
+                           (hf * 16 + j % 16) * 4;
 #pragma unroll
         for (int dt = 0; dt < HD / 32; ++dt) {
-          vf[u][dt][0] = *(const u32x2_t*)(vb + (size_t)dt * 32 * ps);
-          vf[u][dt][1] = *(const u32x2_t*)(vb + (size_t)dt * 32 * ps + 8);
+          vf[u][dt][0] = *(const u32x2_t*)(vb + dt * 512);
+          vf[u][dt][1] = *(const u32x2_t*)(vb + dt * 512 + 128);
         }
       }
       // S^T: rows are the keys kb + (lane % 32), clamped into the keys that exist

@@ -112,13 +112,15 @@ extern "C" int zf_rmsnorm(const float* x, const float* gain, void* out, int out_
 //   v -> the value pool, laid out [page, kv head, hd, row]: the rows (positions) of a page
 //        are contiguous for each element of the head, which is the operand order the
 //        attention kernels' second matrix product wants
+//   tiled: both pools in the MFMA attention kernels' own order inside every group of 16 rows
+//        (see attention.hip); page_size % 16 == 0 and hd % 32 == 0
 template <typename T>
 __global__ void qk_norm_rope_kv_write_kernel(
     T* __restrict__ qkv, const float* __restrict__ q_gain, const float* __restrict__ k_gain,
     float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int* __restrict__ positions, const int* __restrict__ slot_mapping,
     T* __restrict__ k_pool, T* __restrict__ v_pool, T* __restrict__ q_out, int nH, int nKV,
-    int hd, int page_size) {
+    int hd, int page_size, int tiled) {
   const int t = blockIdx.x;
   const int head = blockIdx.y;
   const int lane = threadIdx.x;
@@ -131,20 +133,33 @@ __global__ void qk_norm_rope_kv_write_kernel(
     const int kvh = head - nH - nKV;
     const int slot = slot_mapping[t];
     const int page = slot / page_size, r = slot % page_size;
-    T* dst = v_pool + ((size_t)page * nKV + kvh) * page_size * hd + r;
-    for (int i = lane; i < hd; i += ZF_WAVE) dst[(size_t)i * page_size] = src[i];
+    T* blk = v_pool + ((size_t)page * nKV + kvh) * page_size * hd;
+    if (tiled) {      // the MFMA attention kernels' order inside each group of 16 rows
+      T* grp = blk + (size_t)(r / 16) * 16 * hd + ((r % 16) / 4) * 64 + r % 4;
+      for (int i = lane; i < hd; i += ZF_WAVE) grp[(i / 16) * 256 + (i % 16) * 4] = src[i];
+    } else {
+      for (int i = lane; i < hd; i += ZF_WAVE) blk[(size_t)i * page_size + r] = src[i];
+    }
     return;
   }
   const bool is_q = head < nH;
   const float* gain = is_q ? q_gain : k_gain;
   T* dst;
+  bool k_tiled = false;
+  int r16 = 0;
   if (is_q) {
     dst = q_out ? q_out + (size_t)t * nH * hd + (size_t)head * hd : src;
   } else if (slot_mapping) {
     const int kvh = head - nH;
     const int slot = slot_mapping[t];
     const int page = slot / page_size, r = slot % page_size;
-    dst = k_pool + (((size_t)page * nKV + kvh) * page_size + r) * hd;
+    if (tiled) {      // element d of row r goes to [d / 32][16 * ((d % 32) / 8) + r % 16][d % 8]
+      k_tiled = true;
+      r16 = r % 16;
+      dst = k_pool + ((size_t)page * nKV + kvh) * page_size * hd + (size_t)(r / 16) * 16 * hd;
+    } else {
+      dst = k_pool + (((size_t)page * nKV + kvh) * page_size + r) * hd;
+    }
   } else {
     dst = src;
   }
@@ -173,8 +188,14 @@ __global__ void qk_norm_rope_kv_write_kernel(
       x0 = r0;
       x1 = r1;
     }
-    store_from_float<T>(dst + i, x0);
-    store_from_float<T>(dst + i + half, x1);
+    if (k_tiled) {
+      const int d0 = i, d1 = i + half;
+      store_from_float<T>(dst + (d0 / 32) * 512 + (((d0 % 32) / 8) * 16 + r16) * 8 + d0 % 8, x0);
+      store_from_float<T>(dst + (d1 / 32) * 512 + (((d1 % 32) / 8) * 16 + r16) * 8 + d1 % 8, x1);
+    } else {
+      store_from_float<T>(dst + i, x0);
+      store_from_float<T>(dst + i + half, x1);
+    }
   }
 }
 
@@ -183,17 +204,20 @@ extern "C" int zf_qk_norm_rope_kv_write(void* qkv, int dtype, const float* q_gai
                                         const float* sin_t, const int* positions,
                                         const int* slot_mapping, void* k_pool, void* v_pool,
                                         void* q_out, int T, int nH, int nKV, int hd,
-                                        int page_size, hipStream_t stream) {
+                                        int page_size, int tiled, hipStream_t stream) {
   if (T <= 0) return 0;
+  if (tiled && (page_size % 16 != 0 || hd % 32 != 0)) return -2;
   dim3 grid(T, nH + 2 * nKV);
   if (dtype == ZF_F32)
     hipLaunchKernelGGL(qk_norm_rope_kv_write_kernel<float>, grid, dim3(ZF_WAVE), 0, stream,
                        (float*)qkv, q_gain, k_gain, eps, cos_t, sin_t, positions, slot_mapping,
-                       (float*)k_pool, (float*)v_pool, (float*)q_out, nH, nKV, hd, page_size);
+                       (float*)k_pool, (float*)v_pool, (float*)q_out, nH, nKV, hd, page_size,
+                       tiled);
   else
     hipLaunchKernelGGL(qk_norm_rope_kv_write_kernel<bf16_t>, grid, dim3(ZF_WAVE), 0, stream,
                        (bf16_t*)qkv, q_gain, k_gain, eps, cos_t, sin_t, positions, slot_mapping,
-                       (bf16_t*)k_pool, (bf16_t*)v_pool, (bf16_t*)q_out, nH, nKV, hd, page_size);
+                       (bf16_t*)k_pool, (bf16_t*)v_pool, (bf16_t*)q_out, nH, nKV, hd, page_size,
+                       tiled);
   ZF_CHECK_LAUNCH();
 }
 

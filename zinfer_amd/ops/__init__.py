@@ -83,7 +83,8 @@ def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, cos, sin, positions, slot_ma
     """Per token and head of ``qkv`` [T, (nH + 2 nKV) hd]: optional RMSNorm of q and k heads
     with the [hd] gains, optional half-split rotation from the [max_pos, hd/2] tables at
     ``positions``; q goes to ``q_out`` [T, nH hd] (in place if None), k and v go into the
-    pools at ``slot_mapping`` (k in place if None)."""
+    pools at ``slot_mapping`` (k in place if None).  Pools of a shape the MFMA attention
+    kernels cover (``mfma_attention_covers``) are written in those kernels' own order."""
     _need_gpu(qkv, q_gain, k_gain, cos, sin, positions, slot_mapping, k_pool, v_pool, q_out)
     T = qkv.shape[0]
     width = (n_heads + 2 * n_kv_heads) * head_dim
@@ -110,7 +111,9 @@ def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, cos, sin, positions, slot_ma
     _check(lib.zf_qk_norm_rope_kv_write(
         _ptr(qkv), _dt(qkv), _ptr(q_gain), _ptr(k_gain), ctypes.c_float(eps), _ptr(cos),
         _ptr(sin), _ptr(positions), _ptr(slot_mapping), _ptr(k_pool), _ptr(v_pool), _ptr(q_out),
-        T, n_heads, n_kv_heads, head_dim, page_size, _stream()), "qk_norm_rope_kv_write")
+        T, n_heads, n_kv_heads, head_dim, page_size,
+        1 if mfma_attention_covers(qkv.dtype, n_heads, n_kv_heads, head_dim, page_size) else 0,
+        _stream()), "qk_norm_rope_kv_write")
 
 
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
@@ -332,10 +335,14 @@ def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bo
 
 
 # ------------------------------------------------------------------------- attention
-DECODE_SPLIT_KEYS = 64      # keys per split of the decode kernel (DEC_SPLIT in attention.hip)
+DECODE_SPLIT_KEYS = 256     # keys per split of the decode kernel (DEC_SPLIT in attention.hip)
 
 
 def mfma_attention_covers(dtype, n_heads, n_kv_heads, head_dim, page_size) -> bool:
+    """Whether the bfloat16 MFMA attention kernels serve this shape.  If so, the pools are
+    kept in those kernels' own order inside every group of 16 rows (keys ``[hd / 32][16 *
+    ((d % 32) / 8) + row][d % 8]``, values ``[hd / 16][16 * (row / 4) + d % 16][row % 4]``);
+    otherwise keys are ``[row][hd]`` and values ``[hd][row]`` inside a (page, kv head) block."""
     return dtype == torch.bfloat16 and head_dim in (32, 64, 128, 256) and page_size % 16 == 0 \
         and n_heads // n_kv_heads <= 16
 
