@@ -33,15 +33,16 @@ QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidd
                 torch_dtype="bfloat16")
 
 
-def random_model(raw: dict, dtype: str, seed: int, device: str):
+def random_model(raw: dict, dtype: str, seed: int, device: str, store: str = None):
     """Model of the given shape with weights drawn on the device: matrices and the embedding
-    N(0, 0.02), norm gains 1 + U(-0.1, 0.1)."""
+    N(0, 0.02), norm gains 1 + U(-0.1, 0.1).  ``store`` is the dtype the drawn values are
+    rounded to (default: the compute dtype)."""
     import torch
     from zinfer_amd.config import Qwen3Config
     from zinfer_amd.models.build import build_model, declare_tensors
     cfg = Qwen3Config.from_dict(raw)
     spec = cfg.model_spec()
-    store = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    store = torch.bfloat16 if (store or dtype) == "bfloat16" else torch.float32
     gen = torch.Generator(device=device)
     gen.manual_seed(seed)
     tensors = {}
@@ -137,6 +138,29 @@ def run_decode(llm, cfg, batch: int, prompt_len: int, steps: int, warmup: int, s
     return dt, (ctx0 + ctx1) / 2 + 0.5
 
 
+def check_fp32(llm, cfg, raw, args) -> dict:
+    """The same random weights (bfloat16 values widened) through the 32-bit path: FMA
+    products, wave attention, 32-bit cache.  Reports the largest difference of the last
+    position's logits relative to their largest magnitude, and whether the arg-max agrees."""
+    import torch
+    from zinfer_amd.engine import Engine, StepEntry
+    T = args.check_fp32
+    g = torch.Generator().manual_seed(args.seed + 99)
+    toks = torch.randint(0, cfg.vocab_size, (T,), generator=g).tolist()
+    want = [T - 1]
+    lb = llm.engine.step([StepEntry("chk", toks, want)], end=["chk"]).float().clone()
+    # same seed, same draws, rounded to bfloat16 as the serving model's, then widened
+    _, model32 = random_model(raw, "float32", args.seed, "cuda:0", store="bfloat16")
+    eng32 = Engine(model32, page_size=16, num_pages=(T + 15) // 16 + 1, max_requests=2)
+    t0 = time.perf_counter()
+    lf = eng32.step([StepEntry("chk", toks, want)], end=["chk"]).float()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    err = float((lb - lf).abs().max() / lf.abs().max())
+    return {"tokens": T, "rel_max_diff": round(err, 5), "fp32_ms": round(dt * 1e3, 1),
+            "argmax_equal": bool(int(lb.argmax()) == int(lf.argmax()))}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -149,6 +173,9 @@ def main() -> int:
                     "configuration (both numbers are reported)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--check-fp32", type=int, default=0, metavar="TOKENS",
+                    help="also run a prompt of TOKENS tokens through a true 32-bit engine with "
+                         "the same weights and report how far the logits are apart")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -213,6 +240,8 @@ def main() -> int:
         "points": points,
         "build_s": round(build_s, 1),
     }
+    if args.check_fp32:
+        line["fp32_check"] = check_fp32(llm, cfg, raw, args)
     print(json.dumps(line))
     return 0
 
