@@ -122,13 +122,24 @@ def run_decode(llm, cfg, batch: int, prompt_len: int, steps: int, warmup: int, s
     while sched.waiting or any(r.pending > 1 or not r.generated for r in sched.running):
         sched.step()                         # prompts, one or more per step
     assert len(sched.running) == batch
-    for _ in range(warmup):
-        sched.step()
+    most = sched.multi_step
+
+    def run_exactly(n):
+        """``n`` decode steps of the whole batch; the scheduler may run several in a row on
+        the device per call, never more than are still to do."""
+        done = 0
+        while done < n:
+            sched.multi_step = min(most, n - done)
+            sched.step()
+            assert sched.last_steps >= 1
+            done += sched.last_steps
+        assert done == n
+
+    run_exactly(warmup)
     torch.cuda.synchronize()
     ctx0 = sum(r.n_computed for r in sched.running) / batch
     t0 = time.perf_counter()
-    for _ in range(steps):
-        sched.step()
+    run_exactly(steps)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ctx1 = sum(r.n_computed for r in sched.running) / batch
@@ -232,7 +243,8 @@ def main() -> int:
                    "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
                    "global_batch": args.batch, "prompt_len": args.prompt_len,
                    "seq_len": int(round(mean_ctx)), "page_size": page,
-                   "parallelism": "single GPU", "sampling": "greedy"},
+                   "parallelism": "single GPU", "sampling": "greedy",
+                   "steps_in_a_row": llm.scheduler_options["multi_step"]},
         "prefill": {"value": round(args.prefill_tokens / pre_s, 1), "tokens": args.prefill_tokens,
                     "ms": round(pre_s * 1e3, 3), "frac": round(flops / pre_s / peak, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,

@@ -216,3 +216,51 @@ def test_graph_replays_equal_eager_steps(dtype, tmp_path_factory):
                 eng.release("g1")
             reqs.pop("g1")
     assert a.graph_replays >= 10 and b.graph_replays == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_in_a_row_equal_single_steps(dtype, tmp_path_factory):
+    """Several decode steps without the host between them (the device moves tokens,
+    positions and slots on) against the same steps one by one: the same tokens, greedy and
+    sampled, over page edges, and the same cache afterwards."""
+    from zinfer_amd import ops
+    from zinfer_amd.engine import StepEntry
+    from zinfer_amd.engine.replay import make_engine
+    name = "D"
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    path = tiny.model_dir_of(name, str(tmp_path_factory.getbasetemp()), store)
+    V = tiny.CONFIGS[name]["vocab_size"]
+    a = make_engine(path, dtype, 1024, DEV)
+    b = make_engine(path, dtype, 1024, DEV)
+    reqs = {f"m{i}": tiny.random_tokens(n, V, 700 + i) for i, n in enumerate((70, 33, 127, 2))}
+    cur = None
+    for eng in (a, b):
+        lg = eng.step([StepEntry(r, t, [len(t) - 1]) for r, t in reqs.items()])
+        cur = eng.argmax(lg)
+    rng = np.random.default_rng(5)
+    for n_steps, sampled in ((19, False), (1, False), (9, True), (2, True)):
+        records = None
+        if sampled:
+            records = np.zeros((n_steps, len(reqs)), dtype=ops.SAMPLE_ROW_DTYPE)
+            for s in range(n_steps):
+                for i in range(len(reqs)):
+                    records[s, i] = (0.9, 0.95, 0.0, 40, rng.random())
+        start = cur
+        drawn = a.decode_steps([StepEntry(r, [t], [0]) for r, t in zip(reqs, start)], n_steps,
+                               records)
+        assert len(drawn) == n_steps
+        for s in range(n_steps):
+            lg = b.step([StepEntry(r, [t], [0]) for r, t in zip(reqs, cur)])
+            cur = b.sample(lg, records[s]) if sampled else b.argmax(lg)
+            assert cur == drawn[s], f"{n_steps} steps, step {s}"
+        assert [a.length(r) for r in reqs] == [b.length(r) for r in reqs]
+    entries = [StepEntry(r, [t], [0]) for r, t in zip(reqs, cur)]
+    assert torch.equal(a.step(entries), b.step(entries))
+    # refused before anything runs: too many steps for the pages that are free
+    free = a.cache.num_free_pages()
+    too_many = 4 * free[0] + 32         # four requests, pages of 16: more pages than are free
+    assert too_many < 450               # still inside the position table
+    with pytest.raises(Exception, match="CacheFull"):
+        a.decode_steps([StepEntry(r, [1], [0]) for r in reqs], too_many)
+    assert a.cache.num_free_pages() == free
+    a.cache.check()

@@ -206,6 +206,33 @@ def test_greedy_generation_through_the_entry_point(dtype, tmp_path):
             logits = plain.model_forward_batched(cfg, w, toks)[-1].float().numpy()
             assert g == sample_token(logits, toks, sp2, rng)
             toks.append(g)
+    # without penalties several decode steps run in a row on the device: the same tokens as
+    # with the host between all steps, also when a request stops in the middle of a run
+    sp3 = SamplingParams(temperature=0.9, top_k=30, top_p=0.9, seed=21, max_new_tokens=21,
+                         ignore_eos=True)
+    runs = llm.generate(prompts[1:4], sp3)
+    assert [len(r) for r in runs] == [21, 21, 21]
+    single = LLM(path, dtype=dtype, device=DEV, page_size=tiny.PAGE_SIZE[name], max_tokens=448,
+                 max_step_tokens=48, chunk_size=24, multi_step=1)
+    assert single.generate(prompts[1:4], sp3) == runs
+    assert llm.engine.steps_run == single.engine.steps_run
+    stop = runs[0][12]
+    first = runs[0].index(stop)
+    for params in (SamplingParams(temperature=0.9, top_k=30, top_p=0.9, seed=21,
+                                  max_new_tokens=21, stop_token_ids=(stop,)),
+                   SamplingParams(temperature=0.0, max_new_tokens=19, stop_token_ids=(stop,))):
+        a, b = llm.generate(prompts[1:4], params), single.generate(prompts[1:4], params)
+        assert a == b
+        assert not llm.engine.cache.requests and not single.engine.cache.requests
+    assert llm.generate(prompts[1:4], SamplingParams(
+        temperature=0.9, top_k=30, top_p=0.9, seed=21, max_new_tokens=21,
+        stop_token_ids=(stop,)))[0] == runs[0][:first]
+    if dtype == "float32":
+        toks, rng = list(prompts[1]), Xoshiro256pp(21)
+        for g in runs[0]:
+            logits = plain.model_forward_batched(cfg, w, toks)[-1].float().numpy()
+            assert g == sample_token(logits, toks, sp3, rng)
+            toks.append(g)
 
 
 # ----------------------------------------------------------------------------- toy parts
@@ -381,6 +408,23 @@ def test_toy_architecture_registered_built_and_stepped(kind, tmp_path):
                 eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]])
             held = [g.pages.num_held for g in eng.cache.groups]
             assert held[0] == 6 and held[1] <= 3       # 90 tokens: 6 pages; window 19: <= 3
+            # several decode steps in a row on the device, over page edges of both groups
+            one = make_engine(path, "float32", 256, DEV)
+            many = make_engine(path, "float32", 256, DEV)
+            heads = {r: t[:n] for (r, t), n in zip(requests.items(), (50, 7, 61, 33))}
+            for eng in (one, many):
+                lg = eng.step([StepEntry(r, t, [len(t) - 1]) for r, t in heads.items()])
+                first = eng.argmax(lg)
+            drawn = many.decode_steps([StepEntry(r, [t], [0]) for r, t in zip(heads, first)], 21)
+            cur = first
+            for s in range(21):
+                lg = one.step([StepEntry(r, [t], [0]) for r, t in zip(heads, cur)])
+                cur = one.argmax(lg)
+                assert cur == drawn[s], f"step {s}"
+            for eng in (one, many):
+                eng.cache.check()
+            assert [g.pages.num_held for g in one.cache.groups] == \
+                [g.pages.num_held for g in many.cache.groups]
     finally:
         unregister_architecture("ToyForCausalLM")
         unregister_part("mixer", ToyStateSpec)

@@ -167,3 +167,70 @@ def test_sampled_output_does_not_depend_on_the_batch():
         return s.run()[rid].generated
     assert run(0) == run(3)
     assert len(set(run(0))) > 1
+
+
+class FakeGraphEngine(FakeEngine):
+    """A stand-in whose decode steps may run several in a row (as the engine's graph replays)."""
+    use_graphs = True
+
+    def __init__(self, *args, **kw):
+        super().__init__(*args, **kw)
+        self.runs = []
+
+    def decode_steps(self, entries, n_steps, records=None):
+        assert all(len(e.tokens) == 1 for e in entries)
+        self.runs.append((len(entries), n_steps, records is not None))
+        lens = [(e.request_id, self.cache.length(e.request_id) + n_steps) for e in entries]
+        assert self.cache.can_reserve(lens)
+        for rid, n in lens:
+            self.cache.reserve(rid, n)
+            self.cache.commit(rid, n)
+        self.cache.check()
+        cur = [e.tokens[0] for e in entries]
+        out = []
+        for _ in range(n_steps):
+            cur = [(t + 1) % V for t in cur]
+            out.append(cur)
+        return out
+
+
+def test_decode_steps_in_a_row_only_when_everyone_decodes_and_nobody_waits():
+    eng = FakeGraphEngine(num_pages=64)
+    s = Scheduler(eng, max_step_tokens=8, chunk_size=8, multi_step=4)
+    a = s.add_request([1, 2, 3], SamplingParams(max_new_tokens=11, **GREEDY))
+    b = s.add_request(list(range(10, 22)), SamplingParams(max_new_tokens=7, **GREEDY))
+    out = s.run()
+    assert out[a].generated == list(range(4, 15)) and out[b].generated == list(range(22, 29))
+    # while b is still in its prompt every step goes through the host; afterwards runs of at
+    # most 4, never beyond what a request may still generate
+    assert eng.runs and all(n <= 4 for _, n, _ in eng.runs)
+    assert not any(len(st) == 2 and all(n == 1 for _, n, _ in st) for st in eng.log[3:])
+    assert eng.cache.num_free_pages() == [64] and not eng.cache.requests
+    assert s.n_steps == len(eng.log) + sum(n for _, n, _ in eng.runs)
+
+
+def test_decode_steps_in_a_row_stop_at_eos_and_discard_the_rest():
+    eng = FakeGraphEngine(num_pages=64)
+    s = Scheduler(eng, max_step_tokens=8, multi_step=8, eos_token_ids=(9,))
+    a = s.add_request([3], SamplingParams(temperature=0.0, max_new_tokens=30))
+    b = s.add_request([20], SamplingParams(temperature=0.0, max_new_tokens=12, ignore_eos=True))
+    out = s.run()
+    assert out[a].generated == [4, 5, 6, 7, 8] and out[a].finish_reason == "eos"
+    assert out[b].generated == list(range(21, 33)) and out[b].finish_reason == "length"
+    assert eng.cache.num_free_pages() == [64]
+
+
+def test_decode_steps_in_a_row_shrink_to_the_free_pages_and_skip_penalties():
+    eng = FakeGraphEngine(num_pages=4, page_size=4)
+    s = Scheduler(eng, max_step_tokens=8, multi_step=8)
+    a = s.add_request([1, 2], SamplingParams(max_new_tokens=14, **GREEDY))
+    out = s.run()
+    assert out[a].generated == list(range(3, 17))
+    assert all(n <= 8 for _, n, _ in eng.runs) and s.n_preemptions == 0
+    # penalties need the tokens on the host after every step
+    eng = FakeGraphEngine(num_pages=16)
+    s = Scheduler(eng, max_step_tokens=8, multi_step=8)
+    s.add_request([1, 2], SamplingParams(temperature=0.0, repetition_penalty=1.2,
+                                         max_new_tokens=6, ignore_eos=True))
+    s.run()
+    assert not eng.runs

@@ -39,7 +39,7 @@ Flags:
   --threads <usize>            (accepted, unused: the GPU grid replaces the thread pool)
   --dtype <bfloat16|float32>   --page-size <n>            --max-tokens <n>
   --max-step-tokens <n>        --chunk <n>                --max-seqs <n>
-  --ignore-eos                 --device <cuda:0>
+  --ignore-eos                 --device <cuda:0>          --multi-step <n>
 """
 
 
@@ -84,6 +84,7 @@ class Options:
         self.max_step_tokens = 2048
         self.chunk: Optional[int] = None
         self.max_seqs = 64
+        self.multi_step = 8
         self.ignore_eos = False
         self.device = "cuda:0"
         self.seed = 0
@@ -149,6 +150,8 @@ def parse_flags(flags: List[str], opt: Options) -> None:
             opt.chunk = int(value())
         elif a == "--max-seqs":
             opt.max_seqs = int(value())
+        elif a == "--multi-step":
+            opt.multi_step = int(value())
         elif a == "--ignore-eos":
             opt.ignore_eos = True
         elif a == "--device":
@@ -195,7 +198,8 @@ def _llm(model_dir: str, opt: Options, max_tokens: Optional[int] = None):
     kv = None if opt.kv_cache == "auto" else ("bfloat16" if opt.kv_cache == "bf16" else "float32")
     return LLM(model_dir, dtype=opt.dtype, device=opt.device, page_size=opt.page_size,
                max_tokens=opt.max_tokens or max_tokens, max_step_tokens=opt.max_step_tokens,
-               chunk_size=opt.chunk, max_seqs=opt.max_seqs, kv_dtype=kv)
+               chunk_size=opt.chunk, max_seqs=opt.max_seqs, kv_dtype=kv,
+               multi_step=opt.multi_step)
 
 
 # ------------------------------------------------------------------------- commands

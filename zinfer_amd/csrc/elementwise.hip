@@ -343,3 +343,38 @@ extern "C" int zf_argmax(const float* logits, int* out, void* ws, int n, int V,
                      nchunks);
   ZF_CHECK_LAUNCH();
 }
+
+// ---------------------------------------------------------------- decode metadata, one step on
+// Between two decode steps that run without the host: every request's sampled token becomes
+// its next input, its position and context length go up by one, and the slot of the new
+// position is looked up in the request's block table.  One launch per cache group; only the
+// launch with advance = 1 moves tokens, positions and lengths, the others (advance = 0) find
+// them already moved.  The host guarantees that the tables hold a page for the new position.
+__global__ void advance_decode_kernel(int* __restrict__ token_ids, int* __restrict__ positions,
+                                      int* __restrict__ ctx_len, const int* __restrict__ sampled,
+                                      int* __restrict__ slot_mapping,
+                                      const int* __restrict__ block_table, int n, int max_pages,
+                                      int page_size, int advance) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  int p = positions[i];
+  if (advance) {
+    p += 1;
+    positions[i] = p;
+    ctx_len[i] += 1;
+    token_ids[i] = sampled[i];
+  }
+  const int page = block_table[(size_t)i * max_pages + p / page_size];
+  slot_mapping[i] = page * page_size + p % page_size;
+}
+
+extern "C" int zf_advance_decode(int* token_ids, int* positions, int* ctx_len, const int* sampled,
+                                 int* slot_mapping, const int* block_table, int n, int max_pages,
+                                 int page_size, int advance, hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (max_pages <= 0 || page_size <= 0) return 1;
+  hipLaunchKernelGGL(advance_decode_kernel, dim3((n + 255) / 256), dim3(256), 0, stream,
+                     token_ids, positions, ctx_len, sampled, slot_mapping, block_table, n,
+                     max_pages, page_size, advance);
+  ZF_CHECK_LAUNCH();
+}

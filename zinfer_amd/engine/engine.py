@@ -74,29 +74,7 @@ class Engine:
         [number of wanted places, vocab] in the order of the entries and of their ``want``.
         Requests in ``end`` give back what they hold after the step.  On an error nothing
         has run and the cache is as before."""
-        spec = self.model.spec
-        seen = set()
-        wanted_len = []
-        for e in entries:
-            if e.request_id in seen:
-                raise StepError(f"request {e.request_id!r} appears twice in one step")
-            seen.add(e.request_id)
-            n = len(e.tokens)
-            if n == 0:
-                raise StepError(f"request {e.request_id!r}: a portion must hold a token")
-            for t in e.tokens:
-                if not (0 <= int(t) < spec.vocab_size):
-                    raise TokenIdOutOfBounds(f"TokenIdOutOfBounds: token {t} of request "
-                                             f"{e.request_id!r}, vocabulary {spec.vocab_size}")
-            for w in e.want:
-                if not (0 <= int(w) < n):
-                    raise StepError(f"request {e.request_id!r}: want {w} outside its {n} tokens")
-            start = self.cache.length(e.request_id) if self.cache.has_request(e.request_id) else 0
-            if start + n > spec.max_positions:
-                raise PositionOutOfBounds(
-                    f"PositionOutOfBounds: request {e.request_id!r} would reach position "
-                    f"{start + n - 1}, max_position_embeddings is {spec.max_positions}")
-            wanted_len.append((e.request_id, start + n))
+        seen, wanted_len = self._check_entries(entries)
         for rid in end:
             if rid not in seen and not self.cache.has_request(rid):
                 raise StepError(f"request {rid!r} cannot end: it is not live")
@@ -116,10 +94,89 @@ class Engine:
                 self.cache.commit(rid, new_len)
             self.steps_run += 1
         else:
-            logits = torch.empty((0, spec.vocab_size), dtype=torch.float32, device=self.device)
+            logits = torch.empty((0, self.model.spec.vocab_size), dtype=torch.float32,
+                                 device=self.device)
         for rid in end:
             self.cache.release(rid)
         return logits
+
+    def _check_entries(self, entries: Sequence[StepEntry], extra: int = 0):
+        """What can be refused before anything runs.  Returns the ids of the entries and
+        (id, length after the step plus ``extra`` further tokens) for each."""
+        spec = self.model.spec
+        seen = set()
+        wanted_len = []
+        for e in entries:
+            if e.request_id in seen:
+                raise StepError(f"request {e.request_id!r} appears twice in one step")
+            seen.add(e.request_id)
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"request {e.request_id!r}: a portion must hold a token")
+            for t in e.tokens:
+                if not (0 <= int(t) < spec.vocab_size):
+                    raise TokenIdOutOfBounds(f"TokenIdOutOfBounds: token {t} of request "
+                                             f"{e.request_id!r}, vocabulary {spec.vocab_size}")
+            for w in e.want:
+                if not (0 <= int(w) < n):
+                    raise StepError(f"request {e.request_id!r}: want {w} outside its {n} tokens")
+            start = self.cache.length(e.request_id) if self.cache.has_request(e.request_id) else 0
+            if start + n + extra > spec.max_positions:
+                raise PositionOutOfBounds(
+                    f"PositionOutOfBounds: request {e.request_id!r} would reach position "
+                    f"{start + n + extra - 1}, max_position_embeddings is {spec.max_positions}")
+            wanted_len.append((e.request_id, start + n + extra))
+        return seen, wanted_len
+
+    def decode_steps(self, entries: Sequence[StepEntry], n_steps: int,
+                     records: Optional[np.ndarray] = None) -> List[List[int]]:
+        """``n_steps`` decode steps in a row without the host between them: every entry brings
+        one token; after each step a token is drawn for every request on the device (the
+        arg-max, or with ``records`` [n_steps, requests] of ``ops.SAMPLE_ROW_DTYPE`` the
+        device sampler) and becomes the request's input of the next step.  Returns the drawn
+        tokens [n_steps][requests]; the requests then hold ``n_steps`` more tokens.  Only for
+        models whose steps replay as a graph: nothing on the host sees the steps between."""
+        from .. import ops
+        if not self.use_graphs:
+            raise StepError("decode_steps needs a model whose decode steps replay as a graph")
+        n = len(entries)
+        if n_steps < 1 or n == 0:
+            raise StepError("decode_steps: at least one step and one request")
+        if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
+            raise StepError("decode_steps: every entry brings one token and wants its logits")
+        if records is not None and records.shape != (n_steps, n):
+            raise StepError(f"decode_steps: records must be [{n_steps}, {n}]")
+        extra = n_steps - 1
+        _, wanted_len = self._check_entries(entries, extra)
+        if not self.cache.can_reserve(wanted_len):
+            raise CacheFull(f"CacheFull: {n_steps} steps need more pages or request slots than "
+                            f"are free (free pages per group: {self.cache.num_free_pages()})")
+        for rid, new_len in wanted_len:
+            if not self.cache.has_request(rid):
+                self.cache.add_request(rid)
+            self.cache.reserve(rid, new_len)
+        ctx = self._build_context(entries, bucket_pages=True, extra_tokens=extra)
+        out = self._scratch.get("decoded", (n_steps, n), torch.int32)
+        rec = None
+        if records is not None:
+            rec = torch.from_numpy(records.view(np.uint8).reshape(n_steps, -1).copy()) \
+                .to(self.device)
+        for s in range(n_steps):
+            if s:
+                for g, tables in enumerate(ctx.kv):
+                    ops.advance_decode(ctx.token_ids, ctx.positions, ctx.ctx_len, out[s - 1],
+                                       tables.slot_mapping, tables.block_table, self.page_size,
+                                       advance=(g == 0))
+            logits = self._forward_graphed(ctx)
+            if rec is None:
+                ops.argmax(logits, out[s])
+            else:
+                ops.sample_topk(logits, rec[s], out[s])
+        tokens = out.tolist()
+        for rid, new_len in wanted_len:
+            self.cache.commit(rid, new_len)
+        self.steps_run += n_steps
+        return tokens
 
     def _generations(self) -> tuple:
         from .. import ops
@@ -178,7 +235,10 @@ class Engine:
         return out.tolist()
 
     # ------------------------------------------------------------------ metadata
-    def _build_context(self, entries: Sequence[StepEntry], bucket_pages: bool = False) -> StepContext:
+    def _build_context(self, entries: Sequence[StepEntry], bucket_pages: bool = False,
+                       extra_tokens: int = 0) -> StepContext:
+        """Packs the step's metadata and copies it to the device.  ``extra_tokens``: the block
+        tables (and the bound on the context) also cover this many tokens after the step."""
         ps = self.page_size
         n_seqs = len(entries)
         q_lens = [len(e.tokens) for e in entries]
@@ -193,8 +253,8 @@ class Engine:
             q_start.append(q_start[-1] + n)
         n_want = len(want_rows)
         n_groups = len(self.cache.groups)
-        max_pages = max((c + ps - 1) // ps for c in ctx_lens)
-        max_ctx = max(ctx_lens)
+        max_pages = max((c + extra_tokens + ps - 1) // ps for c in ctx_lens)
+        max_ctx = max(ctx_lens) + extra_tokens
         if bucket_pages:      # a fixed table width (and context bound) per captured graph
             b = self.GRAPH_PAGE_BUCKET
             max_pages = (max_pages + b - 1) // b * b

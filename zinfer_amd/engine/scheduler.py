@@ -13,6 +13,10 @@ never run out; portions, the budget and what happens when pages run out are this
   request is preempted: its pages are freed, it keeps its generated tokens and its random
   stream, goes to the front of the waiting queue and later recomputes prompt + generated;
 * a request that cannot fit even alone raises CacheFull.
+
+When every running request decodes and nobody waits, up to ``multi_step`` decode steps run in
+a row on the device without the host between them; tokens that a request drew after its
+end-of-sequence id are thrown away, which costs at most ``multi_step - 1`` steps of that row.
 """
 from __future__ import annotations
 
@@ -59,7 +63,7 @@ class PlannedEntry:
 
 class Scheduler:
     def __init__(self, engine, *, max_step_tokens: int = 2048, chunk_size: Optional[int] = None,
-                 max_seqs: int = 64, eos_token_ids: Sequence[int] = ()):
+                 max_seqs: int = 64, eos_token_ids: Sequence[int] = (), multi_step: int = 8):
         if max_step_tokens < 1 or max_seqs < 1:
             raise ValueError("max_step_tokens and max_seqs must be at least 1")
         self.engine = engine
@@ -72,7 +76,9 @@ class Scheduler:
         self.running: List[Request] = []           # in admission order
         self.finished: Dict[object, Request] = {}
         self._next_id = 0
-        self.n_steps = 0
+        self.multi_step = multi_step        # most decode steps in a row without the host
+        self.n_steps = 0                    # engine steps so far
+        self.last_steps = 0                 # engine steps the last call of step() ran
         self.n_preemptions = 0
 
     # ------------------------------------------------------------------ requests
@@ -174,7 +180,11 @@ class Scheduler:
     # ------------------------------------------------------------------ one iteration
     def step(self) -> List[Request]:
         """Plans, runs one step, samples, finishes.  Returns the requests finished by it."""
+        k = self._multi_step_count()
+        if k >= 2:
+            return self._decode_multi(k)
         planned = self.plan()
+        self.last_steps = 1 if planned else 0
         if not planned:
             return []
         entries = []
@@ -189,20 +199,70 @@ class Scheduler:
         for p in planned:
             p.request.n_computed += p.n_tokens
         for p, tok in zip(sampling, next_tokens):
-            req = p.request
-            reason = None
-            if not req.params.ignore_eos and (tok in self.eos_token_ids
-                                              or tok in req.params.stop_token_ids):
-                reason = "eos"                    # not stored, not counted
-            else:
-                req.generated.append(tok)
-                if len(req.generated) >= req.params.max_new_tokens:
-                    reason = "length"
-                elif len(req.prompt) + len(req.generated) > self.engine.model.spec.max_positions:
-                    reason = "context"
-            if reason is not None:
-                self._finish(req, reason)
-                done.append(req)
+            if self._accept(p.request, tok):
+                done.append(p.request)
+        return done
+
+    def _accept(self, req: Request, tok: int) -> bool:
+        """Takes a drawn token into the request; True if the request has finished by it."""
+        reason = None
+        if not req.params.ignore_eos and (tok in self.eos_token_ids
+                                          or tok in req.params.stop_token_ids):
+            reason = "eos"                    # not stored, not counted
+        else:
+            req.generated.append(tok)
+            if len(req.generated) >= req.params.max_new_tokens:
+                reason = "length"
+            elif len(req.prompt) + len(req.generated) > self.engine.model.spec.max_positions:
+                reason = "context"
+        if reason is not None:
+            self._finish(req, reason)
+        return reason is not None
+
+    def _multi_step_count(self) -> int:
+        """How many decode steps may run in a row on the device: every running request must
+        decode, be sampled on the device without penalties and have room for that many tokens
+        (in its length limits and in free pages), and nobody may wait for admission."""
+        if self.multi_step < 2 or self.waiting or not self.running \
+                or not getattr(self.engine, "use_graphs", False) \
+                or len(self.running) > self.max_step_tokens:
+            return 0
+        k = self.multi_step
+        max_pos = self.engine.model.spec.max_positions
+        for req in self.running:
+            sp = req.params
+            if req.pending != 1 or not req.generated or sp.has_penalties \
+                    or not (sp.greedy or 1 <= sp.top_k <= 1024):
+                return 0
+            k = min(k, sp.max_new_tokens - len(req.generated),
+                    max_pos - (len(req.prompt) + len(req.generated)) + 1)
+        while k >= 2 and not self.cache.can_reserve(
+                [(req.id, req.n_computed + k) for req in self.running]):
+            k //= 2
+        return k if k >= 2 else 0
+
+    def _decode_multi(self, k: int) -> List[Request]:
+        from ..ops import SAMPLE_ROW_DTYPE
+        reqs = list(self.running)
+        entries = [StepEntry(r.id, [r.generated[-1]], [0]) for r in reqs]
+        records = None
+        if not all(r.params.greedy for r in reqs):
+            records = np.zeros((k, len(reqs)), dtype=SAMPLE_ROW_DTYPE)
+            for i, r in enumerate(reqs):
+                sp = r.params
+                for s in range(k):
+                    records[s, i] = (1.0, 1.0, 0.0, 1, 0.0) if sp.greedy else \
+                        (sp.temperature, sp.top_p, sp.min_p, sp.top_k, r.rng.float64())
+        tokens = self.engine.decode_steps(entries, k, records)
+        self.n_steps += k
+        self.last_steps = k
+        done: List[Request] = []
+        for i, r in enumerate(reqs):
+            r.n_computed += k
+            for s in range(k):
+                if self._accept(r, tokens[s][i]):
+                    done.append(r)
+                    break
         return done
 
     def _finish(self, req: Request, reason: str) -> None:

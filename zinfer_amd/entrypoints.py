@@ -22,10 +22,11 @@ class LLM:
                  page_size: int = 16, max_tokens: Optional[int] = None,
                  num_pages: Optional[int] = None, max_step_tokens: int = 2048,
                  chunk_size: Optional[int] = None, max_seqs: int = 64,
-                 kv_dtype: Optional[str] = None):
+                 kv_dtype: Optional[str] = None, multi_step: int = 8):
         """``max_tokens`` (or ``num_pages``) sizes the cache pool; by default the pool holds
         ``max_seqs`` requests of ``max_position_embeddings`` tokens, capped at 1/2 of the free
-        device memory."""
+        device memory.  ``multi_step``: the most decode steps that run in a row on the device
+        without the host between them (1: the host sees every step)."""
         self.config, self.model = load_model(model_dir, dtype, device)
         spec = self.model.spec
         if num_pages is None:
@@ -37,7 +38,8 @@ class LLM:
                              max_requests=max_seqs,
                              kv_dtype=parse_dtype(kv_dtype) if kv_dtype else None)
         self.scheduler_options = dict(max_step_tokens=max_step_tokens, chunk_size=chunk_size,
-                                      max_seqs=max_seqs, eos_token_ids=spec.eos_token_ids)
+                                      max_seqs=max_seqs, eos_token_ids=spec.eos_token_ids,
+                                      multi_step=multi_step)
 
     def _default_max_tokens(self, spec, page_size: int, max_seqs: int) -> int:
         want = max_seqs * spec.max_positions

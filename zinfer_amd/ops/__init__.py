@@ -148,6 +148,30 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     _check(lib.zf_argmax(_ptr(logits), _ptr(out), _ptr(ws), n, V, _stream()), "argmax")
 
 
+def advance_decode(token_ids: torch.Tensor, positions: torch.Tensor, ctx_len: torch.Tensor,
+                   sampled: torch.Tensor, slot_mapping: torch.Tensor, block_table: torch.Tensor,
+                   page_size: int, advance: bool) -> None:
+    """One decode step on, on the device: with ``advance`` token_ids = sampled, positions and
+    ctx_len + 1; always slot_mapping[i] = block_table[i, p // page_size] * page_size +
+    p % page_size at the (new) position p.  The caller guarantees that the table holds a page
+    there."""
+    _need_gpu(token_ids, positions, ctx_len, sampled, slot_mapping, block_table)
+    for t, name in ((token_ids, "token_ids"), (positions, "positions"), (ctx_len, "ctx_len"),
+                    (sampled, "sampled"), (slot_mapping, "slot_mapping"),
+                    (block_table, "block_table")):
+        _i32(t, name)
+    n = token_ids.shape[0]
+    if block_table.dim() != 2 or block_table.shape[0] != n or not block_table.is_contiguous() \
+            or any(t.shape != (n,) for t in (positions, ctx_len, sampled, slot_mapping)):
+        raise KernelUnavailable("advance_decode: int32 [n] vectors and a contiguous [n, pages] "
+                                "block table")
+    lib = build.load("elementwise")
+    _check(lib.zf_advance_decode(_ptr(token_ids), _ptr(positions), _ptr(ctx_len), _ptr(sampled),
+                                 _ptr(slot_mapping), _ptr(block_table), n, block_table.shape[1],
+                                 int(page_size), 1 if advance else 0, _stream()),
+           "advance_decode")
+
+
 # ------------------------------------------------------------------------- work buffers
 _workspaces = {}
 _workspace_generation = 0
