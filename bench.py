@@ -175,6 +175,8 @@ def check_fp32(llm, cfg, raw, args) -> dict:
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--multi-step", type=int, default=8,
+                    help="most decode steps in a row on the device without the host between")
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
@@ -213,7 +215,8 @@ def main() -> int:
     llm.engine = Engine(model, page_size=page, num_pages=(tokens + page - 1) // page + 8,
                         max_requests=max_batch)
     llm.scheduler_options = dict(max_step_tokens=max(2048, args.prompt_len), chunk_size=None,
-                                 max_seqs=max_batch, eos_token_ids=())
+                                 max_seqs=max_batch, eos_token_ids=(),
+                                 multi_step=args.multi_step)
     build_s = time.perf_counter() - t_build
 
     pre_s = run_prefill(llm, cfg, args.prefill_tokens, args.seed + 1)
