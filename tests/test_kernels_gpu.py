@@ -183,6 +183,50 @@ def test_norm_gemm(M, N, K, kind):
     assert rel_err(got, want) <= 2.0 ** -7
 
 
+@pytest.mark.parametrize("M", [1, 7, 16])
+@pytest.mark.parametrize("H,K1,N2", [(4096, 12288, 6144), (1088, 320, 4160), (64, 64, 128)])
+@pytest.mark.parametrize("kind", ["bf16", "f32", "swiglu"])
+def test_gemm_emit_then_given(M, H, K1, N2, kind):
+    """The residual sum whose epilogue leaves bfloat16(x * gain) and partial sums of x^2 for
+    the norm that follows, and the product that takes them, against sum, norm and product
+    in 64-bit.  Tokens of different scale: a wrong row's 1 / rms would show."""
+    ops = _ops()
+    a = _rand((M, K1), torch.bfloat16, 60, 1.0)
+    w1 = _rand((H, K1), torch.bfloat16, 61, 0.05)
+    base = _rand((M, H), torch.float32, 62, 2.0) * (1 + torch.arange(M).float()[:, None])
+    gain = 1 + 0.1 * _rand((H,), torch.float32, 63)
+    w2 = _rand((N2, H), torch.bfloat16, 64, 0.05)
+    eps = 1e-5
+    if ops.norm_emit_plan(M, H, K1, w1.to(DEV), True) is None:
+        pytest.skip("this size is not covered: the norm runs on its own")
+    x = base.double() + a.double() @ w1.double().T
+    res = base.clone().to(DEV)
+    xg = torch.full((M, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    sq = torch.full((H // 16, 16), float("nan"), dtype=torch.float32, device=DEV)
+    ops.gemm_emit(a.to(DEV), ops.pretile_weight(w1.to(DEV)), res, gain.to(DEV), xg, sq)
+    assert rel_err(res, x) <= tol(torch.float32)
+    assert rel_err(xg, x * gain.double()) <= tol(torch.bfloat16)
+    assert rel_err(sq.sum(0)[:M], (x * x).sum(-1)) <= 1e-5
+    assert torch.equal(sq[:, M:], torch.zeros_like(sq[:, M:]))
+    normed = torch.empty((M, H), dtype=torch.float64)
+    ref.rmsnorm(x, gain, eps, normed)
+    if kind == "swiglu":
+        I = N2 // 2
+        wi = ops.interleave_gate_up(w2[:I].to(DEV), w2[I:].to(DEV))
+        want = torch.empty((M, I), dtype=torch.float64)
+        ref.gemm_swiglu(normed, wi.cpu(), want)
+        got = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.gemm_given(xg, sq, eps, ops.pretile_weight(wi), got, swiglu=True)
+    else:
+        if ops.norm_gemm_plan(M, N2, H, w2.to(DEV), True) is None:
+            pytest.skip("the second product uses a split over workgroups")
+        want = normed @ w2.double().T
+        got = torch.full((M, N2), float("nan"), dtype=torch.bfloat16 if kind == "bf16"
+                         else torch.float32, device=DEV)
+        ops.gemm_given(xg, sq, eps, ops.pretile_weight(w2.to(DEV)), got)
+    assert rel_err(got, want) <= 2.0 ** -7
+
+
 @pytest.mark.parametrize("a_dtype", DTYPES)
 def test_gemm_accumulate_and_one_hot(a_dtype):
     """out += a w^T in 32-bit; a one-hot row picks a column of W (the reference's

@@ -129,7 +129,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
+  return pack_bf16x2(lo, hi);
 }
 
 // keeps elements [n_lo, n_hi) of the 4 bfloat16 in v (element 0 in the low bits), zeroes the rest

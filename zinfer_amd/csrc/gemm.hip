@@ -352,6 +352,25 @@ extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, i
   }
 }
 
+enum { NORM_NONE = 0, NORM_FOLD = 1, NORM_GIVEN = 2 };
+
+// What the weight-streaming kernel needs to know of an RMSNorm around it.
+//   before the product: NORM_FOLD   gain, eps: the rows come as the 32-bit residual stream;
+//                       NORM_GIVEN  eps, sq_in [sq_groups][16]: the rows come as
+//                                   bfloat16(x * gain) with the sums of x^2 per 16 columns,
+//                                   as the kernel that produced x left them (EMIT);
+//   after it (EMIT, with the residual epilogue): gain_out, xg_out [M, N], sq_out [N / 16][16]
+//                                   for the norm that reads the sum next.
+struct SkinnyNorm {
+  const float* gain;
+  float eps;
+  const float* sq_in;
+  int sq_groups;
+  const float* gain_out;
+  bf16_t* xg_out;
+  float* sq_out;
+};
+
 // ---------------------------------------------------------------- small M: weight streaming
 // For M <= 64 the product is bound by reading W once from HBM.  A workgroup owns 16 * RG rows
 // of W (output features) and all M tokens; its 8 waves (times KSPLIT workgroups along
@@ -369,12 +388,15 @@ extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, i
 // when there is no split over workgroups), and the epilogue scales each token's sums by
 // inv = 1 / sqrt(mean(x^2) + eps), all in 32-bit  (n = x w / sqrt(mean(x^2) + eps),
 // src/kernel/core/cpu.zig:38-48 of the reference).
-template <int MT, int RG, int EPI, bool WT, bool NORM>
-__global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
+template <int MT, int RG, int EPI, bool WT, int NORM, int NW = 8, bool EMIT = false>
+__global__ __launch_bounds__(NW * 64) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
-    int N, int K, const float* __restrict__ gain, float eps) {
-  __shared__ float part[8][RG * MT][64][4];
-  __shared__ float ssum[8][MT][16];
+    int N, int K, SkinnyNorm nrm) {
+  constexpr int NSS = NORM == NORM_GIVEN ? NW * 4 : NW;
+  __shared__ float part[NW][RG * MT][64][4];
+  __shared__ float ssum[NSS][MT][16];
+  const float* __restrict__ gain = nrm.gain;
+  const float eps = nrm.eps;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int n0 = blockIdx.x * (16 * RG);
   const int g = lane / 16;
@@ -392,9 +414,14 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
     arow[t] = A + (size_t)min(t * 16 + lane % 16, M - 1) * K;
     xrow[t] = (const float*)A + (size_t)min(t * 16 + lane % 16, M - 1) * K;
   }
+  // lanes of tokens beyond M load nothing and feed zeros
+  bool tok[MT];
   float ss[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) ss[t] = 0.f;
+  for (int t = 0; t < MT; ++t) {
+    tok[t] = t * 16 + lane % 16 < M;
+    ss[t] = 0.f;
+  }
 
   f32x4_t acc[RG][MT];
 #pragma unroll
@@ -403,9 +430,9 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
     for (int t = 0; t < MT; ++t) acc[r][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
   const u32x4_t zero = u32x4_t{0, 0, 0, 0};
-  const int kstride = 512 * gridDim.y;
-  int k0 = (blockIdx.y * 8 + wave) * 64;
-  if (WT && !NORM && RG * MT == 1) {
+  const int kstride = NW * 64 * gridDim.y;
+  int k0 = (blockIdx.y * NW + wave) * 64;
+  if (WT && NORM != NORM_FOLD && RG * MT == 1) {
     // one row group and up to 16 tokens per wave: take 4 k-steps at once so that more loads
     // are in flight (pre-tiled weights need no bounds checks; K % 64 == 0); measured to help
     // only in this case
@@ -423,8 +450,8 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
         }
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
-          a0[u][t] = *(const u32x4_t*)(arow[t] + kk + g * 16);
-          a1[u][t] = *(const u32x4_t*)(arow[t] + kk + g * 16 + 8);
+          a0[u][t] = tok[t] ? *(const u32x4_t*)(arow[t] + kk + g * 16) : zero;
+          a1[u][t] = tok[t] ? *(const u32x4_t*)(arow[t] + kk + g * 16 + 8) : zero;
         }
       }
 #pragma unroll
@@ -455,7 +482,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
       }
     }
     u32x4_t a0[MT], a1[MT];
-    if (NORM) {       // K % 64 == 0 here: 16 floats of x and of the gain per lane
+    if (NORM == NORM_FOLD) {       // K % 64 == 0 here: 16 floats of x and of the gain per lane
       float4 gv[4];
 #pragma unroll
       for (int c = 0; c < 4; ++c) gv[c] = *(const float4*)(gain + k + 4 * c);
@@ -463,15 +490,14 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
       for (int t = 0; t < MT; ++t) {
         float4 xv[4];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) xv[c] = *(const float4*)(xrow[t] + k + 4 * c);
+        for (int c = 0; c < 4; ++c)
+          xv[c] = tok[t] ? *(const float4*)(xrow[t] + k + 4 * c) : float4{0.f, 0.f, 0.f, 0.f};
         uint32_t pk[8];
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
           ss[t] += xv[c].x * xv[c].x + xv[c].y * xv[c].y + xv[c].z * xv[c].z + xv[c].w * xv[c].w;
-          pk[2 * c] = (uint32_t)float_to_bf16(xv[c].x * gv[c].x) |
-                      ((uint32_t)float_to_bf16(xv[c].y * gv[c].y) << 16);
-          pk[2 * c + 1] = (uint32_t)float_to_bf16(xv[c].z * gv[c].z) |
-                          ((uint32_t)float_to_bf16(xv[c].w * gv[c].w) << 16);
+          pk[2 * c] = pack_bf16x2(xv[c].x * gv[c].x, xv[c].y * gv[c].y);
+          pk[2 * c + 1] = pack_bf16x2(xv[c].z * gv[c].z, xv[c].w * gv[c].w);
         }
         a0[t] = u32x4_t{pk[0], pk[1], pk[2], pk[3]};
         a1[t] = u32x4_t{pk[4], pk[5], pk[6], pk[7]};
@@ -479,8 +505,8 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
     } else {
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
-        a0[t] = (k < K) ? *(const u32x4_t*)(arow[t] + k) : zero;
-        a1[t] = (k + 8 < K) ? *(const u32x4_t*)(arow[t] + k + 8) : zero;
+        a0[t] = (tok[t] && k < K) ? *(const u32x4_t*)(arow[t] + k) : zero;
+        a1[t] = (tok[t] && k + 8 < K) ? *(const u32x4_t*)(arow[t] + k + 8) : zero;
       }
     }
 #pragma unroll
@@ -499,7 +525,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
     for (int t = 0; t < MT; ++t)
 #pragma unroll
       for (int e = 0; e < 4; ++e) part[wave][r * MT + t][lane][e] = acc[r][t][e];
-  if (NORM) {
+  if (NORM == NORM_FOLD) {
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       float v = ss[t];
@@ -508,23 +534,31 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
       if (lane < 16) ssum[wave][t][lane] = v;
     }
   }
+  if (NORM == NORM_GIVEN) {
+    // the producer of the rows left sums of squares per 16 columns: [groups][16 tokens];
+    // thread (p, j) adds groups p, p + NSS, ... of token j, the rest follows in order of p
+    const int j = tid % 16, p = tid / 16;
+    float v = 0.f;
+    for (int gidx = p; gidx < nrm.sq_groups; gidx += NSS) v += nrm.sq_in[gidx * 16 + j];
+    ssum[p][0][j] = v;
+  }
   __syncthreads();
-  // the token's 1 / sqrt(mean(x^2) + eps): the waves' partial sums in wave order
+  // the token's 1 / sqrt(mean(x^2) + eps): the partial sums in a fixed order
   auto inv_rms = [&](int t, int j) {
-    if (!NORM) return 1.0f;
+    if (NORM == NORM_NONE) return 1.0f;
     float tot = 0.f;
 #pragma unroll
-    for (int w = 0; w < 8; ++w) tot += ssum[w][t][j];
+    for (int w = 0; w < NSS; ++w) tot += ssum[w][t][j];
     return 1.0f / sqrtf(tot / (float)K + eps);
   };
   if (EPI == EPI_SWIGLU) {
     // row groups alternate gate / up: the pair (2 p, 2 p + 1) gives 16 outputs per token
-    for (int item = tid; item < (RG / 2) * MT * 64; item += 512) {
+    for (int item = tid; item < (RG / 2) * MT * 64; item += NW * 64) {
       const int pt = item / 64, l = item % 64;
       const int p = pt / MT, t = pt % MT;
       float g[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int w = 0; w < 8; ++w)
+      for (int w = 0; w < NW; ++w)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           g[e] += part[w][(2 * p) * MT + t][l][e];
@@ -544,16 +578,17 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
     }
     return;
   }
-  for (int item = tid; item < RG * MT * 64; item += 512) {
+  for (int item = tid; item < RG * MT * 64; item += NW * 64) {
     const int rt = item / 64, l = item % 64;
     const int r = rt / MT, t = rt % MT;
     float s[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int w = 0; w < 8; ++w)
+    for (int w = 0; w < NW; ++w)
 #pragma unroll
       for (int e = 0; e < 4; ++e) s[e] += part[w][rt][l][e];
     // D[i][j]: i = 4 * (l / 16) + e is the W row (output feature), j = l % 16 the token
     const int token = t * 16 + l % 16;
+    float sq = 0.f;
     if (token < M) {
       const float inv = inv_rms(t, l % 16);
 #pragma unroll
@@ -566,15 +601,28 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(
             ((float*)Cv)[((size_t)blockIdx.y * M + token) * N + n] = s[e];   // workspace
           } else {
             const size_t off = (size_t)token * N + n;
-            if (EPI == EPI_STORE_BF16)
+            if (EPI == EPI_STORE_BF16) {
               ((bf16_t*)Cv)[off] = float_to_bf16(s[e]);
-            else if (EPI == EPI_STORE_F32)
+            } else if (EPI == EPI_STORE_F32) {
               ((float*)Cv)[off] = s[e];
-            else
-              ((float*)Cv)[off] += s[e];
+            } else {
+              const float v = ((float*)Cv)[off] + s[e];
+              ((float*)Cv)[off] = v;
+              if (EMIT) {   // what the RMSNorm after this sum needs: v * gain, and v^2
+                nrm.xg_out[off] = float_to_bf16(v * nrm.gain_out[n]);
+                sq += v * v;
+              }
+            }
           }
         }
       }
+    }
+    if (EMIT) {
+      // the 16 columns of this row group: 4 per lane, lanes l, l + 16, l + 32, l + 48 of a
+      // token; every item is a whole wave here (RG * MT * 64 items, NW * 64 threads)
+      sq += __shfl_xor(sq, 16, 64);
+      sq += __shfl_xor(sq, 32, 64);
+      if (l < 16) nrm.sq_out[(size_t)(n0 / 16 + r) * 16 + l] = sq;
     }
   }
 }
@@ -594,28 +642,34 @@ __global__ void skinny_reduce_kernel(const float* __restrict__ ws, void* __restr
     ((float*)Cv)[i] += s;
 }
 
-template <int MT, int RG, bool WT, bool NORM = false>
+template <int MT, int RG, bool WT, int NORM = NORM_NONE, bool EMIT = false>
 static int launch_skinny(const void* A, const void* W, void* C, void* ws, int M, int N, int K,
-                         int epi, int ksplit, hipStream_t stream, const float* gain = nullptr,
-                         float eps = 0.f) {
-  const dim3 grid((N + 16 * RG - 1) / (16 * RG), ksplit), block(512);
+                         int epi, int ksplit, hipStream_t stream, SkinnyNorm nrm = SkinnyNorm{}) {
+  constexpr int NW = 8;
+  const dim3 grid((N + 16 * RG - 1) / (16 * RG), ksplit), block(NW * 64);
   void* dst = ksplit > 1 ? ws : C;
-  if (NORM && (ksplit != 1 || epi == EPI_ACC_F32)) return -3;
+  if (NORM != NORM_NONE && (ksplit != 1 || epi == EPI_ACC_F32)) return -3;
+  if (EMIT) {
+    if (ksplit != 1 || epi != EPI_ACC_F32) return -3;
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_ACC_F32, WT, NORM_NONE, NW, true>), grid,
+                       block, 0, stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K, nrm);
+    return (int)hipGetLastError();
+  }
   if (epi == EPI_SWIGLU) {
     if (RG < 2 || ksplit != 1 || N % 32 != 0) return -3;
-    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, (RG < 2 ? 2 : RG), EPI_SWIGLU, WT, NORM>), grid,
-                       block, 0, stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K, gain, eps);
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, (RG < 2 ? 2 : RG), EPI_SWIGLU, WT, NORM, NW>), grid,
+                       block, 0, stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K, nrm);
     return (int)hipGetLastError();
   }
   if (epi == EPI_STORE_BF16)
-    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_STORE_BF16, WT, NORM>), grid, block, 0,
-                       stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K, gain, eps);
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_STORE_BF16, WT, NORM, NW>), grid, block, 0,
+                       stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K, nrm);
   else if (epi == EPI_STORE_F32)
-    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_STORE_F32, WT, NORM>), grid, block, 0,
-                       stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K, gain, eps);
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_STORE_F32, WT, NORM, NW>), grid, block, 0,
+                       stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K, nrm);
   else
-    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_ACC_F32, WT, false>), grid, block, 0,
-                       stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K, gain, eps);
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_ACC_F32, WT, NORM_NONE, NW>), grid, block, 0,
+                       stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K, nrm);
   if (ksplit > 1) {
     const size_t mn = (size_t)M * N;
     const unsigned blocks = (unsigned)((mn + 255) / 256);
@@ -641,8 +695,8 @@ extern "C" int zf_gemm_bf16_skinny(const void* A, const void* W, void* C, void* 
   if (M <= 0 || N <= 0) return 0;
   if (K % 8 != 0 || M > 64 || ksplit < 1 || ksplit > 16 || (ksplit > 1 && ws == nullptr))
     return -3;
-  if (w_tiled && (N % (16 * rg) != 0 || K % 64 != 0)) return -3;
   const int mt = (M + 15) / 16;
+  if (w_tiled && (N % (16 * rg) != 0 || K % 64 != 0)) return -3;
 #define ZF_SK(MT, RG)                                                                         \
   return w_tiled ? launch_skinny<MT, RG, true>(A, W, C, ws, M, N, K, epi, ksplit, stream)     \
                  : launch_skinny<MT, RG, false>(A, W, C, ws, M, N, K, epi, ksplit, stream)
@@ -660,13 +714,53 @@ extern "C" int zf_norm_gemm_bf16_skinny(const float* X, const float* gain, float
                                         void* C, int M, int N, int K, int epi, int rg,
                                         hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K % 64 != 0 || N % (16 * rg) != 0 || epi == EPI_ACC_F32) return -3;
   const int mt = (M + 15) / 16;
+  if (M > 64 || K % 64 != 0 || N % (16 * rg) != 0 || epi == EPI_ACC_F32) return -3;
+  SkinnyNorm nrm{};
+  nrm.gain = gain;
+  nrm.eps = eps;
 #define ZF_NSK(MT, RG) \
-  return launch_skinny<MT, RG, true, true>(X, W, C, nullptr, M, N, K, epi, 1, stream, gain, eps)
+  return launch_skinny<MT, RG, true, NORM_FOLD>(X, W, C, nullptr, M, N, K, epi, 1, stream, nrm)
   if (rg == 1) { if (mt == 1) ZF_NSK(1, 1); if (mt == 2) ZF_NSK(2, 1); if (mt == 3) ZF_NSK(3, 1); ZF_NSK(4, 1); }
   if (rg == 2) { if (mt == 1) ZF_NSK(1, 2); if (mt == 2) ZF_NSK(2, 2); if (mt == 3) ZF_NSK(3, 2); ZF_NSK(4, 2); }
   if (rg == 4) { if (mt == 1) ZF_NSK(1, 4); if (mt == 2) ZF_NSK(2, 4); if (mt == 3) ZF_NSK(3, 4); ZF_NSK(4, 4); }
 #undef ZF_NSK
+  return -4;
+}
+
+// The same product for rows that come already multiplied by the norm's gain, as bfloat16
+// XG [M <= 16, K], with the sums of squares of the un-normed rows per 16 columns,
+// sq [sq_groups][16] (token j of group g at sq[g * 16 + j]), as zf_gemm_bf16_skinny_emit
+// leaves them: out = (XG W^T) / sqrt(sum_g sq[g][token] / K + eps).
+extern "C" int zf_gemm_bf16_skinny_given(const void* XG, const float* sq, int sq_groups, float eps,
+                                         const void* W, void* C, int M, int N, int K, int epi,
+                                         int rg, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 16 || K % 64 != 0 || N % (16 * rg) != 0 || epi == EPI_ACC_F32 || sq_groups < 1)
+    return -3;
+  SkinnyNorm nrm{};
+  nrm.eps = eps;
+  nrm.sq_in = sq;
+  nrm.sq_groups = sq_groups;
+  if (rg == 1) return launch_skinny<1, 1, true, NORM_GIVEN>(XG, W, C, nullptr, M, N, K, epi, 1, stream, nrm);
+  if (rg == 2) return launch_skinny<1, 2, true, NORM_GIVEN>(XG, W, C, nullptr, M, N, K, epi, 1, stream, nrm);
+  if (rg == 4) return launch_skinny<1, 4, true, NORM_GIVEN>(XG, W, C, nullptr, M, N, K, epi, 1, stream, nrm);
+  return -4;
+}
+
+// C += A W^T (C the float32 residual stream [M <= 16, N], W pre-tiled) and, for the RMSNorm
+// that reads C next: xg_out [M, N] = bfloat16(C * gain_out), sq_out [N / 16][16] = sums of
+// C^2 over each group of 16 columns (tokens beyond M: 0).
+extern "C" int zf_gemm_bf16_skinny_emit(const void* A, const void* W, float* C,
+                                        const float* gain_out, void* xg_out, float* sq_out, int M,
+                                        int N, int K, int rg, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 16 || K % 64 != 0 || N % (16 * rg) != 0) return -3;
+  SkinnyNorm nrm{};
+  nrm.gain_out = gain_out;
+  nrm.xg_out = (bf16_t*)xg_out;
+  nrm.sq_out = sq_out;
+  if (rg == 1) return launch_skinny<1, 1, true, NORM_NONE, true>(A, W, C, nullptr, M, N, K, EPI_ACC_F32, 1, stream, nrm);
+  if (rg == 2) return launch_skinny<1, 2, true, NORM_NONE, true>(A, W, C, nullptr, M, N, K, EPI_ACC_F32, 1, stream, nrm);
   return -4;
 }

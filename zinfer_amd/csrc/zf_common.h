@@ -13,12 +13,19 @@ __device__ __forceinline__ float bf16_to_float(bf16_t b) {
   return __uint_as_float(((uint32_t)b) << 16);
 }
 
-// round to nearest even: (bits + 0x7fff + lsb) >> 16 (bfloat16.zig:8-13); a NaN stays a NaN
+// round to nearest even, (bits + 0x7fff + lsb) >> 16 (bfloat16.zig:8-13), a NaN stays a NaN:
+// gfx950 has an instruction for it (v_cvt_pk_bf16_f32), which the cast below becomes; it
+// gives the same 16 bits as the formula for every one of the 2^32 inputs
 __device__ __forceinline__ bf16_t float_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
+  const __bf16 b = (__bf16)f;
+  return *(const bf16_t*)&b;
+}
+// two values in one register, `lo` in the low half
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef __bf16 bf16x2_native __attribute__((ext_vector_type(2)));
+  typedef float floatx2_native __attribute__((ext_vector_type(2)));
+  const bf16x2_native v = __builtin_convertvector(floatx2_native{lo, hi}, bf16x2_native);
+  return *(const uint32_t*)&v;
 }
 
 template <typename T> __device__ __forceinline__ float load_as_float(const T* p);

@@ -67,6 +67,13 @@ class StepContext:
     slots: List[int]
     n_single: int = 0             # sequences with exactly one token in this step
     meta_offset: int = 0          # address of the packed metadata (part of a graph's key)
+    wants_all_rows: bool = False  # want_rows is 0, 1, ..., n_tokens - 1
+    # A part that adds into the residual stream may, in the same kernel, leave what the norm
+    # reading the stream next needs (``Linear.forward(..., step=step)``): ``norm_after`` is
+    # that norm (set by whoever calls the part), ``norm_ready`` what was left for it.
+    norm_after: object = None
+    norm_after_block: object = None   # the norm that reads the stream first after this block
+    norm_ready: object = None
     _scratch: Scratch = None
 
     def scratch(self, name: str, shape, dtype) -> torch.Tensor:

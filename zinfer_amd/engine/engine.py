@@ -323,6 +323,7 @@ class Engine:
             max_ctx_len=max_ctx, q_lens=q_lens, ctx_lens=ctx_lens, slots=slots,
             meta_offset=self._meta_dev.data_ptr() if self._meta_dev is not None else 0,
             n_single=sum(1 for n in q_lens if n == 1),
+            wants_all_rows=want_rows == list(range(T)),
             _scratch=self._scratch)
 
     def _upload(self, host: np.ndarray) -> torch.Tensor:

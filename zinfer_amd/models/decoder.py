@@ -76,18 +76,33 @@ class DecoderModel:
         T = step.n_tokens
         x = step.scratch("residual", (T, s.hidden_size), torch.float32)
         ops.embed(self.embedding, step.token_ids, x)
+        lazy_final = isinstance(self.final_norm, RmsNorm) and x.is_cuda \
+            and self.ctx.compute_dtype == torch.bfloat16
+        step.norm_ready = None
         for pos, e in enumerate(s.schedule):
+            # the norm that reads the stream after this block: the next block's first, or the
+            # final norm when every row goes to the head as it lies
+            if pos + 1 < len(s.schedule):
+                after = getattr(self.blocks[s.schedule[pos + 1].layer], "entry_norm", None)
+            else:
+                after = self.final_norm if lazy_final and step.wants_all_rows else None
+            step.norm_after_block = after
             self.blocks[e.layer].forward(x, step, caches[pos])
+        ready, step.norm_ready, step.norm_after_block = step.norm_ready, None, None
         n_rows = step.n_want
         logits = step.scratch("logits", (n_rows, s.vocab_size), torch.float32)
         if n_rows == 0:
             return logits
-        rows = step.scratch("want_rows", (n_rows, s.hidden_size), torch.float32)
-        ops.gather_rows(x, step.want_rows, rows)
+        if step.wants_all_rows:
+            rows = x
+        else:
+            ready = None
+            rows = step.scratch("want_rows", (n_rows, s.hidden_size), torch.float32)
+            ops.gather_rows(x, step.want_rows, rows)
         make = lambda: step.scratch("final_normed", (n_rows, s.hidden_size), self.ctx.act_dtype)
-        if isinstance(self.final_norm, RmsNorm) and rows.is_cuda \
-                and self.ctx.compute_dtype == torch.bfloat16:
-            self.head.forward(LazyRmsNorm(self.final_norm, rows, make), logits)   # folded if it can be
+        if lazy_final:
+            given = ready if ready is not None and ready.fits(self.final_norm, rows) else None
+            self.head.forward(LazyRmsNorm(self.final_norm, rows, make, given), logits)
         else:
             self.head.forward(self.final_norm.forward(rows, make()), logits)
         return logits

@@ -321,6 +321,64 @@ def norm_gemm(x: torch.Tensor, gain: torch.Tensor, eps: float, w: torch.Tensor,
                                         _ptr(out), M, N, K, epi, rg, _stream()), "norm_gemm")
 
 
+def norm_emit_plan(M: int, N: int, K: int, w: torch.Tensor, w_tiled: bool):
+    """Row groups per workgroup if ``gemm_emit`` covers out += a w^T (weight-streaming kernel,
+    up to 16 tokens, pre-tiled bfloat16 weight, no split over workgroups), else None."""
+    if not (w_tiled and 0 < M <= NORM_FOLD_MAX_M and w.dtype == torch.bfloat16 and w.is_cuda):
+        return None
+    rg, ks = _skinny_plan(M, N, K, True)
+    return rg if (ks == 1 and rg <= 2) else None
+
+
+def gemm_emit(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, gain: torch.Tensor,
+              xg: torch.Tensor, sq: torch.Tensor) -> None:
+    """residual += a w^T in 32-bit (``w`` pre-tiled) and, for the RMSNorm that reads the sum
+    next, from the same epilogue: xg = bfloat16(residual * gain) [M, N] and sq [N / 16, 16] =
+    the sums of residual^2 over each 16 columns per token, which ``gemm_given`` takes."""
+    _need_gpu(a, w, residual, gain, xg, sq)
+    M, K = a.shape
+    N = w.shape[0]
+    rg = norm_emit_plan(M, N, K, w, True)
+    if rg is None or a.dtype != torch.bfloat16 or w.shape[1] != K or not can_pretile(w) \
+            or residual.shape != (M, N) or residual.dtype != torch.float32 \
+            or gain.shape != (N,) or gain.dtype != torch.float32 \
+            or xg.shape != (M, N) or xg.dtype != torch.bfloat16 \
+            or sq.shape != (N // 16, 16) or sq.dtype != torch.float32 \
+            or not all(t.is_contiguous() for t in (a, residual, xg, sq)):
+        raise KernelUnavailable(f"gemm_emit: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)}, "
+                                f"residual {tuple(residual.shape)} {residual.dtype}")
+    lib = build.load("gemm")
+    _check(lib.zf_gemm_bf16_skinny_emit(_ptr(a), _ptr(w), _ptr(residual), _ptr(gain), _ptr(xg),
+                                        _ptr(sq), M, N, K, rg, _stream()), "gemm_emit")
+
+
+def gemm_given(xg: torch.Tensor, sq: torch.Tensor, eps: float, w: torch.Tensor,
+               out: torch.Tensor, swiglu: bool = False) -> None:
+    """out = rmsnorm(x) w^T from what ``gemm_emit`` left of x: xg = bfloat16(x * gain) and the
+    partial sums of squares sq [groups, 16]; the token's 1 / sqrt(mean(x^2) + eps) scales the
+    32-bit sums of the product.  With ``swiglu`` as ``gemm_swiglu``."""
+    _need_gpu(xg, sq, w, out)
+    M, K = xg.shape
+    N = w.shape[0]
+    rg = norm_gemm_plan(M, N, K, w, True)
+    if swiglu and 0 < M <= NORM_FOLD_MAX_M:
+        rg = 2
+    if rg is None or xg.dtype != torch.bfloat16 or sq.dtype != torch.float32 \
+            or sq.dim() != 2 or sq.shape[1] != 16 or sq.shape[0] * 16 != K \
+            or w.shape[1] != K or not can_pretile(w) \
+            or out.shape != (M, N // 2 if swiglu else N) \
+            or (swiglu and out.dtype != torch.bfloat16) \
+            or not all(t.is_contiguous() for t in (xg, sq, out)):
+        raise KernelUnavailable(f"gemm_given: xg {tuple(xg.shape)} {xg.dtype}, w {tuple(w.shape)}, "
+                                f"out {tuple(out.shape)} {out.dtype}")
+    epi = _EPI_SWIGLU if swiglu else \
+        (_EPI_STORE_BF16 if out.dtype == torch.bfloat16 else _EPI_STORE_F32)
+    lib = build.load("gemm")
+    _check(lib.zf_gemm_bf16_skinny_given(_ptr(xg), _ptr(sq), sq.shape[0], ctypes.c_float(eps),
+                                         _ptr(w), _ptr(out), M, N, K, epi, rg, _stream()),
+           "gemm_given")
+
+
 def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """Rows of the gate and the up projection alternating in groups of 16 (gate 0..15, up
     0..15, gate 16..31, ...): the order ``gemm_swiglu`` wants.  Needs I % 16 == 0."""

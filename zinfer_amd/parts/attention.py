@@ -103,7 +103,7 @@ class GqaAttention(Mixer):
                             0 if s.window is None else int(s.window),
                             s.n_heads, s.n_kv_heads, s.head_dim, cache.page_size,
                             step.max_q_len, step.max_ctx_len, n_single=step.n_single)
-        self.o.forward(attn, residual, accumulate=True)
+        self.o.forward(attn, residual, accumulate=True, step=step)
 
 
 register_part("mixer", GqaAttentionSpec, GqaAttention)

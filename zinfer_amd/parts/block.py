@@ -22,6 +22,8 @@ class PreNormBlock(Block):
         self.feed_forward = build_part("feed_forward", spec.feed_forward, ctx,
                                        prefix + spec.ff_prefix)
         self.parts = (self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward)
+        # the norm that reads the residual stream first, if what a sum leaves for it is of use
+        self.entry_norm = self._lazy(self.mixer_norm, self.mixer)
         self.graph_safe = all(p.graph_safe for p in self.parts)
         self.kernel_modules = tuple(sorted({m for p in self.parts for m in p.kernel_modules}))
 
@@ -42,14 +44,28 @@ class PreNormBlock(Block):
         """The consumer's input: the normed activations, or, for a consumer that says it can
         fold an RMSNorm into its first product, the norm still to be run."""
         make = lambda: step.scratch("normed", x.shape, self.ctx.act_dtype)
+        ready, step.norm_ready, step.norm_after = step.norm_ready, None, None
         if isinstance(norm, RmsNorm) and getattr(consumer, "accepts_lazy_norm", False) \
                 and x.is_cuda and self.ctx.compute_dtype == torch.bfloat16:
-            return LazyRmsNorm(norm, x, make)
+            given = ready if ready is not None and ready.fits(norm, x) else None
+            return LazyRmsNorm(norm, x, make, given)
         return norm.forward(x, make())
 
+    def _lazy(self, norm, consumer):
+        """``norm`` if its reader takes a norm that has not run (and so what a residual sum
+        leaves for it), else None."""
+        return norm if isinstance(norm, RmsNorm) and \
+            getattr(consumer, "accepts_lazy_norm", False) else None
+
     def forward(self, x, step, cache) -> None:
-        self.mixer.forward(self._normed(self.mixer_norm, self.mixer, x, step), x, step, cache)
-        self.feed_forward.forward(self._normed(self.ff_norm, self.feed_forward, x, step), x, step)
+        after_block = step.norm_after_block
+        h = self._normed(self.mixer_norm, self.mixer, x, step)
+        step.norm_after = self._lazy(self.ff_norm, self.feed_forward)
+        self.mixer.forward(h, x, step, cache)
+        h = self._normed(self.ff_norm, self.feed_forward, x, step)
+        step.norm_after = after_block
+        self.feed_forward.forward(h, x, step)
+        step.norm_after = None
 
 
 register_part("block", PreNormBlockSpec, PreNormBlock)

@@ -18,17 +18,32 @@ class Linear:
         self.tiled = bool(pretile and weight.is_cuda and ops.can_pretile(weight))
         self.weight = ops.pretile_weight(weight) if self.tiled else weight.contiguous()
 
-    def forward(self, x, out: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
+    def forward(self, x, out: torch.Tensor, accumulate: bool = False, step=None) -> torch.Tensor:
         """out = x W^T, or out += x W^T (``out`` float32) when ``accumulate``.  ``x`` may be a
         norm that has not run yet (``LazyRmsNorm``): it is folded into the product when the
-        weight-streaming kernel covers it, else it runs first."""
+        weight-streaming kernel covers it, else it runs first.  With ``accumulate`` and a
+        ``step`` that names the norm reading ``out`` next (``step.norm_after``), the sum's
+        kernel leaves that norm's inputs in ``step.norm_ready`` when it can."""
         if hasattr(x, "materialize"):
             M, K = x.shape
             if not accumulate and \
                     ops.norm_gemm_plan(M, self.out_features, K, self.weight, self.tiled) is not None:
-                ops.norm_gemm(x.x, x.gain, x.eps, self.weight, out)
+                if x.given is not None:
+                    ops.gemm_given(x.given.xg, x.given.sq, x.eps, self.weight, out)
+                else:
+                    ops.norm_gemm(x.x, x.gain, x.eps, self.weight, out)
                 return out
             x = x.materialize()
+        norm = getattr(step, "norm_after", None) if accumulate else None
+        if norm is not None and hasattr(norm, "gain") and x.dtype == torch.bfloat16 and \
+                ops.norm_emit_plan(x.shape[0], self.out_features, self.in_features, self.weight,
+                                   self.tiled) is not None:
+            from .norm import GivenRmsNorm
+            xg = step.scratch("normed_by_gain", out.shape, torch.bfloat16)
+            sq = step.scratch("normed_squares", (self.out_features // 16, 16), torch.float32)
+            ops.gemm_emit(x, self.weight, out, norm.gain, xg, sq)
+            step.norm_ready = GivenRmsNorm(norm, out, xg, sq)
+            return out
         ops.gemm(x, self.weight, out, accumulate, w_tiled=self.tiled)
         return out
 

@@ -48,8 +48,11 @@ class SwiGluMlp(FeedForward):
         a = step.scratch("ff_act", (T, I), act)
         if self.fused and hasattr(h, "materialize") and self.gate_up.tiled \
                 and T <= ops.NORM_FOLD_MAX_M:
-            ops.norm_gemm(h.x, h.gain, h.eps, self.gate_up.weight, a, swiglu=True)
-            self.down.forward(a, residual, accumulate=True)
+            if h.given is not None:
+                ops.gemm_given(h.given.xg, h.given.sq, h.eps, self.gate_up.weight, a, swiglu=True)
+            else:
+                ops.norm_gemm(h.x, h.gain, h.eps, self.gate_up.weight, a, swiglu=True)
+            self.down.forward(a, residual, accumulate=True, step=step)
             return
         if hasattr(h, "materialize"):
             h = h.materialize()
@@ -59,7 +62,7 @@ class SwiGluMlp(FeedForward):
             gu = step.scratch("gate_up", (T, 2 * I), act)
             self.gate_up.forward(h, gu)
             ops.swiglu(gu, a)
-        self.down.forward(a, residual, accumulate=True)
+        self.down.forward(a, residual, accumulate=True, step=step)
 
 
 class _probe:

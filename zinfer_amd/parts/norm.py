@@ -28,14 +28,28 @@ class RmsNorm(Norm):
         return out
 
 
+class GivenRmsNorm:
+    """What the kernel that last added into the residual rows ``x`` left for ``norm``:
+    xg = bfloat16(x * gain) and sq [width / 16, 16], the sums of x^2 over each 16 columns per
+    token (``ops.gemm_emit``)."""
+
+    def __init__(self, norm: "RmsNorm", x: torch.Tensor, xg: torch.Tensor, sq: torch.Tensor):
+        self.norm, self.x, self.xg, self.sq = norm, x, xg, sq
+
+    def fits(self, norm, x: torch.Tensor) -> bool:
+        return self.norm is norm and self.x.data_ptr() == x.data_ptr() and self.x.shape == x.shape
+
+
 class LazyRmsNorm:
     """A norm that has not run yet: the residual rows and the norm's parameters.  A consumer
     whose first matrix product can fold the norm in (``Linear.forward``) takes it apart;
-    anyone else calls ``materialize()`` and gets the normed activations (computed once)."""
+    anyone else calls ``materialize()`` and gets the normed activations (computed once).
+    ``given``: what the producer of the rows already left of the norm, if anything."""
 
-    def __init__(self, norm: "RmsNorm", x: torch.Tensor, make_out):
+    def __init__(self, norm: "RmsNorm", x: torch.Tensor, make_out, given: GivenRmsNorm = None):
         self.x, self.gain, self.eps = x, norm.gain, float(norm.spec.eps)
         self.shape = x.shape
+        self.given = given
         self._norm, self._make_out, self._out = norm, make_out, None
 
     def materialize(self) -> torch.Tensor:
