@@ -429,3 +429,205 @@ def test_toy_architecture_registered_built_and_stepped(kind, tmp_path):
     finally:
         unregister_architecture("ToyForCausalLM")
         unregister_part("mixer", ToyStateSpec)
+
+
+# ----------------------------------------------------------------------------- more toy parts
+# Another norm, another position encoding and a feed-forward with routing, defined here and
+# registered from the test: nothing in the framework's files knows of them.
+@dataclass(frozen=True)
+class ToyLayerNormSpec:
+    """(x - mean) / sqrt(var + eps) * w, without a bias."""
+    width: int
+    eps: float
+
+
+@dataclass(frozen=True)
+class ToyLearnedPositionSpec:
+    """A learned vector per position, added to every query and key head."""
+    head_dim: int
+    max_positions: int
+
+
+@dataclass(frozen=True)
+class ToyRoutedSpec:
+    """Top-1 of ``n_experts`` small ReLU networks, weighted by the router's probability."""
+    hidden_size: int
+    inner_size: int
+    n_experts: int
+
+
+def _register_toy_parts():
+    from zinfer_amd.parts import FeedForward, Norm, PositionEncoding, TensorDecl, register_part
+
+    class ToyLayerNorm(Norm):
+        def declare(self):
+            return {self.prefix + "weight": TensorDecl((self.spec.width,), init="gain")}
+
+        def bind(self, tensors):
+            self.w = tensors[self.prefix + "weight"].float().to(self.ctx.device)
+
+        def forward(self, x, out):
+            mu = x.mean(-1, keepdim=True)
+            var = ((x - mu) ** 2).mean(-1, keepdim=True)
+            out.copy_(((x - mu) / torch.sqrt(var + self.spec.eps) * self.w).to(out.dtype))
+            return out
+
+    class ToyLearnedPosition(PositionEncoding):
+        custom_apply = True
+
+        def declare(self):
+            s = self.spec
+            return {self.prefix + "pos_table": TensorDecl((s.max_positions, s.head_dim))}
+
+        def bind(self, tensors):
+            self.table = tensors[self.prefix + "pos_table"].float().to(self.ctx.device)
+
+        def apply(self, q, k, positions):
+            add = self.table[positions.long()][:, None, :]
+            q.add_(add.to(q.dtype))
+            k.add_(add.to(k.dtype))
+
+    class ToyRouted(FeedForward):
+        def declare(self):
+            s, p = self.spec, self.prefix
+            return {p + "router.weight": TensorDecl((s.n_experts, s.hidden_size)),
+                    p + "w_in": TensorDecl((s.n_experts, s.inner_size, s.hidden_size)),
+                    p + "w_out": TensorDecl((s.n_experts, s.hidden_size, s.inner_size))}
+
+        def bind(self, tensors):
+            dev = self.ctx.device
+            self.router = tensors[self.prefix + "router.weight"].float().to(dev)
+            self.w_in = tensors[self.prefix + "w_in"].float().to(dev)
+            self.w_out = tensors[self.prefix + "w_out"].float().to(dev)
+
+        def forward(self, h, residual, step):
+            h = h.float()
+            prob = torch.softmax(h @ self.router.T, dim=-1)          # 32-bit router
+            weight, expert = prob.max(dim=-1)
+            for e in range(self.spec.n_experts):
+                y = torch.relu(h @ self.w_in[e].T) @ self.w_out[e].T
+                residual += ((expert == e) * weight)[:, None] * y
+
+    register_part("norm", ToyLayerNormSpec, ToyLayerNorm)
+    register_part("position", ToyLearnedPositionSpec, ToyLearnedPosition)
+    register_part("feed_forward", ToyRoutedSpec, ToyRouted)
+
+
+@dataclass(frozen=True)
+class ToyRoutedConfig:
+    hidden_size: int
+    inner_size: int
+    n_experts: int
+    n_layers: int
+    vocab_size: int
+    model_type: str = "toy_routed"
+    HEADS, KV_HEADS, HEAD_DIM, MAX_POS, EPS = 3, 1, 16, 256, 1e-4
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(**{k: raw[k] for k in ("hidden_size", "inner_size", "n_experts", "n_layers",
+                                          "vocab_size")})
+
+    def to_dict(self):
+        return dict(architectures=["ToyRoutedForCausalLM"], model_type="toy_routed",
+                    hidden_size=self.hidden_size, inner_size=self.inner_size,
+                    n_experts=self.n_experts, n_layers=self.n_layers, vocab_size=self.vocab_size)
+
+    def model_spec(self):
+        from zinfer_amd.config.specs import (GqaAttentionSpec, ModelSpec, PreNormBlockSpec,
+                                             ScheduleEntry)
+        H = self.hidden_size
+        norm = ToyLayerNormSpec(H, self.EPS)
+        attn = GqaAttentionSpec(H, self.HEADS, self.KV_HEADS, self.HEAD_DIM, None,
+                                ToyLearnedPositionSpec(self.HEAD_DIM, self.MAX_POS), None)
+        ff = ToyRoutedSpec(H, self.inner_size, self.n_experts)
+        blk = PreNormBlockSpec(mixer=attn, feed_forward=ff, mixer_norm=norm, ff_norm=norm)
+        return ModelSpec(vocab_size=self.vocab_size, hidden_size=H, max_positions=self.MAX_POS,
+                         layers=(blk,) * self.n_layers,
+                         schedule=tuple(ScheduleEntry(i) for i in range(self.n_layers)),
+                         final_norm=norm, tie_word_embeddings=False)
+
+
+def _toy_routed_plain(cfg: ToyRoutedConfig, w, toks):
+    """Whole sequence in 64-bit, token after token; returns the logits and, per token and
+    layer, the margin between the two best router probabilities."""
+    nH, nKV, hd, eps = cfg.HEADS, cfg.KV_HEADS, cfg.HEAD_DIM, cfg.EPS
+    W = {k: v.to(F64) for k, v in w.items()}
+
+    def layer_norm(x, g):
+        mu = x.mean()
+        return (x - mu) / torch.sqrt(((x - mu) ** 2).mean() + eps) * g
+
+    caches = [([], []) for _ in range(cfg.n_layers)]
+    rows, margins = [], []
+    for p, tok in enumerate(toks):
+        x = W["model.embed_tokens.weight"][tok]
+        for i in range(cfg.n_layers):
+            pre = f"model.layers.{i}."
+            n = layer_norm(x, W[pre + "input_layernorm.weight"])
+            q = plain.linear(n, W[pre + "self_attn.q_proj.weight"]).reshape(nH, hd)
+            k = plain.linear(n, W[pre + "self_attn.k_proj.weight"]).reshape(nKV, hd)
+            v = plain.linear(n, W[pre + "self_attn.v_proj.weight"]).reshape(nKV, hd)
+            q = q + W[pre + "self_attn.pos_table"][p]
+            k = k + W[pre + "self_attn.pos_table"][p]
+            caches[i][0].append(k); caches[i][1].append(v)
+            o = plain.attention_single_query(q.reshape(-1), torch.stack(caches[i][0]),
+                                             torch.stack(caches[i][1]), nH, nKV, hd, None)
+            x = x + plain.linear(o, W[pre + "self_attn.o_proj.weight"])
+            m = layer_norm(x, W[pre + "post_attention_layernorm.weight"])
+            prob = plain.softmax(plain.linear(m, W[pre + "mlp.router.weight"]))
+            e = int(prob.argmax())
+            top2 = prob.topk(2).values
+            margins.append(float(top2[0] - top2[1]))
+            y = plain.linear(torch.relu(plain.linear(m, W[pre + "mlp.w_in"][e])),
+                             W[pre + "mlp.w_out"][e])
+            x = x + prob[e] * y
+        rows.append(plain.linear(layer_norm(x, W["model.norm.weight"]), W["lm_head.weight"]))
+    return torch.stack(rows).numpy(), min(margins)
+
+
+def test_toy_norm_position_and_routed_feed_forward(tmp_path):
+    """A layer norm, a learned position encoding applied by the part itself and a routed
+    feed-forward, all defined in this file, make a model that the engine builds from its
+    folder and steps under every cutting; compared with the same formulas in 64-bit."""
+    from zinfer_amd.config import register_architecture, unregister_architecture
+    from zinfer_amd.engine import StepEntry
+    from zinfer_amd.engine.replay import make_engine
+    from zinfer_amd.parts import unregister_part
+    from zinfer_amd.weights import SafetensorsFile, write_model_dir
+    _register_toy_parts()
+    register_architecture("ToyRoutedForCausalLM", ToyRoutedConfig, model_type="toy_routed")
+    try:
+        cfg = ToyRoutedConfig(hidden_size=48, inner_size=40, n_experts=3, n_layers=2,
+                              vocab_size=211)
+        path = write_model_dir(str(tmp_path / "toy_routed"), cfg, seed=9, dtype=torch.float32)
+        with SafetensorsFile(os.path.join(path, "model.safetensors")) as f:
+            w = {n: f.tensor(n) for n in f.names()}
+        assert all(any(key in n for n in w) for key in ("router", "pos_table", "w_in", "w_out"))
+        requests = {f"t{i}": tiny.random_tokens(n, 211, 90 + i) for i, n in enumerate((41, 5, 70, 18))}
+        ref, margin = {}, 1.0
+        for rid, t in requests.items():
+            ref[rid], mg = _toy_routed_plain(cfg, w, t)
+            margin = min(margin, mg)
+        assert margin > 1e-5, "two experts nearly tie: the 32-bit router might pick the other"
+        for mode in ("whole", "portions", "mixed"):
+            steps = {"whole": traces.whole, "portions": traces.changing_portions,
+                     "mixed": traces.mixed}[mode](requests)
+            eng = make_engine(path, "float32", traces.peak_tokens(steps, 64), DEV, poison_freed=True)
+            assert not eng.use_graphs          # the toy parts do not claim to be graph-safe
+            got_steps = {}
+            for st in steps:
+                lg = eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]],
+                              end=st["end"])
+                if lg.shape[0]:
+                    got_steps[st["step"]] = lg.cpu().numpy()
+            eng.cache.check()
+            out = traces.collect(steps, got_steps, 211)
+            for rid in requests:
+                err = np.abs(out[rid] - ref[rid]).max() / np.abs(ref[rid]).max()
+                assert err <= 2e-5, f"{mode} {rid}: {err:.3g}"
+    finally:
+        unregister_architecture("ToyRoutedForCausalLM")
+        unregister_part("norm", ToyLayerNormSpec)
+        unregister_part("position", ToyLearnedPositionSpec)
+        unregister_part("feed_forward", ToyRoutedSpec)
