@@ -130,6 +130,32 @@ def test_gemm_pretiled_weights(M, N, K, o_dtype, accumulate):
     assert rel_err(got, plain_out) <= (tol(o_dtype) if not accumulate else 2e-5)
 
 
+@pytest.mark.parametrize("kind", ["store", "accumulate", "swiglu"])
+def test_gemm_many_large_tiles(kind):
+    """Enough 256 x 256 tiles to fill the chip more than once (the kernel that takes
+    pre-tiled W straight into its operands), with edges in M and N that are no multiple of
+    the tile and several k-tiles."""
+    ops = _ops()
+    M, N, K = 4100, 4160, 192
+    a = _rand((M, K), torch.bfloat16, 35)
+    w = _rand((N, K), torch.bfloat16, 36, 0.05)
+    if kind == "swiglu":
+        wi = ops.interleave_gate_up(w[:N // 2].to(DEV), w[N // 2:].to(DEV))
+        want = torch.empty((M, N // 2), dtype=torch.bfloat16)
+        ref.gemm_swiglu(a, wi.cpu(), want)
+        got = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.gemm_swiglu(a.to(DEV), ops.pretile_weight(wi), got, w_tiled=True)
+        assert rel_err(got, want) <= tol(torch.bfloat16)
+        return
+    acc = kind == "accumulate"
+    base = _rand((M, N), torch.float32, 37).to(torch.float32 if acc else torch.bfloat16)
+    want = base.clone()
+    ref.gemm(a, w, want, acc)
+    got = base.clone().to(DEV)
+    ops.gemm(a.to(DEV), ops.pretile_weight(w.to(DEV)), got, acc, w_tiled=True)
+    assert rel_err(got, want) <= (2e-5 if acc else tol(torch.bfloat16))
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64, 65, 200, 300])
 @pytest.mark.parametrize("I,K,tiled", [(32, 64, True), (12288 // 8, 320, True), (96, 136, False),
                                        (352, 4096, True), (8192, 192, True)])

@@ -301,6 +301,231 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_ker
     }
 }
 
+// ---------------------------------------------------------------- large M, pre-tiled W: W not staged
+// 256 x 256 x 64 tiles, 4 waves of 128 x 128.  Only the tokens go through LDS; every wave
+// takes its W operands straight from the pre-tiled matrix (16-byte pieces that lie in runs of
+// 256 bytes), one k-tile ahead in registers.  That halves the LDS traffic per MFMA against
+// the kernel above, whose LDS is as busy as its MFMAs.
+template <int BM, int BN, int WM, int WN, int EPI>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdirect_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
+    int N, int K, int tiles_m, int tiles_n) {
+  constexpr int NWN = BN / WN, NT = (BM / WM) * NWN * 64;
+  constexpr int FM = WM / 32, FN = WN / 32;
+  static_assert(BM * 8 % NT == 0, "tile does not divide over the threads");
+  constexpr int A_CHUNKS = BM * 8 / NT;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  bf16_t* lds = (bf16_t*)lds_raw;       // two stages of BM rows of LDS_ROW elements
+
+  const int nblocks = tiles_m * tiles_n;
+  int b = blockIdx.x;
+  {
+    const int base = nblocks / 8, rem = nblocks % 8;
+    const int xcd = b % 8, idx = b / 8;
+    b = xcd * base + min(xcd, rem) + idx;
+  }
+  const int GROUP = 8;
+  const int in_group = GROUP * tiles_n;
+  const int g = b / in_group;
+  const int first_m = g * GROUP;
+  const int gsize = min(tiles_m - first_m, GROUP);
+  const int tm = first_m + (b % in_group) % gsize;
+  const int tn = (b % in_group) / gsize;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const int tid = threadIdx.x;
+  const int wave = tid / 64, lane = tid % 64;
+  const int wm = wave / NWN, wn = wave % NWN;
+
+  f32x16_t acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // W operand of MFMA (j, ks): column n = n0 + wn * WN + 32 j + lane % 32, k = 16 ks +
+  // 8 (lane / 32) .. + 8 of the k-tile: piece 64 (lane / 32) + 16 ks + n % 16 of the 16-row
+  // group n / 16.  Groups beyond N are clamped (their columns are never stored).
+  const bf16_t* wbase[FN];
+#pragma unroll
+  for (int j = 0; j < FN; ++j) {
+    const int n = n0 + wn * WN + j * 32 + lane % 32;
+    const int grp = min(n / 16, N / 16 - 1);
+    wbase[j] = W + (size_t)grp * (K / 64) * 1024 + ((lane / 32) * 64 + n % 16) * 8;
+  }
+  u32x4_t areg[A_CHUNKS];
+  u32x4_t wreg[TK / 16][FN];
+
+  auto gload_a = [&](int k0) {
+#pragma unroll
+    for (int c = 0; c < A_CHUNKS; ++c) {
+      const int chunk = tid + c * NT;
+      const int row = chunk / 8, kc = (chunk % 8) * 8;
+      const int m = min(m0 + row, M - 1);
+      areg[c] = *(const u32x4_t*)(A + (size_t)m * K + k0 + kc);
+    }
+  };
+  auto gload_w = [&](int kt, int ks) {
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+      wreg[ks][j] = *(const u32x4_t*)(wbase[j] + (size_t)kt * 1024 + ks * 128);
+  };
+  auto lstore = [&](int stage) {
+    bf16_t* a_s = lds + stage * BM * LDS_ROW;
+#pragma unroll
+    for (int c = 0; c < A_CHUNKS; ++c) {
+      const int chunk = tid + c * NT;
+      const int row = chunk / 8, kc = (chunk % 8) * 8;
+      *(u32x4_t*)(a_s + row * LDS_ROW + kc) = areg[c];
+    }
+  };
+
+  const int ktiles = K / TK;
+  gload_a(0);
+#pragma unroll
+  for (int ks = 0; ks < TK / 16; ++ks) gload_w(0, ks);
+  lstore(0);
+  __syncthreads();
+  // One k-tile per trip: MFMAs on LDS stage `kt & 1`; meanwhile the tokens of tile kt + 1
+  // travel through registers into the other stage, and every k-step's W registers are
+  // refilled with their part of tile kt + 1 right after their last use.  No branches around
+  // the loads (the last trip loads its own tile once more), so the compiler can count the
+  // loads in flight and waits for no younger one; the scheduling barriers keep it from
+  // sinking the loads down to their first use, which would expose their whole latency.
+  for (int kt = 0; kt < ktiles; ++kt) {
+    const int stage = kt & 1;
+    const int nxt = min(kt + 1, ktiles - 1);
+    gload_a(nxt * TK);
+    __builtin_amdgcn_sched_barrier(0);
+    const bf16_t* a_s = lds + stage * BM * LDS_ROW + (wm * WM) * LDS_ROW;
+    // the token operands of k-step ks + 1 are read from LDS while the MFMAs of ks run
+    bf16x8_t af[2][FM];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+      af[0][i] = *(const bf16x8_t*)(a_s + (i * 32 + lane % 32) * LDS_ROW + (lane / 32) * 8);
+#pragma unroll
+    for (int ks = 0; ks < TK / 16; ++ks) {
+      if (ks + 1 < TK / 16) {
+        const int koff = (ks + 1) * 16 + (lane / 32) * 8;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+          af[(ks + 1) % 2][i] = *(const bf16x8_t*)(a_s + (i * 32 + lane % 32) * LDS_ROW + koff);
+      }
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              af[ks % 2][i], *(const bf16x8_t*)&wreg[ks][j], acc[i][j], 0, 0, 0);
+      gload_w(nxt, ks);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    lstore(stage ^ 1);
+    __syncthreads();
+  }
+
+  // Epilogue through LDS: a 32x32 MFMA result has a lane's 16 values in 16 different rows,
+  // so direct stores would be 2 or 4 bytes wide in runs of 64 bytes.  Each wave lays 32 rows
+  // of its tile down in its own slab (rows padded by 4 floats) and reads them back along the
+  // rows, 16 bytes per lane.  (The main loop's last barrier has freed the token stages.)
+  constexpr int SLAB_ROW = WN + 4;
+  static_assert((size_t)(BM / WM) * NWN * 32 * SLAB_ROW * 4 <= (size_t)2 * BM * LDS_ROW * 2,
+                "slabs do not fit into the token stages");
+  float* slab = (float*)lds_raw + (size_t)wave * 32 * SLAB_ROW;
+  const int mw = m0 + wm * WM, nw = n0 + wn * WN;
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        slab[(8 * (r / 4) + 4 * (lane / 32) + r % 4) * SLAB_ROW + j * 32 + lane % 32] = acc[i][j][r];
+    __syncthreads();
+    if (EPI == EPI_SWIGLU) {
+      // 16 gate columns, then the 16 up columns that belong to them: 8 outputs per lane
+      constexpr int LPR = WN / 16;                  // lanes per row
+#pragma unroll
+      for (int it = 0; it < 32 * LPR / 64; ++it) {
+        const int row = it * (64 / LPR) + lane / LPR, q = lane % LPR;
+        const int m = mw + i * 32 + row;
+        const int c = (q / 2) * 32 + (q % 2) * 8;   // first gate column inside the wave's tile
+        const int n = nw + c;
+        if (m < M && n < N) {
+          const float* src = slab + row * SLAB_ROW + c;
+          const float4 g0 = *(const float4*)src, g1 = *(const float4*)(src + 4);
+          const float4 u0 = *(const float4*)(src + 16), u1 = *(const float4*)(src + 20);
+          const u32x4_t v = u32x4_t{
+              pack_bf16x2(swiglu_f(g0.x, u0.x), swiglu_f(g0.y, u0.y)),
+              pack_bf16x2(swiglu_f(g0.z, u0.z), swiglu_f(g0.w, u0.w)),
+              pack_bf16x2(swiglu_f(g1.x, u1.x), swiglu_f(g1.y, u1.y)),
+              pack_bf16x2(swiglu_f(g1.z, u1.z), swiglu_f(g1.w, u1.w))};
+          *(u32x4_t*)((bf16_t*)Cv + (size_t)m * (N / 2) + (n / 32) * 16 + (n % 32)) = v;
+        }
+      }
+    } else if (EPI == EPI_STORE_BF16) {
+      constexpr int LPR = WN / 8;
+#pragma unroll
+      for (int it = 0; it < 32 * LPR / 64; ++it) {
+        const int row = it * (64 / LPR) + lane / LPR, c = (lane % LPR) * 8;
+        const int m = mw + i * 32 + row, n = nw + c;
+        if (m < M && n < N) {
+          const float* src = slab + row * SLAB_ROW + c;
+          const float4 x0 = *(const float4*)src, x1 = *(const float4*)(src + 4);
+          const u32x4_t v = u32x4_t{pack_bf16x2(x0.x, x0.y), pack_bf16x2(x0.z, x0.w),
+                                    pack_bf16x2(x1.x, x1.y), pack_bf16x2(x1.z, x1.w)};
+          *(u32x4_t*)((bf16_t*)Cv + (size_t)m * N + n) = v;
+        }
+      }
+    } else {
+      constexpr int LPR = WN / 4;
+#pragma unroll
+      for (int it = 0; it < 32 * LPR / 64; ++it) {
+        const int row = it * (64 / LPR) + lane / LPR, c = (lane % LPR) * 4;
+        const int m = mw + i * 32 + row, n = nw + c;
+        if (m < M && n < N) {
+          float4 x = *(const float4*)(slab + row * SLAB_ROW + c);
+          float4* dst = (float4*)((float*)Cv + (size_t)m * N + n);
+          if (EPI == EPI_ACC_F32) {
+            const float4 old = *dst;
+            x = float4{old.x + x.x, old.y + x.y, old.z + x.z, old.w + x.w};
+          }
+          *dst = x;
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <int BM, int BN, int WM, int WN>
+static int launch_tile_wdirect(const void* A, const void* W, void* C, int M, int N, int K, int epi,
+                               hipStream_t stream) {
+  if (N % 16 != 0 || K % 64 != 0) return -3;
+  constexpr int NT = (BM / WM) * (BN / WN) * 64;
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  const dim3 grid(tiles_m * tiles_n), block(NT);
+  const size_t smem = (size_t)2 * BM * LDS_ROW * sizeof(bf16_t);
+#define ZF_WD(E)                                                                              \
+  do {                                                                                        \
+    auto kern = gemm_bf16_tile_wdirect_kernel<BM, BN, WM, WN, E>;                             \
+    if (smem > 64 * 1024) {                                                                   \
+      hipError_t e = hipFuncSetAttribute((const void*)kern,                                   \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
+      if (e != hipSuccess) return (int)e;                                                     \
+    }                                                                                         \
+    hipLaunchKernelGGL(kern, grid, block, smem, stream, (const bf16_t*)A, (const bf16_t*)W, C, \
+                       M, N, K, tiles_m, tiles_n);                                            \
+  } while (0)
+  if (epi == EPI_STORE_BF16) ZF_WD(EPI_STORE_BF16);
+  else if (epi == EPI_STORE_F32) ZF_WD(EPI_STORE_F32);
+  else if (epi == EPI_SWIGLU) ZF_WD(EPI_SWIGLU);
+  else ZF_WD(EPI_ACC_F32);
+#undef ZF_WD
+  return (int)hipGetLastError();
+}
+
 template <int BM, int BN, int WM, int WN, bool WT>
 static int launch_tile(const void* A, const void* W, void* C, int M, int N, int K, int epi,
                        hipStream_t stream) {
@@ -328,7 +553,9 @@ static int launch_tile(const void* A, const void* W, void* C, int M, int N, int 
 }
 
 // variant: 0 = 128x128 (waves 64x64), 1 = 256x128 (waves 128x64), 2 = 256x256 (waves 128x128),
-//          3 = 128x128 (waves 64x32, 8 waves), 4 = 256x256 (waves 128x64, 8 waves)
+//          3 = 128x128 (waves 64x32, 8 waves), 4 = 256x256 (waves 128x64, 8 waves);
+//          with pre-tiled W only: 5 = 256x256 (waves 128x128), 6 = 128x128 (waves 64x64),
+//          7 = 256x128 (waves 128x64), W straight from memory into the MFMA operands
 //          w_tiled: W is in the pre-tiled layout (needs N % 16 == 0 and K % 64 == 0)
 extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, int N, int K,
                                  int epi, int variant, int w_tiled, hipStream_t stream) {
@@ -336,6 +563,9 @@ extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, i
   if (K % 8 != 0 || (epi == EPI_SWIGLU && N % 32 != 0)) return -3;
   if (w_tiled) {
     if (N % 16 != 0 || K % 64 != 0) return -3;
+    if (variant == 5) return launch_tile_wdirect<256, 256, 128, 128>(A, W, C, M, N, K, epi, stream);
+    if (variant == 6) return launch_tile_wdirect<128, 128, 64, 64>(A, W, C, M, N, K, epi, stream);
+    if (variant == 7) return launch_tile_wdirect<256, 128, 128, 64>(A, W, C, M, N, K, epi, stream);
     switch (variant) {
       case 0: return launch_tile<128, 128, 64, 64, true>(A, W, C, M, N, K, epi, stream);
       case 4: return launch_tile<256, 256, 128, 64, true>(A, W, C, M, N, K, epi, stream);

@@ -224,9 +224,15 @@ def _skinny_plan(M: int, N: int, K: int, tiled: bool):
     return rg, ks
 
 
-def _tile_variant(M: int, N: int) -> int:
-    """256 x 256 tiles when they still fill the chip, else 128 x 128."""
+def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = False) -> int:
+    """Which tiled kernel: with pre-tiled weights the kernels that take W straight from
+    memory (5: 256 x 256 tiles when they fill the chip at least once and the epilogue is a
+    plain store, whose cost a single resident workgroup cannot hide behind others; else 6:
+    128 x 128); otherwise the kernels that stage both operands through LDS (4: 256 x 256 when
+    they still fill the chip, else 0: 128 x 128).  Measured on MI355X at the Qwen3-8B sizes."""
     tiles = ((M + 255) // 256) * ((N + 255) // 256)
+    if w_tiled:
+        return 5 if (tiles >= 256 and not accumulate) else 6
     return 4 if tiles >= 160 else 0
 
 
@@ -278,7 +284,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
                    "gemm (weight streaming)")
         else:
             _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, epi,
-                                         _tile_variant(M, N), 1 if w_tiled else 0, _stream()),
+                                         _tile_variant(M, N, w_tiled, accumulate),
+                                         1 if w_tiled else 0, _stream()),
                    "gemm (tiled)")
         return
     _check(lib.zf_gemm_fma(_ptr(a), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), M, N, K,
@@ -412,7 +419,8 @@ def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bo
                "gemm_swiglu (weight streaming)")
     else:
         _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, _EPI_SWIGLU,
-                                     _tile_variant(M, N), 1 if w_tiled else 0, _stream()),
+                                     _tile_variant(M, N, w_tiled), 1 if w_tiled else 0,
+                                     _stream()),
                "gemm_swiglu (tiled)")
 
 
