@@ -199,6 +199,133 @@ __global__ void qk_norm_rope_kv_write_kernel(
   }
 }
 
+// The same for head sizes that are a multiple of 8 (every size in steps of 16 is): a lane
+// takes 4 consecutive elements of the first half of a head and the 4 that pair with them
+// under the rotation, LPH = the next power of two >= hd / 8 lanes work on a head and a wave
+// takes 64 / LPH heads of one token, so that loads and stores are 8 or 16 bytes wide and
+// there are far fewer waves than (token, head) pairs.
+template <typename T, int LPH>
+__global__ __launch_bounds__(64) void qk_norm_rope_kv_write_vec_kernel(
+    T* __restrict__ qkv, const float* __restrict__ q_gain, const float* __restrict__ k_gain,
+    float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int* __restrict__ positions, const int* __restrict__ slot_mapping,
+    T* __restrict__ k_pool, T* __restrict__ v_pool, T* __restrict__ q_out, int nH, int nKV,
+    int hd, int page_size, int tiled) {
+  constexpr int HPW = 64 / LPH;
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x, li = lane % LPH;
+  const int head = blockIdx.y * HPW + lane / LPH;
+  const int half = hd / 2;
+  const bool active = head < nH + 2 * nKV && 4 * li < half;
+  const int row_width = (nH + 2 * nKV) * hd;
+  T* src = qkv + (size_t)t * row_width + (size_t)min(head, nH + 2 * nKV - 1) * hd;
+  float x0[4] = {0.f, 0.f, 0.f, 0.f}, x1[4] = {0.f, 0.f, 0.f, 0.f};
+  if (active) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {     // consecutive: the compiler makes one load of each
+      x0[e] = load_as_float<T>(src + 4 * li + e);
+      x1[e] = load_as_float<T>(src + half + 4 * li + e);
+    }
+  }
+  const bool is_q = head < nH, is_v = head >= nH + nKV;
+  int slot = 0;
+  if (slot_mapping) slot = slot_mapping[t];
+  const int page = slot / page_size, r = slot % page_size;
+  if (is_v) {
+    if (!active || slot_mapping == nullptr) return;
+    T* blk = v_pool + ((size_t)page * nKV + (head - nH - nKV)) * page_size * hd;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int d0 = 4 * li + e, d1 = half + 4 * li + e;
+      if (tiled) {
+        T* grp = blk + (size_t)(r / 16) * 16 * hd + ((r % 16) / 4) * 64 + r % 4;
+        store_from_float<T>(grp + (d0 / 16) * 256 + (d0 % 16) * 4, x0[e]);
+        store_from_float<T>(grp + (d1 / 16) * 256 + (d1 % 16) * 4, x1[e]);
+      } else {
+        store_from_float<T>(blk + (size_t)d0 * page_size + r, x0[e]);
+        store_from_float<T>(blk + (size_t)d1 * page_size + r, x1[e]);
+      }
+    }
+    return;
+  }
+  // query and key heads (lanes of value heads have left: the shuffles below stay inside
+  // groups of LPH lanes, which are all of one head)
+  const float* gain = is_q ? q_gain : k_gain;
+  if (gain) {
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ss += x0[e] * x0[e] + x1[e] * x1[e];
+#pragma unroll
+    for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
+    if (active) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        x0[e] = x0[e] * inv * gain[4 * li + e];
+        x1[e] = x1[e] * inv * gain[half + 4 * li + e];
+      }
+    }
+  }
+  if (!active) return;
+  if (cos_t) {
+    const int pos = positions[t];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float c = cos_t[(size_t)pos * half + 4 * li + e], sn = sin_t[(size_t)pos * half + 4 * li + e];
+      const float r0 = x0[e] * c - x1[e] * sn;
+      const float r1 = x1[e] * c + x0[e] * sn;
+      x0[e] = r0;
+      x1[e] = r1;
+    }
+  }
+  T* dst0;
+  T* dst1;
+  if (is_q) {
+    T* base = q_out ? q_out + (size_t)t * nH * hd + (size_t)head * hd : src;
+    dst0 = base + 4 * li;
+    dst1 = base + half + 4 * li;
+  } else if (slot_mapping) {
+    T* blk = k_pool + ((size_t)page * nKV + (head - nH)) * page_size * hd;
+    if (tiled) {      // element d of row r: [d / 32][16 * ((d % 32) / 8) + r % 16][d % 8]
+      T* grp = blk + (size_t)(r / 16) * 16 * hd;
+      const int d0 = 4 * li, d1 = half + 4 * li;
+      dst0 = grp + (d0 / 32) * 512 + (((d0 % 32) / 8) * 16 + r % 16) * 8 + d0 % 8;
+      dst1 = grp + (d1 / 32) * 512 + (((d1 % 32) / 8) * 16 + r % 16) * 8 + d1 % 8;
+    } else {
+      dst0 = blk + (size_t)r * hd + 4 * li;
+      dst1 = blk + (size_t)r * hd + half + 4 * li;
+    }
+  } else {
+    dst0 = src + 4 * li;
+    dst1 = src + half + 4 * li;
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    store_from_float<T>(dst0 + e, x0[e]);
+    store_from_float<T>(dst1 + e, x1[e]);
+  }
+}
+
+template <typename T>
+static void launch_qk_vec(T* qkv, const float* q_gain, const float* k_gain, float eps,
+                          const float* cos_t, const float* sin_t, const int* positions,
+                          const int* slot_mapping, T* k_pool, T* v_pool, T* q_out, int Tn, int nH,
+                          int nKV, int hd, int page_size, int tiled, hipStream_t stream) {
+  const int lanes = hd / 8, heads = nH + 2 * nKV;
+#define ZF_QKV(LPH)                                                                            \
+  hipLaunchKernelGGL((qk_norm_rope_kv_write_vec_kernel<T, LPH>),                               \
+                     dim3(Tn, (heads + 64 / LPH - 1) / (64 / LPH)), dim3(64), 0, stream, qkv,  \
+                     q_gain, k_gain, eps, cos_t, sin_t, positions, slot_mapping, k_pool,       \
+                     v_pool, q_out, nH, nKV, hd, page_size, tiled)
+  if (lanes <= 2) ZF_QKV(2);
+  else if (lanes <= 4) ZF_QKV(4);
+  else if (lanes <= 8) ZF_QKV(8);
+  else if (lanes <= 16) ZF_QKV(16);
+  else if (lanes <= 32) ZF_QKV(32);
+  else ZF_QKV(64);
+#undef ZF_QKV
+}
+
 extern "C" int zf_qk_norm_rope_kv_write(void* qkv, int dtype, const float* q_gain,
                                         const float* k_gain, float eps, const float* cos_t,
                                         const float* sin_t, const int* positions,
@@ -207,6 +334,17 @@ extern "C" int zf_qk_norm_rope_kv_write(void* qkv, int dtype, const float* q_gai
                                         int page_size, int tiled, hipStream_t stream) {
   if (T <= 0) return 0;
   if (tiled && (page_size % 16 != 0 || hd % 32 != 0)) return -2;
+  if (hd % 8 == 0 && hd <= 512) {
+    if (dtype == ZF_F32)
+      launch_qk_vec<float>((float*)qkv, q_gain, k_gain, eps, cos_t, sin_t, positions, slot_mapping,
+                           (float*)k_pool, (float*)v_pool, (float*)q_out, T, nH, nKV, hd,
+                           page_size, tiled, stream);
+    else
+      launch_qk_vec<bf16_t>((bf16_t*)qkv, q_gain, k_gain, eps, cos_t, sin_t, positions,
+                            slot_mapping, (bf16_t*)k_pool, (bf16_t*)v_pool, (bf16_t*)q_out, T, nH,
+                            nKV, hd, page_size, tiled, stream);
+    ZF_CHECK_LAUNCH();
+  }
   dim3 grid(T, nH + 2 * nKV);
   if (dtype == ZF_F32)
     hipLaunchKernelGGL(qk_norm_rope_kv_write_kernel<float>, grid, dim3(ZF_WAVE), 0, stream,
