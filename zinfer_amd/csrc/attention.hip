@@ -403,21 +403,16 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
     const int* __restrict__ q_start, const int* __restrict__ ctx_len, bf16_t* __restrict__ out,
     float scale_log2e, int window, int nH, int nKV, int ps, int max_pages, int skip_single,
     int q_tiles) {
-  // Workgroups are handed out in the order of blockIdx.x, kv heads fastest.  Under the causal
-  // bound the last query tiles have the longest key ranges.  A sequence's tiles come heavy
-  // half first, descending, then the light half ascending: when all workgroups are resident
-  // at once (two per CU), the CU that got the heaviest tile in the first round gets the
-  // lightest in the second, and every CU ends up with about the same number of key tiles.
+  // workgroups are handed out in the order of blockIdx.x: kv heads vary fastest and the
+  // last query tiles (the longest key ranges under the causal bound) come first, so the
+  // heavy tiles do not end up as the tail
   const int kvh = blockIdx.x % nKV;
-  const int order = (blockIdx.x / nKV) % q_tiles;
+  const int qt = q_tiles - 1 - (blockIdx.x / nKV) % q_tiles;
   const int s = blockIdx.x / (nKV * q_tiles);
   const int q_len = q_start[s + 1] - q_start[s];
   if (q_len == 1 && skip_single) return;
-  const int own_tiles = (q_len + 31) / 32;
-  if (order >= own_tiles) return;
-  const int heavy = (own_tiles + 1) / 2;
-  const int qt = order < heavy ? own_tiles - 1 - order : order - heavy;
   const int qbase = qt * 32;
+  if (qbase >= q_len) return;
   const int ctx = ctx_len[s];
   const int pos0 = ctx - q_len + qbase;              // position of the tile's first query
   const int nq = min(32, q_len - qbase);
