@@ -362,14 +362,18 @@ def test_paged_attention_mixed_batch(dtype, nH, nKV, hd, page_size, window):
 @pytest.mark.parametrize("nH,nKV,hd,page_size,window", [
     (8, 2, 32, 16, 0), (32, 8, 128, 16, 0), (6, 6, 64, 32, 0), (16, 1, 64, 16, 0),
     (9, 3, 256, 16, 0), (8, 2, 64, 16, 37), (4, 4, 128, 48, 300), (36, 4, 32, 16, 0)])
-@pytest.mark.parametrize("kind", ["decode", "prefill", "mixed"])
+@pytest.mark.parametrize("kind", ["decode", "prefill", "mixed", "whole"])
 def test_paged_attention_mfma(nH, nKV, hd, page_size, window, kind):
     """The bfloat16 MFMA kernels: decode tokens over contexts that end at, before and after a
-    split's and a page's edge; portions that start mid-context; both in one batch."""
+    split's and a page's edge; portions that start mid-context; both in one batch; whole
+    prompts (where the waves of a head split its key tiles between them)."""
     dtype = torch.bfloat16
     if kind == "decode":
         ctx_lens = [1, 15, 16, 17, 255, 256, 257, 600, 1025]
         q_lens = [1] * len(ctx_lens)
+    elif kind == "whole":
+        ctx_lens = [37, 150, 64, 300, 2, 257]
+        q_lens = list(ctx_lens)
     elif kind == "prefill":
         ctx_lens = [37, 150, 64, 129, 700, 2]
         q_lens = [37, 50, 33, 129 - 100, 200, 2]

@@ -402,7 +402,8 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
     const bf16_t* __restrict__ v_pool, const int* __restrict__ block_table,
     const int* __restrict__ q_start, const int* __restrict__ ctx_len, bf16_t* __restrict__ out,
     float scale_log2e, int window, int nH, int nKV, int ps, int max_pages, int skip_single,
-    int q_tiles) {
+    int q_tiles, int nsplit) {
+  extern __shared__ float xch[];      // partials of the waves that took other key tiles
   // workgroups are handed out in the order of blockIdx.x: kv heads vary fastest and the
   // last query tiles (the longest key ranges under the causal bound) come first, so the
   // heavy tiles do not end up as the tail
@@ -424,10 +425,16 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
   const int p_j = pos0 + min(j, nq - 1);
   const int lo_j = (window > 0 && p_j - window + 1 > 0) ? p_j - window + 1 : 0;
   const int lo_min = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int lo_top = (window > 0 && p_max - window + 1 > 0) ? p_max - window + 1 : 0;
   const int* table = block_table + (size_t)s * max_pages;
   const int t_row = q_start[s] + qbase + min(j, nq - 1);
 
-  for (int g = wave; g < G; g += nwaves) {
+  // With few query heads per kv head the waves also split the key tiles of a head between
+  // them (wave `split` takes tiles split, split + nsplit, ...): under the causal bound the
+  // longest chain of dependent tiles, which is what the kernel's time follows, gets nsplit
+  // times shorter.  The partials are combined through LDS in split order.
+  const int head_waves = nwaves / nsplit, split = wave / head_waves;
+  for (int g = wave % head_waves; g < G; g += head_waves) {
     const int head = kvh * G + g;
     bf16x8_t qf[HD / 16];
     {
@@ -459,10 +466,10 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
       for (int stp = 0; stp < HD / 16; ++stp)
         dst[stp] = *(const u32x4_t*)(kblk + (stp / 2) * 512 + (stp % 2) * 256);
     };
-    const int kb0 = (lo_min / 32) * 32;
+    const int kb0 = (lo_min / 32) * 32 + 32 * split, kstep = 32 * nsplit;
     u32x4_t kf[HD / 16];
     load_keys(kb0, kf);
-    for (int kb = kb0; kb <= p_max; kb += 32) {
+    for (int kb = kb0; kb <= p_max; kb += kstep) {
       // values of this tile: keys kb + 16 u .. + 15 (one page) for u = 0, 1
       u32x2_t vf[2][HD / 32][2];
       bool any[2];
@@ -489,15 +496,24 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
 #pragma unroll
       for (int stp = 0; stp < HD / 16; ++stp)
         st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&kf[stp], qf[stp], st, 0, 0, 0);
-      if (kb + 32 <= p_max) load_keys(kb + 32, kf);      // next tile's keys, in flight from here
+      if (kb + kstep <= p_max) load_keys(kb + kstep, kf);   // next tile's keys, in flight from here
       // st[r]: key kb + 8 (r / 4) + 4 hf + r % 4, query column j
       float tmax = -INFINITY;
+      if (kb + 31 <= pos0 && kb >= lo_top) {
+        // every key of the tile is visible to every query of the wave: nothing to mask
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int key = kb + 8 * (r / 4) + 4 * hf + r % 4;
-        const float v = (key <= p_j && key >= lo_j) ? st[r] * scale_log2e : -INFINITY;
-        st[r] = v;
-        tmax = fmaxf(tmax, v);
+        for (int r = 0; r < 16; ++r) {
+          st[r] *= scale_log2e;
+          tmax = fmaxf(tmax, st[r]);
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = kb + 8 * (r / 4) + 4 * hf + r % 4;
+          const float v = (key <= p_j && key >= lo_j) ? st[r] * scale_log2e : -INFINITY;
+          st[r] = v;
+          tmax = fmaxf(tmax, v);
+        }
       }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
       const float m_new = fmaxf(m, tmax);
@@ -513,10 +529,12 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
       psum += __shfl_xor(psum, 32, 64);
       l = l * corr + psum;
       m = m_new;
+      if (__any(corr != 1.0f)) {      // after the first tiles the maxima rarely move
 #pragma unroll
-      for (int dt = 0; dt < HD / 32; ++dt)
+        for (int dt = 0; dt < HD / 32; ++dt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[dt][r] *= corr;
+          for (int r = 0; r < 16; ++r) o[dt][r] *= corr;
+      }
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         // slots e = 0..7 <-> st[8 u + e]: keys kb + 16 u + 4 hf + e (e < 4) and
@@ -543,6 +561,33 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
         }
       }
     }
+    if (nsplit > 1) {     // one pass over g here: every wave comes by exactly once
+      constexpr int PER_LANE = HD / 2 + 2;       // a wave's O^T values per lane, max and sum
+      if (split > 0) {
+        float* dst = xch + (size_t)((split - 1) * head_waves + g) * PER_LANE * 64 + lane;
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) dst[(dt * 16 + r) * 64] = o[dt][r];
+        dst[(HD / 2) * 64] = m;
+        dst[(HD / 2 + 1) * 64] = l;
+      }
+      __syncthreads();
+      if (split > 0) continue;
+      for (int t = 1; t < nsplit; ++t) {
+        const float* src = xch + (size_t)((t - 1) * head_waves + g) * PER_LANE * 64 + lane;
+        const float m_t = src[(HD / 2) * 64], l_t = src[(HD / 2 + 1) * 64];
+        const float m_new = fmaxf(m, m_t);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float ca = exp2f(m - m_use), cb = exp2f(m_t - m_use);
+        l = l * ca + l_t * cb;
+        m = m_new;
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[dt][r] = o[dt][r] * ca + src[(dt * 16 + r) * 64] * cb;
+      }
+    }
     if (q_valid) {
       const float inv = 1.0f / l;
       bf16_t* orow = out + ((size_t)t_row * nH + head) * HD;
@@ -564,19 +609,35 @@ extern "C" int zf_attn_prefill_bf16(const void* q, const void* k_pool, const voi
                                     const int* ctx_len, void* out, float scale, int window,
                                     int n_seqs, int max_q_len, int nH, int nKV, int hd,
                                     int page_size, int max_pages, int skip_single,
-                                    hipStream_t stream) {
+                                    int allow_split, hipStream_t stream) {
   if (n_seqs <= 0 || max_q_len <= 0) return 0;
   if (page_size % 16 != 0 || nKV <= 0 || nH % nKV != 0) return -2;
   const float scale_log2e = scale * 1.4426950408889634f;
   const int G = nH / nKV;
   const int q_tiles = (max_q_len + 31) / 32;
   dim3 grid((unsigned)n_seqs * q_tiles * nKV);
-  dim3 block(64 * (G < 8 ? G : 8));
+  // up to 8 waves: one per query head of the kv head, and with 4 heads or fewer several
+  // waves per head that split its key tiles, as far as the partials fit into LDS
+  // (allow_split: the caller expects short contexts before the portions, where the causal
+  // bound leaves the tiles most unequal, and a grid that does not fill the chip many times)
+  int nsplit = (allow_split && G <= 4 && grid.x <= 1024) ? 8 / G : 1;
+  const size_t per_wave = (size_t)(hd / 2 + 2) * 64 * sizeof(float);
+  while (nsplit > 1 && (size_t)(nsplit - 1) * G * per_wave > 144 * 1024) --nsplit;
+  const int head_waves = G < 8 ? G : 8;
+  dim3 block(64 * head_waves * nsplit);
+  const size_t smem = nsplit > 1 ? (size_t)(nsplit - 1) * G * per_wave : 0;
 #define ZF_PRE(HD)                                                                              \
-  hipLaunchKernelGGL(attn_prefill_kernel<HD>, grid, block, 0, stream, (const bf16_t*)q,         \
-                     (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, q_start,        \
-                     ctx_len, (bf16_t*)out, scale_log2e, window, nH, nKV, page_size, max_pages, \
-                     skip_single, q_tiles)
+  do {                                                                                          \
+    if (smem > 64 * 1024) {                                                                     \
+      hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_kernel<HD>,                  \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
+      if (e != hipSuccess) return (int)e;                                                       \
+    }                                                                                           \
+    hipLaunchKernelGGL(attn_prefill_kernel<HD>, grid, block, smem, stream, (const bf16_t*)q,    \
+                       (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, q_start,      \
+                       ctx_len, (bf16_t*)out, scale_log2e, window, nH, nKV, page_size,          \
+                       max_pages, skip_single, q_tiles, nsplit);                                \
+  } while (0)
   if (hd == 32) ZF_PRE(32);
   else if (hd == 64) ZF_PRE(64);
   else if (hd == 128) ZF_PRE(128);

@@ -486,7 +486,8 @@ def paged_attention(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index,
                 _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), _ptr(q_start),
                 _ptr(ctx_len), _ptr(out), ctypes.c_float(scale), int(window), n_seqs,
                 max_q_len, n_heads, n_kv_heads, head_dim, page_size, max_pages,
-                1 if n_single != 0 else 0, _stream()), "paged_attention (prefill)")
+                1 if n_single != 0 else 0, 1 if max_ctx_len <= 2 * max_q_len else 0,
+                _stream()), "paged_attention (prefill)")
         return
     _check(lib.zf_paged_attention_wave(
         _ptr(q), _ptr(k_pool), _ptr(v_pool), _dt(q), _ptr(block_table), _ptr(q_start),
