@@ -382,10 +382,15 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
     }
   };
 
-  const int ktiles = K / TK;
-  gload_a(0);
+  // gridDim.y workgroups share a tile's k-tiles (split-K for products with few tiles); each
+  // then leaves a float32 partial [gridDim.y, M, N] in Cv for skinny_reduce_kernel
+  const int kt_all = K / TK;
+  const int kt0 = (int)((long long)blockIdx.y * kt_all / gridDim.y);
+  const int ktiles = (int)((long long)(blockIdx.y + 1) * kt_all / gridDim.y);
+  if (gridDim.y > 1) Cv = (float*)Cv + (size_t)blockIdx.y * M * N;
+  gload_a(kt0 * TK);
 #pragma unroll
-  for (int ks = 0; ks < TK / 16; ++ks) gload_w(0, ks);
+  for (int ks = 0; ks < TK / 16; ++ks) gload_w(kt0, ks);
   lstore(0);
   __syncthreads();
   // One k-tile per trip: MFMAs on LDS stage `kt & 1`; meanwhile the tokens of tile kt + 1
@@ -394,8 +399,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
   // the loads (the last trip loads its own tile once more), so the compiler can count the
   // loads in flight and waits for no younger one; the scheduling barriers keep it from
   // sinking the loads down to their first use, which would expose their whole latency.
-  for (int kt = 0; kt < ktiles; ++kt) {
-    const int stage = kt & 1;
+  for (int kt = kt0; kt < ktiles; ++kt) {
+    const int stage = (kt - kt0) & 1;
     const int nxt = min(kt + 1, ktiles - 1);
     gload_a(nxt * TK);
     __builtin_amdgcn_sched_barrier(0);
@@ -499,13 +504,20 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
   }
 }
 
+// adds the float32 partials [ksplit, M, N] in split order and applies the epilogue (defined
+// with the weight-streaming kernel below)
+static int launch_reduce(const void* ws, void* C, int M, int N, int ksplit, int epi,
+                         hipStream_t stream);
+
 template <int BM, int BN, int WM, int WN>
 static int launch_tile_wdirect(const void* A, const void* W, void* C, int M, int N, int K, int epi,
-                               hipStream_t stream) {
+                               hipStream_t stream, void* ws = nullptr, int ksplit = 1) {
   if (N % 16 != 0 || K % 64 != 0) return -3;
+  if (ksplit > 1 && (ws == nullptr || epi == EPI_SWIGLU || ksplit > K / 64)) return -3;
   constexpr int NT = (BM / WM) * (BN / WN) * 64;
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  const dim3 grid(tiles_m * tiles_n), block(NT);
+  const dim3 grid(tiles_m * tiles_n, ksplit), block(NT);
+  const int final_epi = epi;
   const size_t smem = (size_t)2 * BM * LDS_ROW * sizeof(bf16_t);
 #define ZF_WD(E)                                                                              \
   do {                                                                                        \
@@ -518,11 +530,17 @@ static int launch_tile_wdirect(const void* A, const void* W, void* C, int M, int
     hipLaunchKernelGGL(kern, grid, block, smem, stream, (const bf16_t*)A, (const bf16_t*)W, C, \
                        M, N, K, tiles_m, tiles_n);                                            \
   } while (0)
+  void* const final_c = C;
+  if (ksplit > 1) {
+    epi = EPI_STORE_F32;
+    C = ws;
+  }
   if (epi == EPI_STORE_BF16) ZF_WD(EPI_STORE_BF16);
   else if (epi == EPI_STORE_F32) ZF_WD(EPI_STORE_F32);
   else if (epi == EPI_SWIGLU) ZF_WD(EPI_SWIGLU);
   else ZF_WD(EPI_ACC_F32);
 #undef ZF_WD
+  if (ksplit > 1) return launch_reduce(ws, final_c, M, N, ksplit, final_epi, stream);
   return (int)hipGetLastError();
 }
 
@@ -600,6 +618,16 @@ struct SkinnyNorm {
   bf16_t* xg_out;
   float* sq_out;
 };
+
+// The 128 x 128 tiled product on pre-tiled W with ksplit workgroups per tile along K, for
+// products whose tiles alone do not fill the chip (a few hundred tokens, a narrow output).
+// ws: float32 [ksplit, M, N]; epi: store bf16, store f32 or add into f32.
+extern "C" int zf_gemm_bf16_tile_splitk(const void* A, const void* W, void* C, void* ws, int M,
+                                        int N, int K, int epi, int ksplit, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (ksplit < 2 || ksplit > 64 || epi == EPI_SWIGLU) return -3;
+  return launch_tile_wdirect<128, 128, 64, 64>(A, W, C, M, N, K, epi, stream, ws, ksplit);
+}
 
 // ---------------------------------------------------------------- small M: weight streaming
 // For M <= 64 the product is bound by reading W once from HBM.  A workgroup owns 16 * RG rows
@@ -872,6 +900,24 @@ __global__ void skinny_reduce_kernel(const float* __restrict__ ws, void* __restr
     ((float*)Cv)[i] += s;
 }
 
+static int launch_reduce(const void* ws, void* C, int M, int N, int ksplit, int epi,
+                         hipStream_t stream) {
+  const size_t mn = (size_t)M * N;
+  const unsigned blocks = (unsigned)((mn + 255) / 256);
+  if (epi == EPI_STORE_BF16)
+    hipLaunchKernelGGL(skinny_reduce_kernel<EPI_STORE_BF16>, dim3(blocks), dim3(256), 0, stream,
+                       (const float*)ws, C, mn, ksplit);
+  else if (epi == EPI_STORE_F32)
+    hipLaunchKernelGGL(skinny_reduce_kernel<EPI_STORE_F32>, dim3(blocks), dim3(256), 0, stream,
+                       (const float*)ws, C, mn, ksplit);
+  else if (epi == EPI_ACC_F32)
+    hipLaunchKernelGGL(skinny_reduce_kernel<EPI_ACC_F32>, dim3(blocks), dim3(256), 0, stream,
+                       (const float*)ws, C, mn, ksplit);
+  else
+    return -3;
+  return (int)hipGetLastError();
+}
+
 template <int MT, int RG, bool WT, int NORM = NORM_NONE, bool EMIT = false>
 static int launch_skinny(const void* A, const void* W, void* C, void* ws, int M, int N, int K,
                          int epi, int ksplit, hipStream_t stream, SkinnyNorm nrm = SkinnyNorm{}) {
@@ -900,19 +946,7 @@ static int launch_skinny(const void* A, const void* W, void* C, void* ws, int M,
   else
     hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_ACC_F32, WT, NORM_NONE, NW>), grid, block, 0,
                        stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K, nrm);
-  if (ksplit > 1) {
-    const size_t mn = (size_t)M * N;
-    const unsigned blocks = (unsigned)((mn + 255) / 256);
-    if (epi == EPI_STORE_BF16)
-      hipLaunchKernelGGL(skinny_reduce_kernel<EPI_STORE_BF16>, dim3(blocks), dim3(256), 0, stream,
-                         (const float*)ws, C, mn, ksplit);
-    else if (epi == EPI_STORE_F32)
-      hipLaunchKernelGGL(skinny_reduce_kernel<EPI_STORE_F32>, dim3(blocks), dim3(256), 0, stream,
-                         (const float*)ws, C, mn, ksplit);
-    else
-      hipLaunchKernelGGL(skinny_reduce_kernel<EPI_ACC_F32>, dim3(blocks), dim3(256), 0, stream,
-                         (const float*)ws, C, mn, ksplit);
-  }
+  if (ksplit > 1) return launch_reduce(ws, C, M, N, ksplit, epi, stream);
   return (int)hipGetLastError();
 }
 

@@ -236,6 +236,17 @@ def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = Fals
     return 4 if tiles >= 160 else 0
 
 
+def _tile_ksplit(M: int, N: int, K: int) -> int:
+    """Workgroups per 128 x 128 tile along K: products of a few hundred tokens on a narrow
+    output have too few tiles for 256 CUs; split them until about 512 workgroups run, each
+    keeping at least 8 k-tiles.  The partials cost ksplit * M * N floats of traffic."""
+    tiles = ((M + 127) // 128) * ((N + 127) // 128)
+    if tiles >= 192:
+        return 1
+    ksplit = min(512 // tiles, K // 64 // 8, 16)
+    return ksplit if ksplit >= 2 else 1
+
+
 def can_pretile(w: torch.Tensor) -> bool:
     return w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[0] % 64 == 0 \
         and w.shape[1] % 64 == 0
@@ -283,6 +294,13 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
                                            rg, ks, 1 if w_tiled else 0, _stream()),
                    "gemm (weight streaming)")
         else:
+            ksplit = _tile_ksplit(M, N, K) if w_tiled else 1
+            if ksplit > 1:
+                ws = _workspace("gemm_splitk", ksplit * M * N, torch.float32, a.device)
+                _check(lib.zf_gemm_bf16_tile_splitk(_ptr(a), _ptr(w), _ptr(out), _ptr(ws), M, N,
+                                                    K, epi, ksplit, _stream()),
+                       "gemm (tiled, split along K)")
+                return
             _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, epi,
                                          _tile_variant(M, N, w_tiled, accumulate),
                                          1 if w_tiled else 0, _stream()),
