@@ -234,3 +234,19 @@ def test_decode_steps_in_a_row_shrink_to_the_free_pages_and_skip_penalties():
                                          max_new_tokens=6, ignore_eos=True))
     s.run()
     assert not eng.runs
+
+
+def test_abort_gives_everything_back():
+    eng = FakeEngine(num_pages=16)
+    s = Scheduler(eng, max_step_tokens=8, max_seqs=1)
+    a = s.add_request([1, 2, 3], SamplingParams(max_new_tokens=50, **GREEDY))
+    b = s.add_request([7, 8], SamplingParams(max_new_tokens=4, **GREEDY))      # waits: one slot
+    s.step(); s.step()
+    assert s.request(a).generated == [4, 5] and s.request(b) in s.waiting
+    s.abort(b, "stop")                       # from the waiting queue
+    req = s.abort(a, "stop")                 # while running
+    assert req.finished and req.finish_reason == "stop" and req.generated == [4, 5]
+    assert not s.has_work() and eng.cache.num_free_pages() == [16] and not eng.cache.requests
+    assert s.abort(a) is req                 # once more: nothing happens
+    with pytest.raises(KeyError):
+        s.request("nobody")

@@ -3,9 +3,10 @@
 `src/app/cli/args.zig:91-148,352-501` positional forms, presets and flags): sub-commands by
 name, ``[model_dir]`` first and optional, then the prompt, ``max_new_tokens``,
 ``think|no-think``, then ``--flag value`` pairs with the reference's names and meanings.
-Prompts are token ids (``1,2,3``); text is out of this engine's scope.  Options the reference
-has for things this engine does not build (quantised backends and caches, CPU threads) are
-parsed and refused or ignored with a message.
+Prompts are token ids (``1,2,3``), or text when the model folder brings a tokenizer
+(``tokenizer.json``, or ``vocab.json`` + ``merges.txt`` + ``tokenizer_config.json``).  Options
+the reference has for things this engine does not build (quantised backends and caches, CPU
+threads) are parsed and refused or ignored with a message.
 """
 from __future__ import annotations
 
@@ -20,7 +21,12 @@ USAGE = """Usage:
   zinfer inspect-weights [model_dir]
   zinfer inspect-tensor [model_dir] <tensor_name> [count]
   zinfer generate-token-ids [model_dir] <seed_ids_csv> <steps>
-  zinfer generate [model_dir] <ids_csv> [max_new_tokens] [think|no-think] [flags...]
+  zinfer generate [model_dir] <text|ids_csv> [max_new_tokens] [think|no-think] [flags...]
+  zinfer generate-chat [model_dir] <messages_json_path> [max_new_tokens] [think|no-think] [flags...]
+  zinfer tokenize [model_dir] <text>
+  zinfer decode-ids [model_dir] <ids_csv>
+  zinfer serve-batch [model_dir] --requests <file.jsonl> [--out <file.jsonl>] [flags...]
+  zinfer replay --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N   (steps on stdin)
   zinfer bench [model_dir] <ids_csv> [max_new_tokens]
   zinfer bench-batch [model_dir] <ids_csv> <batch_size> [max_new_tokens]
   zinfer bench-continuous [model_dir] <ids_csv> <batch_size> <total_requests> [max_new_tokens]
@@ -29,12 +35,13 @@ USAGE = """Usage:
 
 Defaults:
   model_dir = models/Qwen3-0.6B
-  generate max_new_tokens = 64, bench max_new_tokens = 16
+  generate max_new_tokens = 64, generate-chat max_new_tokens = 128, bench max_new_tokens = 16
 
 Flags:
   --seed <u64>                 --temperature <f32>        --top-p <f32>
   --top-k <usize>              --min-p <f32>              --presence-penalty <f32>
   --frequency-penalty <f32>    --repetition-penalty <f32> --stream
+  --system <text>              --stop <text> (repeatable; text prompts only)
   --backend <auto|bf16>        --kv-cache <auto|bf16|fp32>
   --threads <usize>            (accepted, unused: the GPU grid replaces the thread pool)
   --dtype <bfloat16|float32>   --page-size <n>            --max-tokens <n>
@@ -77,6 +84,8 @@ class Options:
         self.think = think
         self.sampling = thinking_defaults(think)        # `args.zig:352-373`
         self.stream = False
+        self.stop: List[str] = []                       # `args.zig:433-436`
+        self.system: Optional[str] = None
         self.kv_cache = "auto"
         self.dtype = "bfloat16"
         self.page_size = 16
@@ -120,6 +129,10 @@ def parse_flags(flags: List[str], opt: Options) -> None:
             opt.sampling.seed = opt.seed
         elif a == "--stream":
             opt.stream = True
+        elif a == "--stop":
+            opt.stop.append(value())
+        elif a == "--system":
+            opt.system = value()
         elif a == "--backend":
             v = value()
             if v in ("q8", "q6", "q4"):
@@ -161,9 +174,14 @@ def parse_flags(flags: List[str], opt: Options) -> None:
         i += 1
 
 
-def parse_generate(args: List[str], default_new: int) -> Tuple[str, List[int], Options]:
-    """``[model_dir] <ids> [max_new_tokens] [think|no-think] [flags]``: the model folder is
-    there when the third positional is a number (`args.zig:100-131`)."""
+def _looks_like_ids(text: str) -> bool:
+    return bool(text) and all(c.isdigit() or c in ", " for c in text) and any(c.isdigit() for c in text)
+
+
+def parse_generate_text(args: List[str], default_new: int) -> Tuple[str, str, Options]:
+    """``[model_dir] <prompt> [max_new_tokens] [think|no-think] [flags]``: the model folder is
+    there when the third positional is a number (`args.zig:100-131`).  The prompt stays a
+    string: token ids or text."""
     pos, flags = _split_flags(args)
     if not pos:
         raise CliError("InvalidCommand: a prompt is needed")
@@ -172,7 +190,7 @@ def parse_generate(args: List[str], default_new: int) -> Tuple[str, List[int], O
         model_dir, pos = pos[0], pos[1:]
     elif len(pos) >= 2 and not pos[1].isdigit() and pos[1] not in ("think", "no-think"):
         model_dir, pos = pos[0], pos[1:]
-    ids = parse_token_ids(pos[0])
+    prompt = pos[0]
     rest = pos[1:]
     max_new = default_new
     if rest and rest[0].isdigit():
@@ -190,7 +208,13 @@ def parse_generate(args: List[str], default_new: int) -> Tuple[str, List[int], O
     parse_flags(flags, opt)
     opt.sampling.max_new_tokens = opt.max_new_tokens
     opt.sampling.ignore_eos = opt.ignore_eos
-    return model_dir, ids, opt
+    return model_dir, prompt, opt
+
+
+def parse_generate(args: List[str], default_new: int) -> Tuple[str, List[int], Options]:
+    """The same with a prompt of token ids."""
+    model_dir, prompt, opt = parse_generate_text(args, default_new)
+    return model_dir, parse_token_ids(prompt), opt
 
 
 def _llm(model_dir: str, opt: Options, max_tokens: Optional[int] = None):
@@ -296,8 +320,17 @@ def cmd_generate_token_ids(args: List[str]) -> int:
 
 
 def cmd_generate(args: List[str]) -> int:
-    """`src/app/cli/generate.zig:7-37` with token ids in place of text."""
-    model_dir, ids, opt = parse_generate(args, 64)
+    """`src/app/cli/generate.zig:7-37`: a text prompt goes through the family's chat template
+    and the tokenizer and the answer is printed as text; a prompt of token ids is run as it is
+    and the answer is printed as ids."""
+    model_dir, prompt, opt = parse_generate_text(args, 64)
+    if not _looks_like_ids(prompt):
+        from .text import render_single_user
+        print("Zinfer generate")
+        print(f"mode: {'think' if opt.think else 'no-think'}")
+        print(f"prompt: {prompt}")
+        return _generate_text(model_dir, render_single_user(prompt, opt.think, opt.system), opt)
+    ids = parse_token_ids(prompt)
     if not ids:
         raise CliError("EmptyPrompt")
     llm = _llm(model_dir, opt, max_tokens=(len(ids) + opt.max_new_tokens + 63) // 64 * 64)
@@ -310,13 +343,177 @@ def cmd_generate(args: List[str]) -> int:
     shown = 0
     while sched.has_work():
         sched.step()
-        req = sched.finished.get(rid) or next(r for r in sched.running + list(sched.waiting)
-                                              if r.id == rid)
+        req = sched.request(rid)
         for t in req.generated[shown:]:
             sys.stdout.write(("," if shown else "") + str(t))
             sys.stdout.flush()
             shown += 1
     sys.stdout.write("\n")
+    return 0
+
+
+def _generate_text(model_dir: str, prompt_text: str, opt: Options) -> int:
+    """Encodes the rendered prompt, generates until an end-of-sequence id, the token limit or
+    a stop sequence (the family's defaults and ``--stop``), and prints the answer, piece by
+    piece with ``--stream`` (`src/app/cli/runtime/generator.zig:60-140`,
+    `runtime/streaming.zig:41-65`)."""
+    from .text import Tokenizer, analyze_generated_text, effective_stop_sequences
+    tok = Tokenizer.from_dir(model_dir)
+    ids = tok.encode(prompt_text)
+    if not ids:
+        raise CliError("EmptyPrompt")
+    llm = _llm(model_dir, opt, max_tokens=(len(ids) + opt.max_new_tokens + 63) // 64 * 64)
+    stops = effective_stop_sequences(llm.model.spec.default_stop_sequences, opt.stop)
+    sched = llm.new_scheduler()
+    rid = sched.add_request(ids, opt.sampling)
+    sys.stdout.write("response: ")
+    printed, response, seen = 0, None, 0
+    while sched.has_work() and response is None:
+        sched.step()
+        generated = sched.request(rid).generated
+        # token by token, as the reference looks at its text: a step may bring several
+        for k in range(seen + 1, len(generated) + 1):
+            text = tok.decode(generated[:k])
+            printable, hit, response_len = analyze_generated_text(text, stops)
+            if opt.stream and printable > printed:
+                sys.stdout.write(text[printed:printable])
+                sys.stdout.flush()
+                printed = printable
+            if hit:
+                response = text[:response_len]
+                sched.abort(rid, "stop")
+                break
+        seen = len(generated)
+    if response is None:
+        response = tok.decode(sched.request(rid).generated)
+    if opt.stream:
+        sys.stdout.write(response[printed:])
+    else:
+        sys.stdout.write(response)
+    sys.stdout.write("\n")
+    return 0
+
+
+def cmd_generate_chat(args: List[str]) -> int:
+    """`src/app/cli/generate.zig:39-75`: the prompt is a JSON file of messages."""
+    model_dir, path, opt = parse_generate_text(args, 128)
+    from .text.chat import load_messages, render_messages, with_system
+    messages = with_system(load_messages(path), opt.system)
+    print("Zinfer generate-chat")
+    print(f"mode: {'think' if opt.think else 'no-think'}")
+    print(f"messages_path: {path}")
+    return _generate_text(model_dir, render_messages(messages, opt.think), opt)
+
+
+def _dir_and_one(args: List[str], what: str) -> Tuple[str, str]:
+    pos, flags = _split_flags(args)
+    if flags or len(pos) not in (1, 2):
+        raise CliError(f"InvalidCommand: [model_dir] <{what}>")
+    return (pos[0], pos[1]) if len(pos) == 2 else (DEFAULT_MODEL_DIR, pos[0])
+
+
+def cmd_tokenize(args: List[str]) -> int:
+    """`src/app/cli/tools/text.zig:5-36`."""
+    from .text import Tokenizer
+    model_dir, text = _dir_and_one(args, "text")
+    ids = Tokenizer.from_dir(model_dir).encode(text)
+    print("Zinfer tokenize")
+    print(f"text: {text}")
+    print("ids: [" + ", ".join(str(i) for i in ids) + "]")
+    return 0
+
+
+def cmd_decode_ids(args: List[str]) -> int:
+    """`src/app/cli/tools/text.zig:38-75`."""
+    from .text import Tokenizer
+    model_dir, csv = _dir_and_one(args, "ids_csv")
+    ids = parse_token_ids(csv)
+    print("Zinfer decode-ids")
+    print("ids: [" + ", ".join(str(i) for i in ids) + "]")
+    print(f"text: {Tokenizer.from_dir(model_dir).decode(ids)}")
+    return 0
+
+
+def cmd_serve_batch(args: List[str]) -> int:
+    """Runs the scheduler over a file of requests, one JSON object a line:
+    ``{"id": ..., "prompt": [ids] | "text": "...", "max_new_tokens": n, "temperature": ...,
+    "top_k": ..., "top_p": ..., "min_p": ..., "seed": ..., "ignore_eos": bool}``; unknown keys
+    are an error, missing ones take the command's flags.  Writes one line per request,
+    in the order they finish: ``{"id", "tokens", "finish_reason"[, "text"]}``.  The nearest
+    thing in the reference is its continuous-batch benchmark (`src/app/cli/tools/bench/
+    runtime.zig:226-310`), which admits the same prompt again and again."""
+    import json
+    from dataclasses import replace
+    pos, flags = _split_flags(args)
+    requests_path, out_path, rest = None, None, []
+    i = 0
+    while i < len(flags):
+        if flags[i] in ("--requests", "--out"):
+            if i + 1 >= len(flags):
+                raise CliError(f"MissingFlagValue: {flags[i]}")
+            if flags[i] == "--requests":
+                requests_path = flags[i + 1]
+            else:
+                out_path = flags[i + 1]
+            i += 2
+        else:
+            rest.append(flags[i])
+            i += 1
+    if requests_path is None or len(pos) > 1:
+        raise CliError("InvalidCommand: serve-batch [model_dir] --requests <file.jsonl>")
+    model_dir = pos[0] if pos else DEFAULT_MODEL_DIR
+    opt = Options(64)
+    opt.sampling = replace(opt.sampling, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0)
+    parse_flags(rest, opt)
+    opt.sampling.max_new_tokens = opt.max_new_tokens
+    opt.sampling.ignore_eos = opt.ignore_eos
+    allowed = {"id", "prompt", "text", "max_new_tokens", "temperature", "top_k", "top_p", "min_p",
+               "presence_penalty", "frequency_penalty", "repetition_penalty", "seed", "ignore_eos"}
+    tok = None
+    todo = []
+    with open(requests_path, "r", encoding="utf-8") as f:
+        for n, line in enumerate(f):
+            if not line.strip():
+                continue
+            raw = json.loads(line)
+            extra = set(raw) - allowed
+            if extra or ("prompt" in raw) == ("text" in raw):
+                raise CliError(f"InvalidRequest: line {n + 1}: one of prompt/text, no other keys "
+                               f"than {sorted(allowed)} (found {sorted(extra)})")
+            if "text" in raw:
+                if tok is None:
+                    from .text import Tokenizer
+                    tok = Tokenizer.from_dir(model_dir)
+                ids = tok.encode(raw["text"])
+            else:
+                ids = [int(t) for t in raw["prompt"]]
+            sp = replace(opt.sampling, **{k: raw[k] for k in raw if k not in ("id", "prompt", "text")})
+            todo.append((raw.get("id", n), ids, sp))
+    if not todo:
+        raise CliError("InvalidRequest: no requests")
+    llm = _llm(model_dir, opt)
+    sched = llm.new_scheduler()
+    for rid, ids, sp in todo:
+        sched.add_request(ids, sp, request_id=rid)
+    out = open(out_path, "w", encoding="utf-8") if out_path else sys.stdout
+    t0 = time.perf_counter()
+    n_tokens = 0
+    try:
+        while sched.has_work():
+            for req in sched.step():
+                rec = {"id": req.id, "tokens": req.generated, "finish_reason": req.finish_reason}
+                if tok is not None:
+                    rec["text"] = tok.decode(req.generated)
+                n_tokens += len(req.generated)
+                out.write(json.dumps(rec, ensure_ascii=False) + "\n")
+                out.flush()
+    finally:
+        if out_path:
+            out.close()
+    dt = time.perf_counter() - t0
+    print(f"serve-batch: {len(todo)} requests, {n_tokens} generated tokens, {dt:.3f} s, "
+          f"{n_tokens / dt:.1f} tok/s, {sched.n_steps} steps, {sched.n_preemptions} preemptions",
+          file=sys.stderr)
     return 0
 
 
@@ -474,6 +671,17 @@ def main(argv: Optional[List[str]] = None) -> int:
             return cmd_generate_token_ids(args)
         if cmd == "generate":
             return cmd_generate(args)
+        if cmd == "generate-chat":
+            return cmd_generate_chat(args)
+        if cmd == "tokenize":
+            return cmd_tokenize(args)
+        if cmd == "decode-ids":
+            return cmd_decode_ids(args)
+        if cmd == "serve-batch":
+            return cmd_serve_batch(args)
+        if cmd == "replay":
+            from .engine.replay import main as replay_main
+            return replay_main(args)
         if cmd in ("bench", "bench-batch", "bench-continuous"):
             return cmd_bench(args, cmd)
         if cmd == "random-model":
@@ -481,10 +689,10 @@ def main(argv: Optional[List[str]] = None) -> int:
         if cmd == "bench-ops":
             from .bench_ops import main as bench_ops_main
             return bench_ops_main(args)
-        if cmd in ("quantize", "tokenize", "decode-ids", "generate-chat", "chat", "probe-linear",
-                   "probe-block", "probe-model", "bench-suite"):
-            print(f"zinfer: {cmd!r} belongs to what this engine does not build (text front "
-                  "end, quantisation, CPU probes)", file=sys.stderr)
+        if cmd in ("quantize", "chat", "probe-linear", "probe-block", "probe-model",
+                   "bench-suite"):
+            print(f"zinfer: {cmd!r} belongs to what this engine does not build (interactive "
+                  "chat, quantisation, CPU probes)", file=sys.stderr)
             return 2
         print(f"zinfer: unknown command {cmd!r}\n", file=sys.stderr)     # `cli.zig:286`
         sys.stderr.write(USAGE)

@@ -99,6 +99,31 @@ class Scheduler:
     def has_work(self) -> bool:
         return bool(self.waiting or self.running)
 
+    def request(self, rid) -> Request:
+        """The request with this id, wherever it is."""
+        if rid in self.finished:
+            return self.finished[rid]
+        for req in list(self.running) + list(self.waiting):
+            if req.id == rid:
+                return req
+        raise KeyError(rid)
+
+    def abort(self, rid, reason: str = "aborted") -> Request:
+        """Ends a request from outside (a stop sequence in its text, a client that left): what
+        it holds is given back; the tokens it has generated stay."""
+        req = self.request(rid)
+        if req.finished:
+            return req
+        if req in self.running:
+            self._finish(req, reason)
+        else:
+            self.waiting.remove(req)
+            if self.cache.has_request(req.id):
+                self.cache.release(req.id)
+            req.finished, req.finish_reason = True, reason
+            self.finished[req.id] = req
+        return req
+
     # ------------------------------------------------------------------ planning
     def plan(self) -> List[PlannedEntry]:
         """Decides what the next step runs.  May preempt; admits from the waiting queue."""
