@@ -74,3 +74,34 @@ def test_generate_token_ids_through_the_command_line(tmp_path):
     got = json.loads(line[len("tokens: "):])
     want = prompt + plain.greedy_generate(tiny.CONFIGS["B"], tiny.weights_of("B"), prompt, 6)
     assert got == want
+
+
+@pytest.mark.gpu
+def test_random_weights_without_a_model_folder(tmp_path):
+    """``--config f --random-weights S`` and ``LLM.from_config`` draw what ``write_model_dir``
+    stores for the same seed, so the plain implementation over those tensors is the oracle."""
+    from zinfer_amd import LLM, SamplingParams
+    prompt = tiny.random_tokens(9, 512, 3)
+    want = plain.greedy_generate(tiny.CONFIGS["A"], tiny.weights_of("A"), prompt, 5)
+    llm = LLM.from_config(tiny.CONFIGS["A"], seed=tiny.SEEDS["A"], dtype="float32",
+                          max_tokens=128, max_seqs=2)
+    got = llm.generate([prompt], SamplingParams(temperature=0.0, max_new_tokens=5,
+                                                ignore_eos=True))[0]
+    assert got == want
+    cfg = tmp_path / "config.json"
+    cfg.write_text(json.dumps(tiny.CONFIGS["A"]))
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "zinfer"), "generate-token-ids",
+                        ",".join(map(str, prompt)), "5", "--dtype", "float32", "--config",
+                        str(cfg), "--random-weights", str(tiny.SEEDS["A"])],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    line = [l for l in r.stdout.splitlines() if l.startswith("tokens: ")][0]
+    assert json.loads(line[len("tokens: "):]) == prompt + want
+
+
+def test_config_and_random_weights_go_together():
+    from zinfer_amd.cli import CliError, Options, _llm, parse_flags
+    opt = Options(4)
+    parse_flags(["--config", "x.json"], opt)
+    with pytest.raises(CliError, match="go together"):
+        _llm("nowhere", opt)

@@ -47,6 +47,7 @@ Flags:
   --dtype <bfloat16|float32>   --page-size <n>            --max-tokens <n>
   --max-step-tokens <n>        --chunk <n>                --max-seqs <n>
   --ignore-eos                 --device <cuda:0>          --multi-step <n>
+  --config <config.json> --random-weights <seed>   (weights drawn from the seed; no folder read)
 """
 
 
@@ -97,6 +98,8 @@ class Options:
         self.ignore_eos = False
         self.device = "cuda:0"
         self.seed = 0
+        self.config_path: Optional[str] = None          # with --random-weights: no model folder
+        self.random_weights: Optional[int] = None
 
 
 _FLOAT_FLAGS = {"--temperature": "temperature", "--top-p": "top_p", "--min-p": "min_p",
@@ -148,9 +151,13 @@ def parse_flags(flags: List[str], opt: Options) -> None:
             opt.kv_cache = v
         elif a == "--threads":
             value()
-        elif a in ("--system", "--stop", "--q8-layout"):
-            raise CliError(f"UnknownFlag: {a} belongs to the text front end or the quantised "
-                           "cache, which this engine does not build")
+        elif a == "--q8-layout":
+            raise CliError("UnknownFlag: --q8-layout belongs to the quantised cache, which "
+                           "this engine does not build")
+        elif a == "--config":
+            opt.config_path = value()
+        elif a == "--random-weights":
+            opt.random_weights = int(value())
         elif a == "--dtype":
             opt.dtype = value()
         elif a == "--page-size":
@@ -220,7 +227,14 @@ def parse_generate(args: List[str], default_new: int) -> Tuple[str, List[int], O
 def _llm(model_dir: str, opt: Options, max_tokens: Optional[int] = None):
     from .entrypoints import LLM
     kv = None if opt.kv_cache == "auto" else ("bfloat16" if opt.kv_cache == "bf16" else "float32")
-    return LLM(model_dir, dtype=opt.dtype, device=opt.device, page_size=opt.page_size,
+    if (opt.config_path is None) != (opt.random_weights is None):
+        raise CliError("MissingFlagValue: --config <config.json> and --random-weights <seed> "
+                       "go together")
+    if opt.config_path is not None:
+        # weights drawn from the seed instead of read from a folder; the positional model
+        # folder, if one was given, is not opened
+        model_dir = None
+    return LLM(model_dir, config=opt.config_path, random_seed=opt.random_weights, dtype=opt.dtype, device=opt.device, page_size=opt.page_size,
                max_tokens=opt.max_tokens or max_tokens, max_step_tokens=opt.max_step_tokens,
                chunk_size=opt.chunk, max_seqs=opt.max_seqs, kv_dtype=kv,
                multi_step=opt.multi_step)

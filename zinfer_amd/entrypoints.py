@@ -13,21 +13,32 @@ import torch
 
 from .engine import Engine
 from .engine.scheduler import Request, Scheduler
-from .models.build import load_model
+from .models.build import load_model, random_model
 from .sampling import SamplingParams
 
 
 class LLM:
-    def __init__(self, model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0",
+    def __init__(self, model_dir: Optional[str] = None, dtype: str = "bfloat16",
+                 device: str = "cuda:0",
                  page_size: int = 16, max_tokens: Optional[int] = None,
                  num_pages: Optional[int] = None, max_step_tokens: int = 2048,
                  chunk_size: Optional[int] = None, max_seqs: int = 64,
-                 kv_dtype: Optional[str] = None, multi_step: int = 8):
-        """``max_tokens`` (or ``num_pages``) sizes the cache pool; by default the pool holds
+                 kv_dtype: Optional[str] = None, multi_step: int = 8,
+                 config=None, random_seed: Optional[int] = None):
+        """A model folder, or ``config`` (a typed configuration, a dict of config.json keys or
+        the path of a config.json) with ``random_seed``: weights drawn from the seed, the same
+        values that ``write_model_dir`` stores for it.  ``max_tokens`` (or ``num_pages``) sizes the cache pool; by default the pool holds
         ``max_seqs`` requests of ``max_position_embeddings`` tokens, capped at 1/2 of the free
         device memory.  ``multi_step``: the most decode steps that run in a row on the device
         without the host between them (1: the host sees every step)."""
-        self.config, self.model = load_model(model_dir, dtype, device)
+        if (config is None) != (random_seed is None):
+            raise ValueError("config and random_seed go together")
+        if config is not None:
+            self.config, self.model = random_model(config, random_seed, dtype, device)
+        elif model_dir is not None:
+            self.config, self.model = load_model(model_dir, dtype, device)
+        else:
+            raise ValueError("a model folder, or config and random_seed, is needed")
         spec = self.model.spec
         if num_pages is None:
             if max_tokens is None:
@@ -40,6 +51,11 @@ class LLM:
         self.scheduler_options = dict(max_step_tokens=max_step_tokens, chunk_size=chunk_size,
                                       max_seqs=max_seqs, eos_token_ids=spec.eos_token_ids,
                                       multi_step=multi_step)
+
+    @classmethod
+    def from_config(cls, config, seed: int = 0, **options) -> "LLM":
+        """An engine over random weights of ``config``, without a model folder."""
+        return cls(None, config=config, random_seed=seed, **options)
 
     def _default_max_tokens(self, spec, page_size: int, max_seqs: int) -> int:
         want = max_seqs * spec.max_positions

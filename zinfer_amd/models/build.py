@@ -49,3 +49,24 @@ def load_model(model_dir: str, dtype="bfloat16", device="cuda:0"):
     tensors = load_tensors(model_dir, model.declare())
     model.bind(tensors)
     return config, model
+
+
+def random_model(config, seed: int, dtype="bfloat16", device="cuda:0"):
+    """(typed configuration, bound model) with weights drawn from ``seed``: the values that
+    ``write_model_dir(config, seed, dtype)`` stores, without the file.  ``config``: a typed
+    configuration, a dict of config.json keys, or the path of a config.json."""
+    import json
+    from ..config import entry_for
+    from ..weights.random_init import draw_tensors
+    if isinstance(config, str):
+        with open(config, "r", encoding="utf-8") as f:
+            config = json.load(f)
+    if isinstance(config, dict):
+        config = entry_for(config).config_type.from_dict(config)
+    spec = config.model_spec()
+    ctx = BuildContext(parse_dtype(dtype), torch.device(device))
+    model = DecoderModel(spec, ctx)
+    tensors = draw_tensors(model.declare(), seed, ctx.compute_dtype,
+                           tied=spec.tie_word_embeddings, head_name=spec.head_name)
+    model.bind(tensors)
+    return config, model
