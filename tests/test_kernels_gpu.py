@@ -130,6 +130,38 @@ def test_gemm_pretiled_weights(M, N, K, o_dtype, accumulate):
     assert rel_err(got, plain_out) <= (tol(o_dtype) if not accumulate else 2e-5)
 
 
+@pytest.mark.parametrize("M", [17, 32, 33, 47, 64])
+@pytest.mark.parametrize("N,K", [(192, 4096), (4160, 1024), (16448, 512), (320, 384)])
+@pytest.mark.parametrize("kind", ["store", "store32", "accumulate", "swiglu"])
+def test_gemm_17_to_64_tokens(M, N, K, kind):
+    """The kernel for 17 to 64 tokens on pre-tiled weights (the tokens through LDS, 128
+    outputs per workgroup, split along K when the tiles are few): outputs that are no
+    multiple of its tile, one and several workgroups along K, each epilogue.  The tokens
+    differ in scale, so a row that lands in another token's place shows."""
+    ops = _ops()
+    plan = ops._mid_plan(M, N, K, True, kind == "swiglu")
+    if plan is None:
+        pytest.skip("the weight-streaming kernel serves this size")
+    a = _rand((M, K), torch.bfloat16, 70) * (1 + torch.arange(M)[:, None] % 5).to(torch.bfloat16)
+    w = _rand((N, K), torch.bfloat16, 71, 0.05)
+    if kind == "swiglu":
+        wi = ops.interleave_gate_up(w[:N // 2].to(DEV), w[N // 2:].to(DEV))
+        want = torch.empty((M, N // 2), dtype=torch.bfloat16)
+        ref.gemm_swiglu(a, wi.cpu(), want)
+        got = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.gemm_swiglu(a.to(DEV), ops.pretile_weight(wi), got, w_tiled=True)
+        assert rel_err(got, want) <= tol(torch.bfloat16)
+        return
+    acc = kind == "accumulate"
+    o_dtype = torch.bfloat16 if kind == "store" else torch.float32
+    base = _rand((M, N), torch.float32, 72).to(o_dtype)
+    want = base.clone()
+    ref.gemm(a, w, want, acc)
+    got = base.clone().to(DEV)
+    ops.gemm(a.to(DEV), ops.pretile_weight(w.to(DEV)), got, acc, w_tiled=True)
+    assert rel_err(got, want) <= (2e-5 if acc else tol(o_dtype))
+
+
 @pytest.mark.parametrize("kind", ["store", "accumulate", "swiglu"])
 def test_gemm_many_large_tiles(kind):
     """Enough 256 x 256 tiles to fill the chip more than once (the kernel that takes

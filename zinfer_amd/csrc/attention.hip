@@ -175,7 +175,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     int max_pages, int max_splits) {
   __shared__ __attribute__((aligned(16))) float s_o[4][16][HD];
   __shared__ float s_m[4][16], s_l[4][16];
-  const int s = blockIdx.x, kvh = blockIdx.y, sp = blockIdx.z;
+  const int kvh = blockIdx.x, sp = blockIdx.y, s = blockIdx.z;
   if (q_start[s + 1] - q_start[s] != 1) return;
   const int ctx = ctx_len[s], pos = ctx - 1;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
@@ -373,7 +373,7 @@ extern "C" int zf_attn_decode_bf16(const void* q, const void* k_pool, const void
   if (n_seqs <= 0) return 0;
   if (page_size % 16 != 0 || nKV <= 0 || nH % nKV != 0 || nH / nKV > 16) return -2;
   const float scale_log2e = scale * 1.4426950408889634f;
-  dim3 grid(n_seqs, nKV, max_splits);
+  dim3 grid(nKV, max_splits, n_seqs);
 #define ZF_DEC(HD)                                                                              \
   hipLaunchKernelGGL(attn_decode_kernel<HD>, grid, dim3(256), 0, stream, (const bf16_t*)q,      \
                      (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, q_start,        \

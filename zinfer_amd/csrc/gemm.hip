@@ -306,16 +306,17 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_ker
 // takes its W operands straight from the pre-tiled matrix (16-byte pieces that lie in runs of
 // 256 bytes), one k-tile ahead in registers.  That halves the LDS traffic per MFMA against
 // the kernel above, whose LDS is as busy as its MFMAs.
-template <int BM, int BN, int WM, int WN, int EPI>
+template <int BM, int BN, int WM, int WN, int EPI, int TKM = TK>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdirect_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
     int N, int K, int tiles_m, int tiles_n) {
   constexpr int NWN = BN / WN, NT = (BM / WM) * NWN * 64;
   constexpr int FM = WM / 32, FN = WN / 32;
-  static_assert(BM * 8 % NT == 0, "tile does not divide over the threads");
-  constexpr int A_CHUNKS = BM * 8 / NT;
+  constexpr int LROW = TKM + 8, KCH = TKM / 8;      // LDS row in elements; 16-byte chunks per row
+  static_assert(BM * KCH % NT == 0 && TKM % 64 == 0, "tile does not divide over the threads");
+  constexpr int A_CHUNKS = BM * KCH / NT;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  bf16_t* lds = (bf16_t*)lds_raw;       // two stages of BM rows of LDS_ROW elements
+  bf16_t* lds = (bf16_t*)lds_raw;       // two stages of BM rows of LROW elements
 
   const int nblocks = tiles_m * tiles_n;
   int b = blockIdx.x;
@@ -356,13 +357,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
     wbase[j] = W + (size_t)grp * (K / 64) * 1024 + ((lane / 32) * 64 + n % 16) * 8;
   }
   u32x4_t areg[A_CHUNKS];
-  u32x4_t wreg[TK / 16][FN];
+  u32x4_t wreg[TKM / 16][FN];
 
   auto gload_a = [&](int k0) {
 #pragma unroll
     for (int c = 0; c < A_CHUNKS; ++c) {
       const int chunk = tid + c * NT;
-      const int row = chunk / 8, kc = (chunk % 8) * 8;
+      const int row = chunk / KCH, kc = (chunk % KCH) * 8;
       const int m = min(m0 + row, M - 1);
       areg[c] = *(const u32x4_t*)(A + (size_t)m * K + k0 + kc);
     }
@@ -370,27 +371,28 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
   auto gload_w = [&](int kt, int ks) {
 #pragma unroll
     for (int j = 0; j < FN; ++j)
-      wreg[ks][j] = *(const u32x4_t*)(wbase[j] + (size_t)kt * 1024 + ks * 128);
+      wreg[ks][j] = *(const u32x4_t*)(wbase[j] + ((size_t)kt * (TKM / 64) + ks / 4) * 1024 +
+                                      (ks % 4) * 128);
   };
   auto lstore = [&](int stage) {
-    bf16_t* a_s = lds + stage * BM * LDS_ROW;
+    bf16_t* a_s = lds + stage * BM * LROW;
 #pragma unroll
     for (int c = 0; c < A_CHUNKS; ++c) {
       const int chunk = tid + c * NT;
-      const int row = chunk / 8, kc = (chunk % 8) * 8;
-      *(u32x4_t*)(a_s + row * LDS_ROW + kc) = areg[c];
+      const int row = chunk / KCH, kc = (chunk % KCH) * 8;
+      *(u32x4_t*)(a_s + row * LROW + kc) = areg[c];
     }
   };
 
   // gridDim.y workgroups share a tile's k-tiles (split-K for products with few tiles); each
   // then leaves a float32 partial [gridDim.y, M, N] in Cv for skinny_reduce_kernel
-  const int kt_all = K / TK;
+  const int kt_all = K / TKM;
   const int kt0 = (int)((long long)blockIdx.y * kt_all / gridDim.y);
   const int ktiles = (int)((long long)(blockIdx.y + 1) * kt_all / gridDim.y);
   if (gridDim.y > 1) Cv = (float*)Cv + (size_t)blockIdx.y * M * N;
-  gload_a(kt0 * TK);
+  gload_a(kt0 * TKM);
 #pragma unroll
-  for (int ks = 0; ks < TK / 16; ++ks) gload_w(kt0, ks);
+  for (int ks = 0; ks < TKM / 16; ++ks) gload_w(kt0, ks);
   lstore(0);
   __syncthreads();
   // One k-tile per trip: MFMAs on LDS stage `kt & 1`; meanwhile the tokens of tile kt + 1
@@ -402,21 +404,21 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
   for (int kt = kt0; kt < ktiles; ++kt) {
     const int stage = (kt - kt0) & 1;
     const int nxt = min(kt + 1, ktiles - 1);
-    gload_a(nxt * TK);
+    gload_a(nxt * TKM);
     __builtin_amdgcn_sched_barrier(0);
-    const bf16_t* a_s = lds + stage * BM * LDS_ROW + (wm * WM) * LDS_ROW;
+    const bf16_t* a_s = lds + stage * BM * LROW + (wm * WM) * LROW;
     // the token operands of k-step ks + 1 are read from LDS while the MFMAs of ks run
     bf16x8_t af[2][FM];
 #pragma unroll
     for (int i = 0; i < FM; ++i)
-      af[0][i] = *(const bf16x8_t*)(a_s + (i * 32 + lane % 32) * LDS_ROW + (lane / 32) * 8);
+      af[0][i] = *(const bf16x8_t*)(a_s + (i * 32 + lane % 32) * LROW + (lane / 32) * 8);
 #pragma unroll
-    for (int ks = 0; ks < TK / 16; ++ks) {
-      if (ks + 1 < TK / 16) {
+    for (int ks = 0; ks < TKM / 16; ++ks) {
+      if (ks + 1 < TKM / 16) {
         const int koff = (ks + 1) * 16 + (lane / 32) * 8;
 #pragma unroll
         for (int i = 0; i < FM; ++i)
-          af[(ks + 1) % 2][i] = *(const bf16x8_t*)(a_s + (i * 32 + lane % 32) * LDS_ROW + koff);
+          af[(ks + 1) % 2][i] = *(const bf16x8_t*)(a_s + (i * 32 + lane % 32) * LROW + koff);
       }
 #pragma unroll
       for (int i = 0; i < FM; ++i)
@@ -435,9 +437,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
   // so direct stores would be 2 or 4 bytes wide in runs of 64 bytes.  Each wave lays 32 rows
   // of its tile down in its own slab (rows padded by 4 floats) and reads them back along the
   // rows, 16 bytes per lane.  (The main loop's last barrier has freed the token stages.)
-  constexpr int SLAB_ROW = WN + 4;
-  static_assert((size_t)(BM / WM) * NWN * 32 * SLAB_ROW * 4 <= (size_t)2 * BM * LDS_ROW * 2,
-                "slabs do not fit into the token stages");
+  constexpr int SLAB_ROW = WN + 4;     // the launch sizes the LDS for stages and slabs
   float* slab = (float*)lds_raw + (size_t)wave * 32 * SLAB_ROW;
   const int mw = m0 + wm * WM, nw = n0 + wn * WN;
 #pragma unroll
@@ -509,19 +509,21 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
 static int launch_reduce(const void* ws, void* C, int M, int N, int ksplit, int epi,
                          hipStream_t stream);
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int TKM = TK>
 static int launch_tile_wdirect(const void* A, const void* W, void* C, int M, int N, int K, int epi,
                                hipStream_t stream, void* ws = nullptr, int ksplit = 1) {
-  if (N % 16 != 0 || K % 64 != 0) return -3;
-  if (ksplit > 1 && (ws == nullptr || epi == EPI_SWIGLU || ksplit > K / 64)) return -3;
+  if (N % 16 != 0 || K % TKM != 0) return -3;
+  if (ksplit > 1 && (ws == nullptr || epi == EPI_SWIGLU || ksplit > K / TKM)) return -3;
   constexpr int NT = (BM / WM) * (BN / WN) * 64;
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const dim3 grid(tiles_m * tiles_n, ksplit), block(NT);
   const int final_epi = epi;
-  const size_t smem = (size_t)2 * BM * LDS_ROW * sizeof(bf16_t);
+  constexpr size_t stages = (size_t)2 * BM * (TKM + 8) * sizeof(bf16_t);
+  constexpr size_t slabs = (size_t)(BM / WM) * (BN / WN) * 32 * (WN + 4) * sizeof(float);
+  const size_t smem = stages > slabs ? stages : slabs;
 #define ZF_WD(E)                                                                              \
   do {                                                                                        \
-    auto kern = gemm_bf16_tile_wdirect_kernel<BM, BN, WM, WN, E>;                             \
+    auto kern = gemm_bf16_tile_wdirect_kernel<BM, BN, WM, WN, E, TKM>;                             \
     if (smem > 64 * 1024) {                                                                   \
       hipError_t e = hipFuncSetAttribute((const void*)kern,                                   \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
@@ -598,6 +600,21 @@ extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, i
     case 4: return launch_tile<256, 256, 128, 64, false>(A, W, C, M, N, K, epi, stream);
     default: return -4;
   }
+}
+
+// 17 to 64 tokens on pre-tiled W.  The weight-streaming kernel below re-reads the tokens for
+// every 16 * RG rows of W, which at 64 tokens is as much traffic as W itself; here a workgroup
+// takes 128 rows of W, the tokens of a k-tile go through LDS once for its 4 waves, and the
+// k-tiles are 128 or 256 wide so that 32 or 64 KB of W are in flight per workgroup.  ksplit
+// workgroups share a tile's K (ws: float32 [ksplit, M, N]) when the tiles do not fill the chip.
+//   M <= 32: tiles of 32 tokens, K % 256 == 0;  M <= 64: tiles of 64 tokens, K % 128 == 0.
+extern "C" int zf_gemm_bf16_mid(const void* A, const void* W, void* C, void* ws, int M, int N,
+                                int K, int epi, int ksplit, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || ksplit < 1 || (epi == EPI_SWIGLU && N % 32 != 0)) return -3;
+  if (M <= 32)
+    return launch_tile_wdirect<32, 128, 32, 32, 256>(A, W, C, M, N, K, epi, stream, ws, ksplit);
+  return launch_tile_wdirect<64, 128, 64, 32, 128>(A, W, C, M, N, K, epi, stream, ws, ksplit);
 }
 
 enum { NORM_NONE = 0, NORM_FOLD = 1, NORM_GIVEN = 2 };

@@ -224,6 +224,22 @@ def _skinny_plan(M: int, N: int, K: int, tiled: bool):
     return rg, ks
 
 
+def _mid_plan(M: int, N: int, K: int, w_tiled: bool, swiglu: bool = False):
+    """Workgroups along K if the kernel for 17 to 64 tokens (128 outputs per workgroup, the
+    tokens through LDS) covers the product, else None: above 32 tokens, and from 17 on a wide
+    output, it beats the weight-streaming kernel, which re-reads the tokens for every few
+    rows of the weight.  Split along K until about 192 workgroups run, each keeping 1024 of K.
+    Measured on MI355X at the Qwen3-8B sizes."""
+    if not (w_tiled and 16 < M <= 64 and N % 16 == 0 and K % (256 if M <= 32 else 128) == 0):
+        return None
+    if M <= 32 and N < 16384:
+        return None
+    if swiglu:
+        return 1
+    tiles = (N + 127) // 128
+    return max(1, min(192 // tiles, K // 1024))
+
+
 def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = False) -> int:
     """Which tiled kernel: with pre-tiled weights the kernels that take W straight from
     memory (5: 256 x 256 tiles when they fill the chip at least once and the epilogue is a
@@ -287,7 +303,12 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and K % 8 == 0 and M > 0:
         epi = _EPI_ACC_F32 if accumulate else \
             (_EPI_STORE_BF16 if out.dtype == torch.bfloat16 else _EPI_STORE_F32)
-        if M <= SKINNY_MAX_M:
+        mid = _mid_plan(M, N, K, w_tiled)
+        if mid is not None:
+            ws = _workspace("gemm_splitk", mid * M * N, torch.float32, a.device) if mid > 1 else None
+            _check(lib.zf_gemm_bf16_mid(_ptr(a), _ptr(w), _ptr(out), _ptr(ws), M, N, K, epi, mid,
+                                        _stream()), "gemm (17 to 64 tokens)")
+        elif M <= SKINNY_MAX_M:
             rg, ks = _skinny_plan(M, N, K, w_tiled)
             ws = _workspace("gemm_splitk", ks * M * N, torch.float32, a.device) if ks > 1 else None
             _check(lib.zf_gemm_bf16_skinny(_ptr(a), _ptr(w), _ptr(out), _ptr(ws), M, N, K, epi,
@@ -430,7 +451,10 @@ def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bo
     if M == 0:
         return
     lib = build.load("gemm")
-    if M <= SKINNY_MAX_M:
+    if _mid_plan(M, N, K, w_tiled, swiglu=True) is not None:
+        _check(lib.zf_gemm_bf16_mid(_ptr(a), _ptr(w), _ptr(out), _ptr(None), M, N, K, _EPI_SWIGLU,
+                                    1, _stream()), "gemm_swiglu (17 to 64 tokens)")
+    elif M <= SKINNY_MAX_M:
         rg = 4 if (M > 16 and N >= 16384) else 2
         _check(lib.zf_gemm_bf16_skinny(_ptr(a), _ptr(w), _ptr(out), _ptr(None), M, N, K,
                                        _EPI_SWIGLU, rg, 1, 1 if w_tiled else 0, _stream()),
