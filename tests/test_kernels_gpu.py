@@ -162,6 +162,37 @@ def test_gemm_17_to_64_tokens(M, N, K, kind):
     assert rel_err(got, want) <= (2e-5 if acc else tol(o_dtype))
 
 
+@pytest.mark.parametrize("M", [17, 33, 64, 65, 200])
+@pytest.mark.parametrize("N,K", [(192, 4096), (4160, 2048), (8192, 1024)])
+def test_gemm_sum_norm(M, N, K):
+    """The residual sum whose split-K partials are added, summed into the residual and normed
+    by one kernel, against sum and norm in 64-bit.  Tokens of different scale: another row's
+    1 / rms would show."""
+    ops = _ops()
+    a = _rand((M, K), torch.bfloat16, 80)
+    w = _rand((N, K), torch.bfloat16, 81, 0.05)
+    base = _rand((M, N), torch.float32, 82, 2.0) * (1 + torch.arange(M).float()[:, None] % 7)
+    gain = 1 + 0.1 * _rand((N,), torch.float32, 83)
+    eps = 1e-5
+    wt = ops.pretile_weight(w.to(DEV))
+    if ops.sum_norm_plan(M, N, K, wt, True) is None:
+        pytest.skip("this product is not split along K: the norm runs on its own")
+    x = base.double() + a.double() @ w.double().T
+    want = torch.empty((M, N), dtype=torch.float64)
+    ref.rmsnorm(x, gain, eps, want)
+    res = base.clone().to(DEV)
+    normed = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_sum_norm(a.to(DEV), wt, res, gain.to(DEV), eps, normed)
+    assert rel_err(res, x) <= tol(torch.float32)
+    assert rel_err(normed, want) <= tol(torch.bfloat16)
+    # and the same bits as the separate kernels
+    res2 = base.clone().to(DEV)
+    ops.gemm(a.to(DEV), wt, res2, True, w_tiled=True)
+    normed2 = torch.empty_like(normed)
+    ops.rmsnorm(res2, gain.to(DEV), eps, normed2)
+    assert torch.equal(res, res2) and torch.equal(normed, normed2)
+
+
 @pytest.mark.parametrize("kind", ["store", "accumulate", "swiglu"])
 def test_gemm_many_large_tiles(kind):
     """Enough 256 x 256 tiles to fill the chip more than once (the kernel that takes

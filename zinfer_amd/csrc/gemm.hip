@@ -109,6 +109,7 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
 
 #define EPI_STORE_BF16 0
 #define EPI_STORE_F32 1
@@ -511,7 +512,8 @@ static int launch_reduce(const void* ws, void* C, int M, int N, int ksplit, int 
 
 template <int BM, int BN, int WM, int WN, int TKM = TK>
 static int launch_tile_wdirect(const void* A, const void* W, void* C, int M, int N, int K, int epi,
-                               hipStream_t stream, void* ws = nullptr, int ksplit = 1) {
+                               hipStream_t stream, void* ws = nullptr, int ksplit = 1,
+                               bool reduce = true) {
   if (N % 16 != 0 || K % TKM != 0) return -3;
   if (ksplit > 1 && (ws == nullptr || epi == EPI_SWIGLU || ksplit > K / TKM)) return -3;
   constexpr int NT = (BM / WM) * (BN / WN) * 64;
@@ -542,7 +544,7 @@ static int launch_tile_wdirect(const void* A, const void* W, void* C, int M, int
   else if (epi == EPI_SWIGLU) ZF_WD(EPI_SWIGLU);
   else ZF_WD(EPI_ACC_F32);
 #undef ZF_WD
-  if (ksplit > 1) return launch_reduce(ws, final_c, M, N, ksplit, final_epi, stream);
+  if (ksplit > 1 && reduce) return launch_reduce(ws, final_c, M, N, ksplit, final_epi, stream);
   return (int)hipGetLastError();
 }
 
@@ -932,6 +934,74 @@ static int launch_reduce(const void* ws, void* C, int M, int N, int ksplit, int 
                        (const float*)ws, C, mn, ksplit);
   else
     return -3;
+  return (int)hipGetLastError();
+}
+
+// The split-K partials of a residual sum whose reader is an RMSNorm: one workgroup per token
+// adds the partials in split order into the 32-bit residual row (as skinny_reduce_kernel
+// does), keeps the row in registers, and writes the norm of the sum,
+// n = x * gain / sqrt(mean(x^2) + eps) (src/kernel/core/cpu.zig:38-48 of the reference), as
+// bfloat16: the reduce and the norm kernel in one, the row read once.  N % 4 == 0, N <= 8192.
+__global__ __launch_bounds__(256) void reduce_sum_norm_kernel(
+    const float* __restrict__ ws, float* __restrict__ C, const float* __restrict__ gain,
+    bf16_t* __restrict__ normed, int M, int N, int ksplit, float eps) {
+  __shared__ float red[16];
+  const int m = blockIdx.x, n4 = N / 4;
+  float4* row = (float4*)(C + (size_t)m * N);
+  float4 v[8];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = threadIdx.x + i * 256;
+    v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (c < n4) {
+      float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int k = 0; k < ksplit; ++k) {
+        const float4 p = ((const float4*)(ws + ((size_t)k * M + m) * N))[c];
+        s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
+      }
+      const float4 old = row[c];
+      v[i] = make_float4(old.x + s.x, old.y + s.y, old.z + s.z, old.w + s.w);
+      row[c] = v[i];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)N + eps);
+  bf16_t* o = normed + (size_t)m * N;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = threadIdx.x + i * 256;
+    if (c < n4) {
+      const float4 g = ((const float4*)gain)[c];
+      *(u32x2_t*)(o + 4 * c) = u32x2_t{pack_bf16x2(v[i].x * inv * g.x, v[i].y * inv * g.y),
+                                       pack_bf16x2(v[i].z * inv * g.z, v[i].w * inv * g.w)};
+    }
+  }
+}
+
+// C += A W^T in 32-bit with ksplit >= 2 workgroups along K, and normed = bfloat16 RMSNorm of
+// the sum's rows, from the kernel that adds the partials.  M <= 64: the kernel for 17 to 64
+// tokens; above: 128 x 128 tiles.  W pre-tiled; ws: float32 [ksplit, M, N].
+extern "C" int zf_gemm_bf16_splitk_sum_norm(const void* A, const void* W, void* C, void* ws,
+                                            const float* gain, float eps, void* normed, int M,
+                                            int N, int K, int ksplit, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (ksplit < 2 || ksplit > 64 || N % 16 != 0 || N > 8192 || ws == nullptr) return -3;
+  int rc;
+  if (M <= 32)
+    rc = launch_tile_wdirect<32, 128, 32, 32, 256>(A, W, C, M, N, K, EPI_ACC_F32, stream, ws,
+                                                   ksplit, false);
+  else if (M <= 64)
+    rc = launch_tile_wdirect<64, 128, 64, 32, 128>(A, W, C, M, N, K, EPI_ACC_F32, stream, ws,
+                                                   ksplit, false);
+  else
+    rc = launch_tile_wdirect<128, 128, 64, 64>(A, W, C, M, N, K, EPI_ACC_F32, stream, ws, ksplit,
+                                               false);
+  if (rc != 0) return rc;
+  hipLaunchKernelGGL(reduce_sum_norm_kernel, dim3(M), dim3(256), 0, stream, (const float*)ws,
+                     (float*)C, gain, (bf16_t*)normed, M, N, ksplit, eps);
   return (int)hipGetLastError();
 }
 

@@ -367,6 +367,39 @@ def norm_gemm(x: torch.Tensor, gain: torch.Tensor, eps: float, w: torch.Tensor,
                                         _ptr(out), M, N, K, epi, rg, _stream()), "norm_gemm")
 
 
+def sum_norm_plan(M: int, N: int, K: int, w: torch.Tensor, w_tiled: bool):
+    """Workgroups along K if ``gemm_sum_norm`` covers residual += a w^T: a product that is
+    split along K anyway (17 to 64 tokens, or a few hundred tokens on a narrow output), whose
+    partials one kernel can add, sum into the residual and norm; else None."""
+    if not (w_tiled and w.dtype == torch.bfloat16 and w.is_cuda and N % 16 == 0 and N <= 8192):
+        return None
+    ks = _mid_plan(M, N, K, True) if M <= SKINNY_MAX_M else _tile_ksplit(M, N, K)
+    return ks if ks is not None and ks >= 2 else None
+
+
+def gemm_sum_norm(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, gain: torch.Tensor,
+                  eps: float, normed: torch.Tensor) -> None:
+    """residual += a w^T in 32-bit (``w`` pre-tiled) and normed = bfloat16(rmsnorm(residual,
+    gain, eps)), the norm from the kernel that adds the product's partials."""
+    _need_gpu(a, w, residual, gain, normed)
+    M, K = a.shape
+    N = w.shape[0]
+    ks = sum_norm_plan(M, N, K, w, True)
+    if ks is None or a.dtype != torch.bfloat16 or w.shape[1] != K or not can_pretile(w) \
+            or residual.shape != (M, N) or residual.dtype != torch.float32 \
+            or gain.shape != (N,) or gain.dtype != torch.float32 \
+            or normed.shape != (M, N) or normed.dtype != torch.bfloat16 \
+            or not all(t.is_contiguous() for t in (a, residual, normed)):
+        raise KernelUnavailable(f"gemm_sum_norm: a {tuple(a.shape)} {a.dtype}, w "
+                                f"{tuple(w.shape)}, residual {tuple(residual.shape)} "
+                                f"{residual.dtype}")
+    ws = _workspace("gemm_splitk", ks * M * N, torch.float32, a.device)
+    lib = build.load("gemm")
+    _check(lib.zf_gemm_bf16_splitk_sum_norm(_ptr(a), _ptr(w), _ptr(residual), _ptr(ws), _ptr(gain),
+                                            ctypes.c_float(eps), _ptr(normed), M, N, K, ks,
+                                            _stream()), "gemm_sum_norm")
+
+
 def norm_emit_plan(M: int, N: int, K: int, w: torch.Tensor, w_tiled: bool):
     """Row groups per workgroup if ``gemm_emit`` covers out += a w^T (weight-streaming kernel,
     up to 16 tokens, pre-tiled bfloat16 weight, no split over workgroups), else None."""

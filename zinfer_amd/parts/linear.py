@@ -26,7 +26,7 @@ class Linear:
         kernel leaves that norm's inputs in ``step.norm_ready`` when it can."""
         if hasattr(x, "materialize"):
             M, K = x.shape
-            if not accumulate and \
+            if not x.done and not accumulate and \
                     ops.norm_gemm_plan(M, self.out_features, K, self.weight, self.tiled) is not None:
                 if x.given is not None:
                     ops.gemm_given(x.given.xg, x.given.sq, x.eps, self.weight, out)
@@ -43,6 +43,14 @@ class Linear:
             sq = step.scratch("normed_squares", (self.out_features // 16, 16), torch.float32)
             ops.gemm_emit(x, self.weight, out, norm.gain, xg, sq)
             step.norm_ready = GivenRmsNorm(norm, out, xg, sq)
+            return out
+        if norm is not None and hasattr(norm, "gain") and x.dtype == torch.bfloat16 and \
+                ops.sum_norm_plan(x.shape[0], self.out_features, self.in_features, self.weight,
+                                  self.tiled) is not None:
+            from .norm import DoneRmsNorm
+            normed = step.scratch("normed_by_sum", out.shape, torch.bfloat16)
+            ops.gemm_sum_norm(x, self.weight, out, norm.gain, float(norm.spec.eps), normed)
+            step.norm_ready = DoneRmsNorm(norm, out, normed)
             return out
         ops.gemm(x, self.weight, out, accumulate, w_tiled=self.tiled)
         return out

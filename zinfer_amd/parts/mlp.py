@@ -46,7 +46,7 @@ class SwiGluMlp(FeedForward):
         I = self.spec.intermediate_size
         act = self.ctx.act_dtype
         a = step.scratch("ff_act", (T, I), act)
-        if self.fused and hasattr(h, "materialize") and self.gate_up.tiled \
+        if self.fused and hasattr(h, "materialize") and not h.done and self.gate_up.tiled \
                 and T <= ops.NORM_FOLD_MAX_M:
             if h.given is not None:
                 ops.gemm_given(h.given.xg, h.given.sq, h.eps, self.gate_up.weight, a, swiglu=True)

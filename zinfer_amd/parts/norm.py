@@ -40,17 +40,35 @@ class GivenRmsNorm:
         return self.norm is norm and self.x.data_ptr() == x.data_ptr() and self.x.shape == x.shape
 
 
+class DoneRmsNorm:
+    """The norm of the residual rows ``x`` already run by the kernel that last added into them
+    (``ops.gemm_sum_norm``): ``normed`` holds the result."""
+
+    def __init__(self, norm: "RmsNorm", x: torch.Tensor, normed: torch.Tensor):
+        self.norm, self.x, self.normed = norm, x, normed
+
+    def fits(self, norm, x: torch.Tensor) -> bool:
+        return self.norm is norm and self.x.data_ptr() == x.data_ptr() and self.x.shape == x.shape
+
+
 class LazyRmsNorm:
     """A norm that has not run yet: the residual rows and the norm's parameters.  A consumer
     whose first matrix product can fold the norm in (``Linear.forward``) takes it apart;
     anyone else calls ``materialize()`` and gets the normed activations (computed once).
-    ``given``: what the producer of the rows already left of the norm, if anything."""
+    ``given``: what the producer of the rows already left of the norm, if anything: its
+    inputs (``GivenRmsNorm``) or its whole result (``DoneRmsNorm``)."""
 
     def __init__(self, norm: "RmsNorm", x: torch.Tensor, make_out, given: GivenRmsNorm = None):
         self.x, self.gain, self.eps = x, norm.gain, float(norm.spec.eps)
         self.shape = x.shape
-        self.given = given
         self._norm, self._make_out, self._out = norm, make_out, None
+        if isinstance(given, DoneRmsNorm):
+            given, self._out = None, given.normed
+        self.given = given
+
+    @property
+    def done(self) -> bool:
+        return self._out is not None
 
     def materialize(self) -> torch.Tensor:
         if self._out is None:
