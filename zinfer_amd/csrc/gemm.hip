@@ -303,10 +303,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_ker
 }
 
 // ---------------------------------------------------------------- large M, pre-tiled W: W not staged
-// 256 x 256 x 64 tiles, 4 waves of 128 x 128.  Only the tokens go through LDS; every wave
+// Tiles of BM tokens x BN outputs, k-tiles of TKM.  Only the tokens go through LDS; every wave
 // takes its W operands straight from the pre-tiled matrix (16-byte pieces that lie in runs of
 // 256 bytes), one k-tile ahead in registers.  That halves the LDS traffic per MFMA against
-// the kernel above, whose LDS is as busy as its MFMAs.
+// the kernel above, whose LDS is as busy as its MFMAs.  With the waves side by side along the
+// outputs (WM == BM) no two of them load the same part of W.
 template <int BM, int BN, int WM, int WN, int EPI, int TKM = TK>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdirect_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
@@ -574,31 +575,22 @@ static int launch_tile(const void* A, const void* W, void* C, int M, int N, int 
   return (int)hipGetLastError();
 }
 
-// variant: 0 = 128x128 (waves 64x64), 1 = 256x128 (waves 128x64), 2 = 256x256 (waves 128x128),
-//          3 = 128x128 (waves 64x32, 8 waves), 4 = 256x256 (waves 128x64, 8 waves);
-//          with pre-tiled W only: 5 = 256x256 (waves 128x128), 6 = 128x128 (waves 64x64),
-//          7 = 256x128 (waves 128x64), W straight from memory into the MFMA operands
-//          w_tiled: W is in the pre-tiled layout (needs N % 16 == 0 and K % 64 == 0)
+// variant, plain W: 0 = 128x128 (waves 64x64), 4 = 256x256 (waves 128x64, 8 waves);
+//          pre-tiled W (w_tiled; N % 16 == 0 and K % 64 == 0), taken straight from memory
+//          into the MFMA operands: 6 = 128x128 (waves 64x64), 10 = 128x256 (waves 128x64: no
+//          two waves load the same part of W, and two workgroups share a CU)
 extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, int N, int K,
                                  int epi, int variant, int w_tiled, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K % 8 != 0 || (epi == EPI_SWIGLU && N % 32 != 0)) return -3;
   if (w_tiled) {
     if (N % 16 != 0 || K % 64 != 0) return -3;
-    if (variant == 5) return launch_tile_wdirect<256, 256, 128, 128>(A, W, C, M, N, K, epi, stream);
     if (variant == 6) return launch_tile_wdirect<128, 128, 64, 64>(A, W, C, M, N, K, epi, stream);
-    if (variant == 7) return launch_tile_wdirect<256, 128, 128, 64>(A, W, C, M, N, K, epi, stream);
-    switch (variant) {
-      case 0: return launch_tile<128, 128, 64, 64, true>(A, W, C, M, N, K, epi, stream);
-      case 4: return launch_tile<256, 256, 128, 64, true>(A, W, C, M, N, K, epi, stream);
-      default: return -4;
-    }
+    if (variant == 10) return launch_tile_wdirect<128, 256, 128, 64>(A, W, C, M, N, K, epi, stream);
+    return -4;
   }
   switch (variant) {
     case 0: return launch_tile<128, 128, 64, 64, false>(A, W, C, M, N, K, epi, stream);
-    case 1: return launch_tile<256, 128, 128, 64, false>(A, W, C, M, N, K, epi, stream);
-    case 2: return launch_tile<256, 256, 128, 128, false>(A, W, C, M, N, K, epi, stream);
-    case 3: return launch_tile<128, 128, 64, 32, false>(A, W, C, M, N, K, epi, stream);
     case 4: return launch_tile<256, 256, 128, 64, false>(A, W, C, M, N, K, epi, stream);
     default: return -4;
   }

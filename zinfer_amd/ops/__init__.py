@@ -242,13 +242,12 @@ def _mid_plan(M: int, N: int, K: int, w_tiled: bool, swiglu: bool = False):
 
 def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = False) -> int:
     """Which tiled kernel: with pre-tiled weights the kernels that take W straight from
-    memory (5: 256 x 256 tiles when they fill the chip at least once and the epilogue is a
-    plain store, whose cost a single resident workgroup cannot hide behind others; else 6:
+    memory (10: 128 x 256 tiles, two workgroups to a CU, when they fill the chip; else 6:
     128 x 128); otherwise the kernels that stage both operands through LDS (4: 256 x 256 when
     they still fill the chip, else 0: 128 x 128).  Measured on MI355X at the Qwen3-8B sizes."""
-    tiles = ((M + 255) // 256) * ((N + 255) // 256)
     if w_tiled:
-        return 5 if (tiles >= 256 and not accumulate) else 6
+        return 10 if ((M + 127) // 128) * ((N + 255) // 256) >= 192 else 6
+    tiles = ((M + 255) // 256) * ((N + 255) // 256)
     return 4 if tiles >= 160 else 0
 
 
