@@ -194,12 +194,13 @@ def test_gemm_sum_norm(M, N, K):
 
 
 @pytest.mark.parametrize("kind", ["store", "accumulate", "swiglu"])
-def test_gemm_many_large_tiles(kind):
-    """Enough 256 x 256 tiles to fill the chip more than once (the kernel that takes
+@pytest.mark.parametrize("K", [192, 256, 64])
+def test_gemm_many_large_tiles(kind, K):
+    """Enough 128 x 256 tiles to fill the chip more than once (the kernel that takes
     pre-tiled W straight into its operands), with edges in M and N that are no multiple of
-    the tile and several k-tiles."""
+    the tile; an odd and an even number of k-tiles (W one or two k-tiles ahead) and one."""
     ops = _ops()
-    M, N, K = 4100, 4160, 192
+    M, N = 4100, 4160
     a = _rand((M, K), torch.bfloat16, 35)
     w = _rand((N, K), torch.bfloat16, 36, 0.05)
     if kind == "swiglu":

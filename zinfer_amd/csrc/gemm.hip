@@ -4,6 +4,8 @@
 //  * gemm_fma: 32-bit FMA, any storage types, any sizes.  Every output element is the sum of
 //    its products in ascending k, whatever M is and wherever the row lies in the batch, so a
 //    token's result does not depend on how the batch was cut.  This is the true 32-bit path.
+#include <type_traits>
+
 #include "zf_common.h"
 
 #define GF_BM 64
@@ -308,7 +310,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_ker
 // 256 bytes), one k-tile ahead in registers.  That halves the LDS traffic per MFMA against
 // the kernel above, whose LDS is as busy as its MFMAs.  With the waves side by side along the
 // outputs (WM == BM) no two of them load the same part of W.
-template <int BM, int BN, int WM, int WN, int EPI, int TKM = TK>
+template <int BM, int BN, int WM, int WN, int EPI, int TKM = TK, bool W2 = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdirect_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
     int N, int K, int tiles_m, int tiles_n) {
@@ -359,7 +361,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
     wbase[j] = W + (size_t)grp * (K / 64) * 1024 + ((lane / 32) * 64 + n % 16) * 8;
   }
   u32x4_t areg[A_CHUNKS];
-  u32x4_t wreg[TKM / 16][FN];
+  u32x4_t wreg[W2 ? 2 : 1][TKM / 16][FN];
 
   auto gload_a = [&](int k0) {
 #pragma unroll
@@ -370,10 +372,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
       areg[c] = *(const u32x4_t*)(A + (size_t)m * K + k0 + kc);
     }
   };
-  auto gload_w = [&](int kt, int ks) {
+  auto gload_w = [&](auto BUF, int kt, int ks) {
+    constexpr int B = decltype(BUF)::value;
 #pragma unroll
     for (int j = 0; j < FN; ++j)
-      wreg[ks][j] = *(const u32x4_t*)(wbase[j] + ((size_t)kt * (TKM / 64) + ks / 4) * 1024 +
+      wreg[B][ks][j] = *(const u32x4_t*)(wbase[j] + ((size_t)kt * (TKM / 64) + ks / 4) * 1024 +
                                       (ks % 4) * 128);
   };
   auto lstore = [&](int stage) {
@@ -392,20 +395,29 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
   const int kt0 = (int)((long long)blockIdx.y * kt_all / gridDim.y);
   const int ktiles = (int)((long long)(blockIdx.y + 1) * kt_all / gridDim.y);
   if (gridDim.y > 1) Cv = (float*)Cv + (size_t)blockIdx.y * M * N;
+  using Buf0 = std::integral_constant<int, 0>;
+  using Buf1 = std::integral_constant<int, 1>;
   gload_a(kt0 * TKM);
 #pragma unroll
-  for (int ks = 0; ks < TKM / 16; ++ks) gload_w(kt0, ks);
+  for (int ks = 0; ks < TKM / 16; ++ks) gload_w(Buf0{}, kt0, ks);
+  if (W2) {
+#pragma unroll
+    for (int ks = 0; ks < TKM / 16; ++ks) gload_w(Buf1{}, min(kt0 + 1, ktiles - 1), ks);
+  }
   lstore(0);
   __syncthreads();
-  // One k-tile per trip: MFMAs on LDS stage `kt & 1`; meanwhile the tokens of tile kt + 1
+  // One k-tile per step: MFMAs on LDS stage `stage`; meanwhile the tokens of tile kt + 1
   // travel through registers into the other stage, and every k-step's W registers are
-  // refilled with their part of tile kt + 1 right after their last use.  No branches around
-  // the loads (the last trip loads its own tile once more), so the compiler can count the
-  // loads in flight and waits for no younger one; the scheduling barriers keep it from
-  // sinking the loads down to their first use, which would expose their whole latency.
-  for (int kt = kt0; kt < ktiles; ++kt) {
-    const int stage = (kt - kt0) & 1;
+  // refilled right after their last use with their part of tile kt + 1 (W2: of tile kt + 2,
+  // from the other of two register sets, so that a miss in L2 has two k-tiles to arrive).
+  // No branches around the loads (the last steps load their own tile once more), so the
+  // compiler can count the loads in flight and waits for no younger one; the scheduling
+  // barriers keep it from sinking the loads down to their first use, which would expose
+  // their whole latency.
+  auto step = [&](int kt, int stage, auto BUF) {
+    constexpr int B = decltype(BUF)::value;
     const int nxt = min(kt + 1, ktiles - 1);
+    const int wnxt = W2 ? min(kt + 2, ktiles - 1) : nxt;
     gload_a(nxt * TKM);
     __builtin_amdgcn_sched_barrier(0);
     const bf16_t* a_s = lds + stage * BM * LROW + (wm * WM) * LROW;
@@ -427,12 +439,20 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
 #pragma unroll
         for (int j = 0; j < FN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              af[ks % 2][i], *(const bf16x8_t*)&wreg[ks][j], acc[i][j], 0, 0, 0);
-      gload_w(nxt, ks);
+              af[ks % 2][i], *(const bf16x8_t*)&wreg[B][ks][j], acc[i][j], 0, 0, 0);
+      gload_w(BUF, wnxt, ks);
       __builtin_amdgcn_sched_barrier(0);
     }
     lstore(stage ^ 1);
     __syncthreads();
+  };
+  if (W2) {       // an even number of k-tiles (the launch sees to it)
+    for (int kt = kt0; kt < ktiles; kt += 2) {
+      step(kt, 0, Buf0{});
+      step(kt + 1, 1, Buf1{});
+    }
+  } else {
+    for (int kt = kt0; kt < ktiles; ++kt) step(kt, (kt - kt0) & 1, Buf0{});
   }
 
   // Epilogue through LDS: a 32x32 MFMA result has a lane's 16 values in 16 different rows,
@@ -511,11 +531,12 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
 static int launch_reduce(const void* ws, void* C, int M, int N, int ksplit, int epi,
                          hipStream_t stream);
 
-template <int BM, int BN, int WM, int WN, int TKM = TK>
+template <int BM, int BN, int WM, int WN, int TKM = TK, bool W2 = false>
 static int launch_tile_wdirect(const void* A, const void* W, void* C, int M, int N, int K, int epi,
                                hipStream_t stream, void* ws = nullptr, int ksplit = 1,
                                bool reduce = true) {
   if (N % 16 != 0 || K % TKM != 0) return -3;
+  if (W2 && (ksplit != 1 || (K / TKM) % 2 != 0)) return -3;
   if (ksplit > 1 && (ws == nullptr || epi == EPI_SWIGLU || ksplit > K / TKM)) return -3;
   constexpr int NT = (BM / WM) * (BN / WN) * 64;
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
@@ -526,7 +547,7 @@ static int launch_tile_wdirect(const void* A, const void* W, void* C, int M, int
   const size_t smem = stages > slabs ? stages : slabs;
 #define ZF_WD(E)                                                                              \
   do {                                                                                        \
-    auto kern = gemm_bf16_tile_wdirect_kernel<BM, BN, WM, WN, E, TKM>;                             \
+    auto kern = gemm_bf16_tile_wdirect_kernel<BM, BN, WM, WN, E, TKM, W2>;                             \
     if (smem > 64 * 1024) {                                                                   \
       hipError_t e = hipFuncSetAttribute((const void*)kern,                                   \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
@@ -578,7 +599,8 @@ static int launch_tile(const void* A, const void* W, void* C, int M, int N, int 
 // variant, plain W: 0 = 128x128 (waves 64x64), 4 = 256x256 (waves 128x64, 8 waves);
 //          pre-tiled W (w_tiled; N % 16 == 0 and K % 64 == 0), taken straight from memory
 //          into the MFMA operands: 6 = 128x128 (waves 64x64), 10 = 128x256 (waves 128x64: no
-//          two waves load the same part of W, and two workgroups share a CU)
+//          two waves load the same part of W, two workgroups share a CU, and W is loaded
+//          two k-tiles ahead when their number is even)
 extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, int N, int K,
                                  int epi, int variant, int w_tiled, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
@@ -586,7 +608,11 @@ extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, i
   if (w_tiled) {
     if (N % 16 != 0 || K % 64 != 0) return -3;
     if (variant == 6) return launch_tile_wdirect<128, 128, 64, 64>(A, W, C, M, N, K, epi, stream);
-    if (variant == 10) return launch_tile_wdirect<128, 256, 128, 64>(A, W, C, M, N, K, epi, stream);
+    if (variant == 10) {
+      if (K % (2 * TK) == 0)     // W two k-tiles ahead: an even number of k-tiles
+        return launch_tile_wdirect<128, 256, 128, 64, TK, true>(A, W, C, M, N, K, epi, stream);
+      return launch_tile_wdirect<128, 256, 128, 64>(A, W, C, M, N, K, epi, stream);
+    }
     return -4;
   }
   switch (variant) {
