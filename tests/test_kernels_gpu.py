@@ -185,12 +185,11 @@ def test_gemm_sum_norm(M, N, K):
     ops.gemm_sum_norm(a.to(DEV), wt, res, gain.to(DEV), eps, normed)
     assert rel_err(res, x) <= tol(torch.float32)
     assert rel_err(normed, want) <= tol(torch.bfloat16)
-    # and the same bits as the separate kernels
+    # the residual has the same bits as from the separate kernels (partials added in the same
+    # order); the norm's sum of squares is added over another number of threads
     res2 = base.clone().to(DEV)
     ops.gemm(a.to(DEV), wt, res2, True, w_tiled=True)
-    normed2 = torch.empty_like(normed)
-    ops.rmsnorm(res2, gain.to(DEV), eps, normed2)
-    assert torch.equal(res, res2) and torch.equal(normed, normed2)
+    assert torch.equal(res, res2)
 
 
 @pytest.mark.parametrize("kind", ["store", "accumulate", "swiglu"])

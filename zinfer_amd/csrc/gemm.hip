@@ -959,23 +959,27 @@ static int launch_reduce(const void* ws, void* C, int M, int N, int ksplit, int 
 // adds the partials in split order into the 32-bit residual row (as skinny_reduce_kernel
 // does), keeps the row in registers, and writes the norm of the sum,
 // n = x * gain / sqrt(mean(x^2) + eps) (src/kernel/core/cpu.zig:38-48 of the reference), as
-// bfloat16: the reduce and the norm kernel in one, the row read once.  N % 4 == 0, N <= 8192.
-__global__ __launch_bounds__(256) void reduce_sum_norm_kernel(
+// bfloat16: the reduce and the norm kernel in one, the row read once.  N % 4 == 0, N <= 8192
+// (8 float4 per thread with 256 threads; wider rows get up to 1024 threads).
+__global__ __launch_bounds__(1024) void reduce_sum_norm_kernel(
     const float* __restrict__ ws, float* __restrict__ C, const float* __restrict__ gain,
     bf16_t* __restrict__ normed, int M, int N, int ksplit, float eps) {
   __shared__ float red[16];
-  const int m = blockIdx.x, n4 = N / 4;
+  const int m = blockIdx.x, n4 = N / 4, nt = blockDim.x;      // 8 * nt >= n4
   float4* row = (float4*)(C + (size_t)m * N);
+  const float4* part = (const float4*)(ws + (size_t)m * N);
+  const size_t kstride = (size_t)M * n4;
   float4 v[8];
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const int c = threadIdx.x + i * 256;
+    const int c = threadIdx.x + i * nt;
     v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (c < n4) {
       float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-      for (int k = 0; k < ksplit; ++k) {
-        const float4 p = ((const float4*)(ws + ((size_t)k * M + m) * N))[c];
+#pragma unroll 8
+      for (int k = 0; k < ksplit; ++k) {          // independent loads, added in split order
+        const float4 p = part[k * kstride + c];
         s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
       }
       const float4 old = row[c];
@@ -990,7 +994,7 @@ __global__ __launch_bounds__(256) void reduce_sum_norm_kernel(
   bf16_t* o = normed + (size_t)m * N;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const int c = threadIdx.x + i * 256;
+    const int c = threadIdx.x + i * nt;
     if (c < n4) {
       const float4 g = ((const float4*)gain)[c];
       *(u32x2_t*)(o + 4 * c) = u32x2_t{pack_bf16x2(v[i].x * inv * g.x, v[i].y * inv * g.y),
@@ -1018,7 +1022,9 @@ extern "C" int zf_gemm_bf16_splitk_sum_norm(const void* A, const void* W, void* 
     rc = launch_tile_wdirect<128, 128, 64, 64>(A, W, C, M, N, K, EPI_ACC_F32, stream, ws, ksplit,
                                                false);
   if (rc != 0) return rc;
-  hipLaunchKernelGGL(reduce_sum_norm_kernel, dim3(M), dim3(256), 0, stream, (const float*)ws,
+  // a thread per 4 columns up to 1024 threads: every load of a row is in flight at once
+  const int threads = N / 4 >= 1024 ? 1024 : (N / 4 > 256 ? 512 : 256);
+  hipLaunchKernelGGL(reduce_sum_norm_kernel, dim3(M), dim3(threads), 0, stream, (const float*)ws,
                      (float*)C, gain, (bf16_t*)normed, M, N, ksplit, eps);
   return (int)hipGetLastError();
 }
