@@ -21,7 +21,7 @@ LOGITS_TOL_F32 = 2e-5
 LOGITS_TOL_BF16 = 2e-2
 
 LENGTHS = {"A": (5, 17, 40, 70), "B": (1, 9, 33, 64, 130), "C": (3, 48, 65, 100),
-           "D": (2, 31, 97, 300, 520)}
+           "D": (2, 31, 97, 300, 520), "E": (40, 64, 150, 333)}
 _plain_cache = {}
 
 
@@ -83,7 +83,7 @@ MODES = {"whole": traces.whole, "prefill_then_32": traces.prefill_then_single,
 
 @pytest.mark.parametrize("mode", list(MODES))
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_replay_modes(name, dtype, mode, tmp_path_factory):
     path, cfg, requests, ref = _setup(name, dtype, tmp_path_factory)
     steps = MODES[mode](requests)

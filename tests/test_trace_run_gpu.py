@@ -39,13 +39,14 @@ def run_trace(model_dir, dtype, steps, out_dir, max_tokens):
 
 
 @pytest.mark.parametrize("name,dtype", [("A", "float32"), ("D", "bfloat16"), ("B", "bfloat16"),
-                                        ("D", "float32")])
+                                        ("D", "float32"), ("E", "bfloat16")])
 def test_every_cutting_through_trace_run(name, dtype, tmp_path):
     store = torch.float32 if dtype == "float32" else torch.bfloat16
     model_dir = tiny.model_dir_of(name, str(tmp_path), store)
     cfg = tiny.CONFIGS[name]
     V = cfg["vocab_size"]
-    lens = {"A": (40, 70, 5, 100), "B": (33, 130, 64, 9, 80), "D": (97, 300, 31, 150, 64)}[name]
+    lens = {"A": (40, 70, 5, 100), "B": (33, 130, 64, 9, 80), "D": (97, 300, 31, 150, 64),
+            "E": (40, 150, 64, 333, 20)}[name]
     requests = {f"t{i}": tiny.random_tokens(n, V, 900 + i) for i, n in enumerate(lens)}
     w = tiny.weights_of(name, store)
     ref = {rid: plain.model_forward_batched(cfg, w, t).numpy() for rid, t in requests.items()}

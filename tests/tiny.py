@@ -36,9 +36,18 @@ TINY_D = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden
               intermediate_size=456, vocab_size=1210, rope_theta=100000.0, rms_norm_eps=2e-6,
               tie_word_embeddings=True, max_position_embeddings=640, torch_dtype="bfloat16")
 
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
-PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16}
-SEEDS = {"A": 11, "B": 22, "C": 33, "D": 44}
+# a fifth shape with the serving model's head size and widths that are multiples of 128 (and a
+# feed-forward width of 2048), so that the kernels chosen by size run inside the engine tests:
+# the product for 17 to 64 tokens, the products split along K whose partials one kernel adds,
+# sums into the residual and norms, the 128 x 256 tiles, the head-size-128 attention
+TINY_E = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2,
+              hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=128,
+              intermediate_size=2048, vocab_size=2304, rope_theta=500000.0, rms_norm_eps=1e-6,
+              tie_word_embeddings=False, max_position_embeddings=768, torch_dtype="bfloat16")
+
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
+PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 16}
+SEEDS = {"A": 11, "B": 22, "C": 33, "D": 44, "E": 55}
 
 
 def config_of(name: str) -> Qwen3Config:
