@@ -21,7 +21,7 @@ LOGITS_TOL_F32 = 2e-5
 LOGITS_TOL_BF16 = 2e-2
 
 LENGTHS = {"A": (5, 17, 40, 70), "B": (1, 9, 33, 64, 130), "C": (3, 48, 65, 100),
-           "D": (2, 31, 97, 300, 520), "E": (40, 64, 150, 333)}
+           "D": (2, 31, 97, 300, 520), "E": (40, 64, 150, 333), "W": (8, 24, 50, 64, 300)}
 _plain_cache = {}
 
 
@@ -91,6 +91,19 @@ def test_replay_modes(name, dtype, mode, tmp_path_factory):
     tolerance = LOGITS_TOL_F32 if dtype == "float32" else LOGITS_TOL_BF16
     worst = _compare(steps, outputs, ref, cfg["vocab_size"], tolerance)
     print(f"{name} {dtype} {mode}: worst error {worst:.3g}")
+
+
+@pytest.mark.parametrize("mode", ["whole", "mixed", "prefill_then_32"])
+def test_serving_widths(mode, tmp_path_factory):
+    """Two layers of the served model's widths in bfloat16: whole prompts of 8 to 300 tokens
+    (one kernel choice each: weight streaming, 17 to 64 tokens, tiled, with their splits along
+    K), mixed batches, and decoding, against the plain implementation."""
+    name = "W"
+    path, cfg, requests, ref = _setup(name, "bfloat16", tmp_path_factory)
+    steps = MODES[mode](requests)
+    outputs, eng = _replay(path, "bfloat16", steps, tiny.PAGE_SIZE[name])
+    worst = _compare(steps, outputs, ref, cfg["vocab_size"], LOGITS_TOL_BF16)
+    print(f"{name} bfloat16 {mode}: worst error {worst:.3g}")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -45,9 +45,17 @@ TINY_E = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden
               intermediate_size=2048, vocab_size=2304, rope_theta=500000.0, rms_norm_eps=1e-6,
               tie_word_embeddings=False, max_position_embeddings=768, torch_dtype="bfloat16")
 
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
-PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 16}
-SEEDS = {"A": 11, "B": 22, "C": 33, "D": 44, "E": 55}
+# two layers of the widths that are served (hidden 4096, 32 / 8 heads of 128, feed-forward
+# 12288) under a small vocabulary that is no multiple of 64: the kernels at the sizes and
+# with the splits along K that the benchmark runs them with, against the plain implementation
+WIDE = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2,
+            hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+            intermediate_size=12288, vocab_size=8200, rope_theta=1000000.0, rms_norm_eps=1e-6,
+            tie_word_embeddings=False, max_position_embeddings=1024, torch_dtype="bfloat16")
+
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "W": WIDE}
+PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 16, "W": 16}
+SEEDS = {"A": 11, "B": 22, "C": 33, "D": 44, "E": 55, "W": 66}
 
 
 def config_of(name: str) -> Qwen3Config:
