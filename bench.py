@@ -234,7 +234,7 @@ def main() -> int:
     peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
     flops = prefill_flops(cfg, args.prefill_tokens)
     line = {
-        "metric": "decode tok/s, Qwen3-8B shape, batch %d, 2048-token prompts" % args.batch,
+        "metric": "decode tok/s, Qwen3-8B shape, batch %d, %d-token prompts" % (args.batch, args.prompt_len),
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(dt / args.steps * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
