@@ -128,6 +128,11 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
 
+// 2^x for x <= 0 as the bare v_exp_f32 (1 ulp; -inf gives 0, results below 2^-126 may come
+// out as 0): exp2f() wraps the same instruction in five more that rescale such tiny results,
+// which a soft-max term does not need.
+__device__ __forceinline__ float exp2_raw(float x) { return __builtin_amdgcn_exp2f(x); }
+
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   return pack_bf16x2(lo, hi);
 }
@@ -255,7 +260,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     m = fmaxf(m, __shfl_xor(m, 32, 64));
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      sc[e] = exp2f(sc[e] - m);
+      sc[e] = exp2_raw(sc[e] - m);
       l += sc[e];
     }
     l += __shfl_xor(l, 16, 64);
@@ -503,32 +508,30 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
         st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&kf[stp], qf[stp], st, 0, 0, 0);
       if (kb + kstep <= p_max) load_keys(kb + kstep, kf);   // next tile's keys, in flight from here
       // st[r]: key kb + 8 (r / 4) + 4 hf + r % 4, query column j
+      // the scale (> 0) goes into the exponent's multiply-add: max over the raw scores
       float tmax = -INFINITY;
       if (kb + 31 <= pos0 && kb >= lo_top) {
         // every key of the tile is visible to every query of the wave: nothing to mask
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          st[r] *= scale_log2e;
-          tmax = fmaxf(tmax, st[r]);
-        }
+        for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, st[r]);
       } else {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = kb + 8 * (r / 4) + 4 * hf + r % 4;
-          const float v = (key <= p_j && key >= lo_j) ? st[r] * scale_log2e : -INFINITY;
+          const float v = (key <= p_j && key >= lo_j) ? st[r] : -INFINITY;
           st[r] = v;
           tmax = fmaxf(tmax, v);
         }
       }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * scale_log2e;
       const float m_new = fmaxf(m, tmax);
       // a query whose window lies wholly beyond this tile has no key here yet
       const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      const float corr = exp2f(m - m_use);
+      const float corr = exp2_raw(m - m_use);
       float psum = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        st[r] = exp2f(st[r] - m_use);
+        st[r] = exp2_raw(fmaf(st[r], scale_log2e, -m_use));
         psum += st[r];
       }
       psum += __shfl_xor(psum, 32, 64);
