@@ -424,7 +424,8 @@ def test_paged_attention_mixed_batch(dtype, nH, nKV, hd, page_size, window):
 
 @pytest.mark.parametrize("nH,nKV,hd,page_size,window", [
     (8, 2, 32, 16, 0), (32, 8, 128, 16, 0), (6, 6, 64, 32, 0), (16, 1, 64, 16, 0),
-    (9, 3, 256, 16, 0), (8, 2, 64, 16, 37), (4, 4, 128, 48, 300), (36, 4, 32, 16, 0)])
+    (9, 3, 256, 16, 0), (8, 2, 64, 16, 37), (4, 4, 128, 48, 300), (36, 4, 32, 16, 0),
+    (16, 2, 128, 16, 0), (8, 2, 128, 32, 100), (16, 2, 128, 16, 45)])
 @pytest.mark.parametrize("kind", ["decode", "prefill", "mixed", "whole"])
 def test_paged_attention_mfma(nH, nKV, hd, page_size, window, kind):
     """The bfloat16 MFMA kernels: decode tokens over contexts that end at, before and after a

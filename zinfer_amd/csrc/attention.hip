@@ -406,13 +406,18 @@ extern "C" int zf_attn_decode_bf16(const void* q, const void* k_pool, const void
 // O^T tiles of 32 head elements x 32 queries.  A query at position p reads keys lo..p; a
 // portion may start anywhere in the context (earlier pages plus its own tokens).
 // Sequences with a single query token are left to the decode kernel when skip_single is set.
-template <int HD>
+// POW2: the page size is 1 << ps_shift, so the page and the row of a key are a shift and a
+// mask; a division by a page size known only at run time costs some 30 instructions, five
+// times a tile.
+template <int HD, bool POW2>
 __global__ __launch_bounds__(512) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int* __restrict__ block_table,
     const int* __restrict__ q_start, const int* __restrict__ ctx_len, bf16_t* __restrict__ out,
     float scale_log2e, int window, int nH, int nKV, int ps, int max_pages, int skip_single,
-    int q_tiles, int nsplit) {
+    int q_tiles, int nsplit, int ps_shift) {
+  auto page_of = [&](int key) { return POW2 ? key >> ps_shift : key / ps; };
+  auto row_of = [&](int key) { return POW2 ? key & (ps - 1) : key % ps; };
   extern __shared__ float xch[];      // partials of the waves that took other key tiles
   // workgroups are handed out in the order of blockIdx.x: kv heads vary fastest and the
   // last query tiles (the longest key ranges under the causal bound) come first, so the
@@ -429,7 +434,9 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
   const int nq = min(32, q_len - qbase);
   const int p_max = pos0 + nq - 1;
   const int G = nH / nKV;
-  const int wave = threadIdx.x / 64, nwaves = blockDim.x / 64;
+  // the wave's number as a scalar: what follows from it (its head, its key tiles, the pages
+  // of the value rows) is then computed once per wave, not per lane
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64), nwaves = blockDim.x / 64;
   const int lane = threadIdx.x % 64, j = lane % 32, hf = lane / 32;
   const bool q_valid = j < nq;
   const int p_j = pos0 + min(j, nq - 1);
@@ -468,10 +475,10 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
     // memory latency overlap the MFMAs and the soft-max.
     auto load_keys = [&](int kb, u32x4_t* dst) {
       const int key = min(max(kb + j, lo_min), p_max);
-      const int kpage = table[key / ps];
+      const int kpage = table[page_of(key)];
       // tiled pool: head elements 16 stp + 8 hf .. + 8 of row key % 16 of its 16-row group
       const bf16_t* kblk = k_pool + ((size_t)kpage * nKV + kvh) * ps * HD +
-                           (size_t)((key % ps) / 16) * 16 * HD + (hf * 16 + key % 16) * 8;
+                           (size_t)(row_of(key) / 16) * 16 * HD + (hf * 16 + key % 16) * 8;
 #pragma unroll
       for (int stp = 0; stp < HD / 16; ++stp)
         dst[stp] = *(const u32x4_t*)(kblk + (stp / 2) * 512 + (stp % 2) * 256);
@@ -488,10 +495,10 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
         const int base = kb + 16 * u;
         any[u] = base <= p_max && base + 16 > lo_min;
         const int safe = any[u] ? max(base, lo_min) : p_max;
-        const int vpage = table[safe / ps];
+        const int vpage = table[page_of(safe)];
         // tiled pool: head element 32 dt + j, rows 4 hf .. + 3 and 8 + 4 hf .. + 3 of the group
         const bf16_t* vb = v_pool + ((size_t)vpage * nKV + kvh) * ps * HD +
-                           (size_t)((base % ps) / 16) * 16 * HD + (j / 16) * 256 +
+                           (size_t)(row_of(base) / 16) * 16 * HD + (j / 16) * 256 +
                            (hf * 16 + j % 16) * 4;
 #pragma unroll
         for (int dt = 0; dt < HD / 32; ++dt) {
@@ -543,6 +550,7 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
 #pragma unroll
           for (int r = 0; r < 16; ++r) o[dt][r] *= corr;
       }
+      const bool edge_tile = !(kb >= lo_min && kb + 16 <= p_max && kb + 32 <= ctx);
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         // slots e = 0..7 <-> st[8 u + e]: keys kb + 16 u + 4 hf + e (e < 4) and
@@ -554,15 +562,22 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
         const bf16x8_t pf = *(bf16x8_t*)&pk;
         // keys at or beyond ctx hold nothing of this request; keys below lo_min may lie in
         // a page that was given back: both are zeroed (0 * NaN would poison the sum)
-        const int a0 = kb + 16 * u + 4 * hf, a1 = a0 + 8;
-        const int hi_lim = any[u] ? ctx : 0;
-        const bool edge = !any[u] || a0 < lo_min || a1 + 4 > ctx;
+        // (only tiles at an end of the key range have such rows: one test per wave, and the
+        // masks per lane are formed behind it)
+        u32x2_t keep0 = u32x2_t{~0u, ~0u}, keep1 = keep0;
+        if (edge_tile) {
+          const int a0 = kb + 16 * u + 4 * hf, a1 = a0 + 8;
+          const int hi_lim = any[u] ? ctx : 0;
+          keep0 = keep_range4(keep0, lo_min - a0, hi_lim - a0);
+          keep1 = keep_range4(keep1, lo_min - a1, hi_lim - a1);
+        }
 #pragma unroll
         for (int dt = 0; dt < HD / 32; ++dt) {
           u32x2_t v0 = vf[u][dt][0], v1 = vf[u][dt][1];
-          if (edge) {
-            v0 = keep_range4(v0, lo_min - a0, hi_lim - a0);
-            v1 = keep_range4(v1, lo_min - a1, hi_lim - a1);
+          if (edge_tile) {
+            asm volatile("");      // a real branch: as selects this costs every tile 16 operations
+            v0 = u32x2_t{v0[0] & keep0[0], v0[1] & keep0[1]};
+            v1 = u32x2_t{v1[0] & keep1[0], v1[1] & keep1[1]};
           }
           u32x4_t vv = u32x4_t{v0[0], v0[1], v1[0], v1[1]};
           o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8_t*)&vv, pf, o[dt], 0, 0, 0);
@@ -634,17 +649,25 @@ extern "C" int zf_attn_prefill_bf16(const void* q, const void* k_pool, const voi
   const int head_waves = G < 8 ? G : 8;
   dim3 block(64 * head_waves * nsplit);
   const size_t smem = nsplit > 1 ? (size_t)(nsplit - 1) * G * per_wave : 0;
-#define ZF_PRE(HD)                                                                              \
+  int ps_shift = -1;
+  for (int b = 4; b < 31; ++b)
+    if (page_size == (1 << b)) ps_shift = b;
+#define ZF_PRE_K(KERN)                                                                          \
   do {                                                                                          \
     if (smem > 64 * 1024) {                                                                     \
-      hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_kernel<HD>,                  \
+      hipError_t e = hipFuncSetAttribute((const void*)KERN,                                     \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
       if (e != hipSuccess) return (int)e;                                                       \
     }                                                                                           \
-    hipLaunchKernelGGL(attn_prefill_kernel<HD>, grid, block, smem, stream, (const bf16_t*)q,    \
+    hipLaunchKernelGGL(KERN, grid, block, smem, stream, (const bf16_t*)q,                       \
                        (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, q_start,      \
                        ctx_len, (bf16_t*)out, scale_log2e, window, nH, nKV, page_size,          \
-                       max_pages, skip_single, q_tiles, nsplit);                                \
+                       max_pages, skip_single, q_tiles, nsplit, ps_shift);                      \
+  } while (0)
+#define ZF_PRE(HD)                                                                              \
+  do {                                                                                          \
+    if (ps_shift >= 0) ZF_PRE_K((attn_prefill_kernel<HD, true>));                               \
+    else ZF_PRE_K((attn_prefill_kernel<HD, false>));                                            \
   } while (0)
   if (hd == 32) ZF_PRE(32);
   else if (hd == 64) ZF_PRE(64);
@@ -652,5 +675,6 @@ extern "C" int zf_attn_prefill_bf16(const void* q, const void* k_pool, const voi
   else if (hd == 256) ZF_PRE(256);
   else return -2;
 #undef ZF_PRE
+#undef ZF_PRE_K
   ZF_CHECK_LAUNCH();
 }
