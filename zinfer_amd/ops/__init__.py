@@ -246,7 +246,10 @@ def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = Fals
     128 x 128); otherwise the kernels that stage both operands through LDS (4: 256 x 256 when
     they still fill the chip, else 0: 128 x 128).  Measured on MI355X at the Qwen3-8B sizes."""
     if w_tiled:
-        return 10 if ((M + 127) // 128) * ((N + 255) // 256) >= 192 else 6
+        tiles = ((M + 127) // 128) * ((N + 255) // 256)
+        # between one and two 128 x 256 tiles per CU half the CUs hold two workgroups and half
+        # one, and the smaller tiles finish sooner (2048 tokens into 6144 outputs)
+        return 10 if tiles >= 192 and not 256 < tiles < 512 else 6
     tiles = ((M + 255) // 256) * ((N + 255) // 256)
     return 4 if tiles >= 160 else 0
 
