@@ -10,6 +10,8 @@
 //  * paged_attention_wave: one wave per (token, query head), 64 keys at a time with an
 //    online softmax, all in 32-bit.  Its result for a token depends only on that token's own
 //    keys, never on how the batch was cut.  Any head size, any page size.
+#include <type_traits>
+
 #include "zf_common.h"
 
 template <typename T>
@@ -486,26 +488,36 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
     const int kb0 = (lo_min / 32) * 32 + 32 * split, kstep = 32 * nsplit;
     u32x4_t kf[HD / 16];
     load_keys(kb0, kf);
-    for (int kb = kb0; kb <= p_max; kb += kstep) {
-      // values of this tile: keys kb + 16 u .. + 15 (one page) for u = 0, 1
-      u32x2_t vf[2][HD / 32][2];
-      bool any[2];
+    // values of a tile: keys kb + 16 u .. + 15 (one page) for u = 0, 1, into one of two
+    // register sets: a tile's values are requested a whole tile before its second product
+    // needs them (its keys: right after the first product of the tile before)
+    u32x2_t vfs[2][2][HD / 32][2];
+    bool anys[2][2];
+    auto load_vals = [&](int kb, auto BUF) {
+      constexpr int B = decltype(BUF)::value;
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         const int base = kb + 16 * u;
-        any[u] = base <= p_max && base + 16 > lo_min;
-        const int safe = any[u] ? max(base, lo_min) : p_max;
+        anys[B][u] = base <= p_max && base + 16 > lo_min;
+        const int safe = anys[B][u] ? max(base, lo_min) : p_max;
         const int vpage = table[page_of(safe)];
         // tiled pool: head element 32 dt + j, rows 4 hf .. + 3 and 8 + 4 hf .. + 3 of the group
         const bf16_t* vb = v_pool + ((size_t)vpage * nKV + kvh) * ps * HD +
-                           (size_t)(row_of(base) / 16) * 16 * HD + (j / 16) * 256 +
-                           (hf * 16 + j % 16) * 4;
+                           (size_t)(row_of(anys[B][u] ? base : safe) / 16) * 16 * HD +
+                           (j / 16) * 256 + (hf * 16 + j % 16) * 4;
 #pragma unroll
         for (int dt = 0; dt < HD / 32; ++dt) {
-          vf[u][dt][0] = *(const u32x2_t*)(vb + dt * 512);
-          vf[u][dt][1] = *(const u32x2_t*)(vb + dt * 512 + 128);
+          vfs[B][u][dt][0] = *(const u32x2_t*)(vb + dt * 512);
+          vfs[B][u][dt][1] = *(const u32x2_t*)(vb + dt * 512 + 128);
         }
       }
+    };
+    using Buf0 = std::integral_constant<int, 0>;
+    using Buf1 = std::integral_constant<int, 1>;
+    auto tile = [&](int kb, auto BUF, auto OTHER) {
+      constexpr int B = decltype(BUF)::value;
+      load_vals(kb + kstep, OTHER);      // any kb is safe: rows are clamped into live keys
+      __builtin_amdgcn_sched_barrier(0);
       // S^T: rows are the keys kb + (lane % 32), clamped into the keys that exist
       f32x16_t st;
 #pragma unroll
@@ -513,7 +525,7 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
 #pragma unroll
       for (int stp = 0; stp < HD / 16; ++stp)
         st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&kf[stp], qf[stp], st, 0, 0, 0);
-      if (kb + kstep <= p_max) load_keys(kb + kstep, kf);   // next tile's keys, in flight from here
+      load_keys(kb + kstep, kf);       // next tile's keys, in flight from here (rows clamped)
       // st[r]: key kb + 8 (r / 4) + 4 hf + r % 4, query column j
       // the scale (> 0) goes into the exponent's multiply-add: max over the raw scores
       float tmax = -INFINITY;
@@ -567,13 +579,13 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
         u32x2_t keep0 = u32x2_t{~0u, ~0u}, keep1 = keep0;
         if (edge_tile) {
           const int a0 = kb + 16 * u + 4 * hf, a1 = a0 + 8;
-          const int hi_lim = any[u] ? ctx : 0;
+          const int hi_lim = anys[B][u] ? ctx : 0;
           keep0 = keep_range4(keep0, lo_min - a0, hi_lim - a0);
           keep1 = keep_range4(keep1, lo_min - a1, hi_lim - a1);
         }
 #pragma unroll
         for (int dt = 0; dt < HD / 32; ++dt) {
-          u32x2_t v0 = vf[u][dt][0], v1 = vf[u][dt][1];
+          u32x2_t v0 = vfs[B][u][dt][0], v1 = vfs[B][u][dt][1];
           if (edge_tile) {
             asm volatile("");      // a real branch: as selects this costs every tile 16 operations
             v0 = u32x2_t{v0[0] & keep0[0], v0[1] & keep0[1]};
@@ -583,6 +595,12 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
           o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8_t*)&vv, pf, o[dt], 0, 0, 0);
         }
       }
+    };
+    load_vals(kb0, Buf0{});
+    for (int kb = kb0; kb <= p_max; kb += 2 * kstep) {
+      tile(kb, Buf0{}, Buf1{});
+      if (kb + kstep <= p_max) tile(kb + kstep, Buf1{}, Buf0{});
+      else load_vals(kb + 2 * kstep, Buf0{});     // keeps the register sets in step (unused)
     }
     if (nsplit > 1) {     // one pass over g here: every wave comes by exactly once
       constexpr int PER_LANE = HD / 2 + 2;       // a wave's O^T values per lane, max and sum
