@@ -106,6 +106,22 @@ def test_serving_widths(mode, tmp_path_factory):
     print(f"{name} bfloat16 {mode}: worst error {worst:.3g}")
 
 
+def test_pages_that_do_not_divide_64(tmp_path_factory):
+    """Pages of 48 rows: a request of 64 tokens needs two of them, which the pool made for
+    `max_tokens` (requests rounded up to 64) has to allow for."""
+    name, dtype = "D", "bfloat16"
+    path = tiny.model_dir_of(name, str(tmp_path_factory.getbasetemp()), torch.bfloat16)
+    cfg = tiny.CONFIGS[name]
+    requests = {f"p{i}": tiny.random_tokens(n, cfg["vocab_size"], 700 + i)
+                for i, n in enumerate((64, 65, 130, 33))}
+    w = tiny.weights_of(name, torch.bfloat16)
+    ref = {rid: plain.model_forward_batched(cfg, w, t).numpy() for rid, t in requests.items()}
+    for mode in ("whole", "mixed"):
+        steps = MODES[mode](requests)
+        outputs, _ = _replay(path, dtype, steps, 48)
+        _compare(steps, outputs, ref, cfg["vocab_size"], LOGITS_TOL_BF16)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_mixed_many_requests_reuse_pages(dtype, tmp_path_factory):
     """Nine requests through a pool that holds four: every page is used several times."""

@@ -38,7 +38,11 @@ def make_engine(model_dir: str, dtype: str, max_tokens: int, device: str = "cuda
                 page_size: int = PAGE_SIZE, poison_freed: bool = False) -> Engine:
     from ..models.build import load_model
     _, model = load_model(model_dir, dtype, device)
-    num_pages = (max_tokens + page_size - 1) // page_size
+    # max_tokens counts every live request rounded up to 64 tokens; with pages that do not
+    # divide 64 a request of 64 tokens still needs ceil(64 / page_size) of them
+    units = (max_tokens + 63) // 64
+    num_pages = max((max_tokens + page_size - 1) // page_size,
+                    units * ((64 + page_size - 1) // page_size) if 64 % page_size else 0)
     return Engine(model, page_size=page_size, num_pages=num_pages,
                   max_requests=MAX_LIVE_REQUESTS, poison_freed=poison_freed)
 
