@@ -247,6 +247,41 @@ def test_graph_replays_equal_eager_steps(dtype, tmp_path_factory):
     assert a.graph_replays >= 10 and b.graph_replays == 0
 
 
+def test_graph_replays_with_forty_requests(tmp_path_factory):
+    """Forty decode tokens in a step: the product for 17 to 64 tokens and the kernel that adds
+    its partials, sums them into the residual and norms, inside a captured graph, against the
+    same kernels launched one by one and against the plain implementation."""
+    from zinfer_amd.engine import Engine, StepEntry
+    from zinfer_amd.models.build import load_model
+    name, dtype = "E", "bfloat16"
+    path = tiny.model_dir_of(name, str(tmp_path_factory.getbasetemp()), torch.bfloat16)
+    cfg = tiny.CONFIGS[name]
+    V = cfg["vocab_size"]
+    reqs = {f"q{i}": tiny.random_tokens(3 + i % 7 + 8, V, 800 + i) for i in range(40)}
+    w = tiny.weights_of(name, torch.bfloat16)
+    engines = []
+    for graphs in (True, False):
+        _, model = load_model(path, dtype, DEV)
+        engines.append(Engine(model, page_size=16, num_pages=40 * 2 + 8, max_requests=48,
+                              use_graphs=graphs))
+    a, b = engines
+    for eng in (a, b):
+        eng.step([StepEntry(r, t[:-8], []) for r, t in reqs.items()])
+    got = {r: [] for r in reqs}
+    for k in range(8, 0, -1):
+        entries = [StepEntry(r, t[len(t) - k:len(t) - k + 1], [0]) for r, t in reqs.items()]
+        la, lb = a.step(entries), b.step(entries)
+        assert torch.equal(la, lb), f"decode step {8 - k}: replay differs from eager launches"
+        for i, r in enumerate(reqs):
+            got[r].append(la[i].float().cpu().numpy())
+        torch.cuda.synchronize()
+    assert a.graph_replays >= 6 and b.graph_replays == 0
+    for r in list(reqs)[::7]:
+        ref = plain.model_forward_batched(cfg, w, reqs[r]).numpy()[-8:]
+        err = np.abs(np.stack(got[r]).astype(np.float64) - ref).max() / np.abs(ref).max()
+        assert err <= LOGITS_TOL_BF16, (r, err)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decode_steps_in_a_row_equal_single_steps(dtype, tmp_path_factory):
     """Several decode steps without the host between them (the device moves tokens,
