@@ -1,0 +1,49 @@
+"""Which kernel serves which size: the pure decisions of `zinfer_amd.ops`, without a GPU."""
+import pytest
+
+from zinfer_amd import ops
+
+SHAPES = [(6144, 4096), (4096, 4096), (24576, 4096), (4096, 12288), (151936, 4096), (192, 64),
+          (1024, 320), (4160, 1088)]
+
+
+@pytest.mark.parametrize("N,K", SHAPES)
+def test_products_of_17_to_64_tokens(N, K):
+    for M in range(1, 200):
+        plan = ops._mid_plan(M, N, K, True)
+        if plan is None:
+            continue
+        assert 16 < M <= 64 and N % 16 == 0 and K % (256 if M <= 32 else 128) == 0
+        assert 1 <= plan <= K // (256 if M <= 32 else 128), "more splits than k-tiles"
+        assert ops._mid_plan(M, N, K, True, swiglu=True) == 1, "SwiGLU is never split along K"
+        assert ops._mid_plan(M, N, K, False) is None, "only pre-tiled weights"
+    # the served sizes do take this kernel at 64 tokens (and the wide one from 17 on)
+    if K % 128 == 0 and N % 16 == 0:
+        assert ops._mid_plan(64, N, K, True) is not None
+    if K % 256 == 0 and N >= 16384:
+        assert ops._mid_plan(17, N, K, True) is not None
+
+
+@pytest.mark.parametrize("N,K", SHAPES)
+def test_tiled_products(N, K):
+    for M in (65, 100, 128, 300, 512, 1024, 2048, 8192):
+        ks = ops._tile_ksplit(M, N, K)
+        assert 1 <= ks <= 16
+        if ks > 1:
+            assert K // 64 // ks >= 8, "every workgroup keeps at least 8 k-tiles"
+            tiles = ((M + 127) // 128) * ((N + 127) // 128)
+            assert tiles < 192 and tiles * ks <= 512
+        assert ops._tile_variant(M, N, True) in (6, 10)
+        assert ops._tile_variant(M, N, False) in (0, 4)
+    # 2048 tokens at the served widths: 128 x 256 tiles, except where they would fill the chip
+    # one and a half times
+    assert ops._tile_variant(2048, 24576, True) == 10 and ops._tile_variant(2048, 4096, True) == 10
+    assert ops._tile_variant(2048, 6144, True) == 6
+
+
+def test_weight_streaming_plans():
+    for N, K in SHAPES:
+        for M in (1, 8, 16, 17, 64):
+            for tiled in (True, False):
+                rg, ks = ops._skinny_plan(M, N, K, tiled)
+                assert rg in (1, 2, 4) and 1 <= ks <= 16
