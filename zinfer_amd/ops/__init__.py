@@ -228,7 +228,7 @@ def _mid_plan(M: int, N: int, K: int, w_tiled: bool, swiglu: bool = False):
     """Workgroups along K if the kernel for 17 to 64 tokens (128 outputs per workgroup, the
     tokens through LDS) covers the product, else None: above 32 tokens, and from 17 on a wide
     output, it beats the weight-streaming kernel, which re-reads the tokens for every few
-    rows of the weight.  Split along K until about 192 workgroups run, each keeping 1024 of K.
+    rows of the weight.  Split along K until up to 256 workgroups run, each keeping 1024 of K.
     Measured on MI355X at the Qwen3-8B sizes."""
     if not (w_tiled and 16 < M <= 64 and N % 16 == 0 and K % (256 if M <= 32 else 128) == 0):
         return None
@@ -237,7 +237,7 @@ def _mid_plan(M: int, N: int, K: int, w_tiled: bool, swiglu: bool = False):
     if swiglu:
         return 1
     tiles = (N + 127) // 128
-    return max(1, min(192 // tiles, K // 1024))
+    return max(1, min(256 // tiles, K // 1024))
 
 
 def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = False) -> int:
