@@ -31,19 +31,34 @@ class Scratch:
     def __init__(self, device):
         self.device = device
         self._bufs: Dict[str, torch.Tensor] = {}
+        self._views: Dict[str, Dict[tuple, torch.Tensor]] = {}   # per buffer: (shape, dtype) -> view
         self.generation = 0            # goes up whenever a buffer moves (captured graphs die)
 
     def get(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+        key = (tuple(shape), dtype)
+        views = self._views.get(name)
+        if views is not None:
+            view = views.get(key)
+            if view is not None:
+                return view
         n = 1
         for d in shape:
             n *= int(d)
-        nbytes = max(n, 1) * torch.empty((), dtype=dtype).element_size()
+        size = _ELEMENT_SIZE.get(dtype) or torch.empty((), dtype=dtype).element_size()
+        nbytes = max(n, 1) * size
         buf = self._bufs.get(name)
         if buf is None or buf.numel() < nbytes:
             buf = torch.empty(((nbytes + 255) // 256 * 256,), dtype=torch.uint8, device=self.device)
             self._bufs[name] = buf
+            self._views[name] = {}
             self.generation += 1
-        return buf[:n * torch.empty((), dtype=dtype).element_size()].view(dtype).view(*shape)
+        view = buf[:n * size].view(dtype).view(*shape)
+        self._views[name][key] = view
+        return view
+
+
+_ELEMENT_SIZE = {torch.float32: 4, torch.bfloat16: 2, torch.int32: 4, torch.int64: 8,
+                 torch.float16: 2, torch.uint8: 1, torch.float64: 8}
 
 
 @dataclass
