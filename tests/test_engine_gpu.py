@@ -96,7 +96,7 @@ def test_replay_modes(name, dtype, mode, tmp_path_factory):
 @pytest.mark.parametrize("mode", ["whole", "mixed", "prefill_then_32"])
 def test_serving_widths(mode, tmp_path_factory):
     """Two layers of the served model's widths in bfloat16: whole prompts of 8 to 300 tokens
-    (one kernel choice each: weight streaming, 17 to 64 tokens, tiled, with their splits along
+    (one kernel choice each: weight streaming, 17 to 128 tokens, tiled, with their splits along
     K), mixed batches, and decoding, against the plain implementation."""
     name = "W"
     path, cfg, requests, ref = _setup(name, "bfloat16", tmp_path_factory)
@@ -248,7 +248,7 @@ def test_graph_replays_equal_eager_steps(dtype, tmp_path_factory):
 
 
 def test_graph_replays_with_forty_requests(tmp_path_factory):
-    """Forty decode tokens in a step: the product for 17 to 64 tokens and the kernel that adds
+    """Forty decode tokens in a step: the product for 17 to 128 tokens and the kernel that adds
     its partials, sums them into the residual and norms, inside a captured graph, against the
     same kernels launched one by one and against the plain implementation."""
     from zinfer_amd.engine import Engine, StepEntry

@@ -8,18 +8,19 @@ SHAPES = [(6144, 4096), (4096, 4096), (24576, 4096), (4096, 12288), (151936, 409
 
 
 @pytest.mark.parametrize("N,K", SHAPES)
-def test_products_of_17_to_64_tokens(N, K):
+def test_products_of_17_to_128_tokens(N, K):
     for M in range(1, 200):
         plan = ops._mid_plan(M, N, K, True)
         if plan is None:
             continue
-        assert 16 < M <= 64 and N % 16 == 0 and K % (256 if M <= 32 else 128) == 0
+        assert 16 < M <= 128 and N % 16 == 0 and K % (256 if M <= 32 else 128) == 0
         assert 1 <= plan <= K // (256 if M <= 32 else 128), "more splits than k-tiles"
         assert ops._mid_plan(M, N, K, True, swiglu=True) == 1, "SwiGLU is never split along K"
         assert ops._mid_plan(M, N, K, False) is None, "only pre-tiled weights"
-    # the served sizes do take this kernel at 64 tokens (and the wide one from 17 on)
+    # the served sizes do take this kernel at 64 and 128 tokens (and the wide one from 17 on)
     if K % 128 == 0 and N % 16 == 0:
         assert ops._mid_plan(64, N, K, True) is not None
+        assert ops._mid_plan(128, N, K, True) is not None and ops._mid_plan(129, N, K, True) is None
     if K % 256 == 0 and N >= 16384:
         assert ops._mid_plan(17, N, K, True) is not None
 

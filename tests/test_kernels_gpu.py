@@ -130,11 +130,11 @@ def test_gemm_pretiled_weights(M, N, K, o_dtype, accumulate):
     assert rel_err(got, plain_out) <= (tol(o_dtype) if not accumulate else 2e-5)
 
 
-@pytest.mark.parametrize("M", [17, 32, 33, 47, 64])
+@pytest.mark.parametrize("M", [17, 32, 33, 47, 64, 65, 100, 128])
 @pytest.mark.parametrize("N,K", [(192, 4096), (4160, 1024), (16448, 512), (320, 384)])
 @pytest.mark.parametrize("kind", ["store", "store32", "accumulate", "swiglu"])
-def test_gemm_17_to_64_tokens(M, N, K, kind):
-    """The kernel for 17 to 64 tokens on pre-tiled weights (the tokens through LDS, 128
+def test_gemm_17_to_128_tokens(M, N, K, kind):
+    """The kernel for 17 to 128 tokens on pre-tiled weights (the tokens through LDS, 128
     outputs per workgroup, split along K when the tiles are few): outputs that are no
     multiple of its tile, one and several workgroups along K, each epilogue.  The tokens
     differ in scale, so a row that lands in another token's place shows."""
@@ -162,8 +162,8 @@ def test_gemm_17_to_64_tokens(M, N, K, kind):
     assert rel_err(got, want) <= (2e-5 if acc else tol(o_dtype))
 
 
-@pytest.mark.parametrize("M", [17, 33, 64, 65, 200])
-@pytest.mark.parametrize("N,K", [(192, 4096), (4160, 2048), (8192, 1024)])
+@pytest.mark.parametrize("M", [17, 33, 64, 65, 128, 129, 200])
+@pytest.mark.parametrize("N,K", [(192, 4096), (4160, 2048), (8192, 1024), (256, 2112)])
 def test_gemm_sum_norm(M, N, K):
     """The residual sum whose split-K partials are added, summed into the residual and normed
     by one kernel, against sum and norm in 64-bit.  Tokens of different scale: another row's

@@ -38,7 +38,7 @@ TINY_D = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden
 
 # a fifth shape with the serving model's head size and widths that are multiples of 128 (and a
 # feed-forward width of 2048), so that the kernels chosen by size run inside the engine tests:
-# the product for 17 to 64 tokens, the products split along K whose partials one kernel adds,
+# the product for 17 to 128 tokens, the products split along K whose partials one kernel adds,
 # sums into the residual and norms, the 128 x 256 tiles, the head-size-128 attention
 TINY_E = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2,
               hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=128,

@@ -622,19 +622,23 @@ extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, i
   }
 }
 
-// 17 to 64 tokens on pre-tiled W.  The weight-streaming kernel below re-reads the tokens for
+// 17 to 128 tokens on pre-tiled W.  The weight-streaming kernel below re-reads the tokens for
 // every 16 * RG rows of W, which at 64 tokens is as much traffic as W itself; here a workgroup
-// takes 128 rows of W, the tokens of a k-tile go through LDS once for its 4 waves, and the
-// k-tiles are 128 or 256 wide so that 32 or 64 KB of W are in flight per workgroup.  ksplit
-// workgroups share a tile's K (ws: float32 [ksplit, M, N]) when the tiles do not fill the chip.
-//   M <= 32: tiles of 32 tokens, K % 256 == 0;  M <= 64: tiles of 64 tokens, K % 128 == 0.
+// takes 128 rows of W, its 4 waves side by side along them, the tokens of a k-tile go through
+// LDS once for all of them, and the k-tiles are 128 or 256 wide so that 32 or 64 KB of W are
+// in flight per workgroup.  ksplit workgroups share a tile's K (ws: float32 [ksplit, M, N])
+// when the tiles do not fill the chip.
+//   M <= 32: tiles of 32 tokens, K % 256 == 0;  M <= 64: 64 tokens;  M <= 128: 128 tokens;
+//   both K % 128 == 0.
 extern "C" int zf_gemm_bf16_mid(const void* A, const void* W, void* C, void* ws, int M, int N,
                                 int K, int epi, int ksplit, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || ksplit < 1 || (epi == EPI_SWIGLU && N % 32 != 0)) return -3;
+  if (M > 128 || ksplit < 1 || (epi == EPI_SWIGLU && N % 32 != 0)) return -3;
   if (M <= 32)
     return launch_tile_wdirect<32, 128, 32, 32, 256>(A, W, C, M, N, K, epi, stream, ws, ksplit);
-  return launch_tile_wdirect<64, 128, 64, 32, 128>(A, W, C, M, N, K, epi, stream, ws, ksplit);
+  if (M <= 64)
+    return launch_tile_wdirect<64, 128, 64, 32, 128>(A, W, C, M, N, K, epi, stream, ws, ksplit);
+  return launch_tile_wdirect<128, 128, 128, 32, 128>(A, W, C, M, N, K, epi, stream, ws, ksplit);
 }
 
 enum { NORM_NONE = 0, NORM_FOLD = 1, NORM_GIVEN = 2 };
@@ -1004,7 +1008,7 @@ __global__ __launch_bounds__(1024) void reduce_sum_norm_kernel(
 }
 
 // C += A W^T in 32-bit with ksplit >= 2 workgroups along K, and normed = bfloat16 RMSNorm of
-// the sum's rows, from the kernel that adds the partials.  M <= 64: the kernel for 17 to 64
+// the sum's rows, from the kernel that adds the partials.  M <= 128: the kernels for 17 to 128
 // tokens; above: 128 x 128 tiles.  W pre-tiled; ws: float32 [ksplit, M, N].
 extern "C" int zf_gemm_bf16_splitk_sum_norm(const void* A, const void* W, void* C, void* ws,
                                             const float* gain, float eps, void* normed, int M,
@@ -1018,6 +1022,9 @@ extern "C" int zf_gemm_bf16_splitk_sum_norm(const void* A, const void* W, void* 
   else if (M <= 64)
     rc = launch_tile_wdirect<64, 128, 64, 32, 128>(A, W, C, M, N, K, EPI_ACC_F32, stream, ws,
                                                    ksplit, false);
+  else if (M <= 128 && K % 128 == 0)
+    rc = launch_tile_wdirect<128, 128, 128, 32, 128>(A, W, C, M, N, K, EPI_ACC_F32, stream, ws,
+                                                     ksplit, false);
   else
     rc = launch_tile_wdirect<128, 128, 64, 64>(A, W, C, M, N, K, EPI_ACC_F32, stream, ws, ksplit,
                                                false);

@@ -232,13 +232,18 @@ def _skinny_plan(M: int, N: int, K: int, tiled: bool):
     return rg, ks
 
 
+MID_MAX_M = 128
+
+
 def _mid_plan(M: int, N: int, K: int, w_tiled: bool, swiglu: bool = False):
-    """Workgroups along K if the kernel for 17 to 64 tokens (128 outputs per workgroup, the
+    """Workgroups along K if the kernel for 17 to 128 tokens (128 outputs per workgroup, the
     tokens through LDS) covers the product, else None: above 32 tokens, and from 17 on a wide
     output, it beats the weight-streaming kernel, which re-reads the tokens for every few
-    rows of the weight.  Split along K until up to 256 workgroups run, each keeping 1024 of K.
-    Measured on MI355X at the Qwen3-8B sizes."""
-    if not (w_tiled and 16 < M <= 64 and N % 16 == 0 and K % (256 if M <= 32 else 128) == 0):
+    rows of the weight, and from 65 to 128 tokens the 128 x 128 tiles, two of whose waves load
+    each part of the weight.  Split along K until up to 256 workgroups run, each keeping 1024
+    of K.  Measured on MI355X at the Qwen3-8B sizes."""
+    if not (w_tiled and 16 < M <= MID_MAX_M and N % 16 == 0
+            and K % (256 if M <= 32 else 128) == 0):
         return None
     if M <= 32 and N < 16384:
         return None
@@ -317,7 +322,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         if mid is not None:
             ws = _workspace("gemm_splitk", mid * M * N, torch.float32, a.device) if mid > 1 else None
             _check(lib.zf_gemm_bf16_mid(_ptr(a), _ptr(w), _ptr(out), _ptr(ws), M, N, K, epi, mid,
-                                        _stream()), "gemm (17 to 64 tokens)")
+                                        _stream()), "gemm (17 to 128 tokens)")
         elif M <= SKINNY_MAX_M:
             rg, ks = _skinny_plan(M, N, K, w_tiled)
             ws = _workspace("gemm_splitk", ks * M * N, torch.float32, a.device) if ks > 1 else None
@@ -379,11 +384,13 @@ def norm_gemm(x: torch.Tensor, gain: torch.Tensor, eps: float, w: torch.Tensor,
 
 def sum_norm_plan(M: int, N: int, K: int, w: torch.Tensor, w_tiled: bool):
     """Workgroups along K if ``gemm_sum_norm`` covers residual += a w^T: a product that is
-    split along K anyway (17 to 64 tokens, or a few hundred tokens on a narrow output), whose
+    split along K anyway (17 to 128 tokens, or a few hundred tokens on a narrow output), whose
     partials one kernel can add, sum into the residual and norm; else None."""
     if not (w_tiled and w.dtype == torch.bfloat16 and w.is_cuda and N % 16 == 0 and N <= 8192):
         return None
-    ks = _mid_plan(M, N, K, True) if M <= SKINNY_MAX_M else _tile_ksplit(M, N, K)
+    ks = _mid_plan(M, N, K, True) if M <= MID_MAX_M else None
+    if ks is None and M > SKINNY_MAX_M:
+        ks = _tile_ksplit(M, N, K)
     return ks if ks is not None and ks >= 2 else None
 
 
@@ -496,7 +503,7 @@ def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bo
     lib = build.load("gemm")
     if _mid_plan(M, N, K, w_tiled, swiglu=True) is not None:
         _check(lib.zf_gemm_bf16_mid(_ptr(a), _ptr(w), _ptr(out), _ptr(None), M, N, K, _EPI_SWIGLU,
-                                    1, _stream()), "gemm_swiglu (17 to 64 tokens)")
+                                    1, _stream()), "gemm_swiglu (17 to 128 tokens)")
     elif M <= SKINNY_MAX_M:
         rg = 4 if (M > 16 and N >= 16384) else 2
         _check(lib.zf_gemm_bf16_skinny(_ptr(a), _ptr(w), _ptr(out), _ptr(None), M, N, K,
