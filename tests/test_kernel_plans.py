@@ -33,8 +33,10 @@ def test_tiled_products(N, K):
         if ks > 1:
             assert K // 64 // ks >= 8, "every workgroup keeps at least 8 k-tiles"
             tiles = ((M + 127) // 128) * ((N + 127) // 128)
-            assert tiles < 192 and tiles * ks <= 512
-        assert ops._tile_variant(M, N, True) in (6, 10)
+            assert tiles < 192 and tiles * ks <= 256
+        assert ops._tile_variant(M, N, True, False, K) in (6, 10, 16)
+        if ops._tile_variant(M, N, True, False, K) == 16:
+            assert K % 128 == 0
         assert ops._tile_variant(M, N, False) in (0, 4)
     # 2048 tokens at the served widths: 128 x 256 tiles, except where they would fill the chip
     # one and a half times

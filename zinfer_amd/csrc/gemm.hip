@@ -598,7 +598,8 @@ static int launch_tile(const void* A, const void* W, void* C, int M, int N, int 
 
 // variant, plain W: 0 = 128x128 (waves 64x64), 4 = 256x256 (waves 128x64, 8 waves);
 //          pre-tiled W (w_tiled; N % 16 == 0 and K % 64 == 0), taken straight from memory
-//          into the MFMA operands: 6 = 128x128 (waves 64x64), 10 = 128x256 (waves 128x64: no
+//          into the MFMA operands: 6 = 128x128 (waves 64x64), 16 = 128x128 with k-tiles of 128
+//          and the waves side by side (128x32: for few tiles; K % 128 == 0), 10 = 128x256 (waves 128x64: no
 //          two waves load the same part of W, two workgroups share a CU, and W is loaded
 //          two k-tiles ahead when their number is even)
 extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, int N, int K,
@@ -608,6 +609,8 @@ extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, i
   if (w_tiled) {
     if (N % 16 != 0 || K % 64 != 0) return -3;
     if (variant == 6) return launch_tile_wdirect<128, 128, 64, 64>(A, W, C, M, N, K, epi, stream);
+    if (variant == 16)
+      return launch_tile_wdirect<128, 128, 128, 32, 128>(A, W, C, M, N, K, epi, stream);
     if (variant == 10) {
       if (K % (2 * TK) == 0)     // W two k-tiles ahead: an even number of k-tiles
         return launch_tile_wdirect<128, 256, 128, 64, TK, true>(A, W, C, M, N, K, epi, stream);
@@ -667,6 +670,8 @@ extern "C" int zf_gemm_bf16_tile_splitk(const void* A, const void* W, void* C, v
                                         int N, int K, int epi, int ksplit, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (ksplit < 2 || ksplit > 64 || epi == EPI_SWIGLU) return -3;
+  if (K % 128 == 0)      // the waves side by side along the outputs: W is loaded once
+    return launch_tile_wdirect<128, 128, 128, 32, 128>(A, W, C, M, N, K, epi, stream, ws, ksplit);
   return launch_tile_wdirect<128, 128, 64, 64>(A, W, C, M, N, K, epi, stream, ws, ksplit);
 }
 
@@ -1022,7 +1027,7 @@ extern "C" int zf_gemm_bf16_splitk_sum_norm(const void* A, const void* W, void* 
   else if (M <= 64)
     rc = launch_tile_wdirect<64, 128, 64, 32, 128>(A, W, C, M, N, K, EPI_ACC_F32, stream, ws,
                                                    ksplit, false);
-  else if (M <= 128 && K % 128 == 0)
+  else if (K % 128 == 0)
     rc = launch_tile_wdirect<128, 128, 128, 32, 128>(A, W, C, M, N, K, EPI_ACC_F32, stream, ws,
                                                      ksplit, false);
   else

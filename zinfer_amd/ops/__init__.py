@@ -253,28 +253,34 @@ def _mid_plan(M: int, N: int, K: int, w_tiled: bool, swiglu: bool = False):
     return max(1, min(256 // tiles, K // 1024))
 
 
-def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = False) -> int:
+def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = False,
+                  K: int = 0) -> int:
     """Which tiled kernel: with pre-tiled weights the kernels that take W straight from
-    memory (10: 128 x 256 tiles, two workgroups to a CU, when they fill the chip; else 6:
-    128 x 128); otherwise the kernels that stage both operands through LDS (4: 256 x 256 when
-    they still fill the chip, else 0: 128 x 128).  Measured on MI355X at the Qwen3-8B sizes."""
+    memory (10: 128 x 256 tiles, two workgroups to a CU, when they fill the chip; else 128 x
+    128 tiles, 16: with the waves side by side and k-tiles of 128 when there are few of them,
+    6: with 2 x 2 waves); otherwise the kernels that stage both operands through LDS (4: 256
+    x 256 when they still fill the chip, else 0: 128 x 128).  Measured on MI355X at the
+    Qwen3-8B sizes."""
     if w_tiled:
         tiles = ((M + 127) // 128) * ((N + 255) // 256)
         # between one and two 128 x 256 tiles per CU half the CUs hold two workgroups and half
         # one, and the smaller tiles finish sooner (2048 tokens into 6144 outputs)
-        return 10 if tiles >= 192 and not 256 < tiles < 512 else 6
+        if tiles >= 192 and not 256 < tiles < 512:
+            return 10
+        small = ((M + 127) // 128) * ((N + 127) // 128)
+        return 16 if small < 256 and K > 0 and K % 128 == 0 else 6
     tiles = ((M + 255) // 256) * ((N + 255) // 256)
     return 4 if tiles >= 160 else 0
 
 
 def _tile_ksplit(M: int, N: int, K: int) -> int:
     """Workgroups per 128 x 128 tile along K: products of a few hundred tokens on a narrow
-    output have too few tiles for 256 CUs; split them until about 512 workgroups run, each
-    keeping at least 8 k-tiles.  The partials cost ksplit * M * N floats of traffic."""
+    output have too few tiles for 256 CUs; split them until about 256 workgroups run, each
+    keeping at least 8 k-tiles of 64.  The partials cost ksplit * M * N floats of traffic."""
     tiles = ((M + 127) // 128) * ((N + 127) // 128)
     if tiles >= 192:
         return 1
-    ksplit = min(512 // tiles, K // 64 // 8, 16)
+    ksplit = min(256 // tiles, K // 64 // 8, 16)
     return ksplit if ksplit >= 2 else 1
 
 
@@ -338,7 +344,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
                        "gemm (tiled, split along K)")
                 return
             _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, epi,
-                                         _tile_variant(M, N, w_tiled, accumulate),
+                                         _tile_variant(M, N, w_tiled, accumulate, K),
                                          1 if w_tiled else 0, _stream()),
                    "gemm (tiled)")
         return
@@ -511,7 +517,7 @@ def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bo
                "gemm_swiglu (weight streaming)")
     else:
         _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, _EPI_SWIGLU,
-                                     _tile_variant(M, N, w_tiled), 1 if w_tiled else 0,
+                                     _tile_variant(M, N, w_tiled, False, K), 1 if w_tiled else 0,
                                      _stream()),
                "gemm_swiglu (tiled)")
 
