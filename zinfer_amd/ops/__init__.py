@@ -308,7 +308,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     ``w`` went through ``pretile_weight``.
 
     bfloat16 operands with K a multiple of 8 go to the MFMA kernels (weight streaming for up
-    to 64 rows of ``a``, LDS-tiled above); everything else, the whole 32-bit path included,
+    to 16 rows of ``a``, and up to 64 where the kernel for 17 to 128 rows does not cover the
+    sizes; LDS-tiled above); everything else, the whole 32-bit path included,
     goes to the FMA kernel, whose results do not depend on how rows are batched."""
     _need_gpu(a, w, out)
     M, K = a.shape
