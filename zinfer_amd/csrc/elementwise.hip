@@ -2,6 +2,9 @@
 // arg-max.  Formulas follow the reference's CPU kernels (src/kernel/core/cpu.zig,
 // src/kernel/attention/rope.zig); all arithmetic is 32-bit, storage is float or bfloat16.
 #include "zf_common.h"
+#include "zf_no_alloc.h"
+#include <mutex>
+#include <stdio.h>
 
 // ---------------------------------------------------------------- embedding: x[t,:] = E[id[t],:]
 template <typename TW>
@@ -479,6 +482,58 @@ extern "C" int zf_argmax(const float* logits, int* out, void* ws, int n, int V,
                      pidx, V, nchunks);
   hipLaunchKernelGGL(argmax_final_kernel, dim3(n), dim3(256), 0, stream, pval, pidx, out,
                      nchunks);
+  ZF_CHECK_LAUNCH();
+}
+
+// The same arg-max with its partial results in a device array of this file instead of a buffer
+// of the caller's: for callers that cannot allocate (zf_no_alloc.h).  In host code `scratch`
+// is only a stand-in for the symbol, not a device address: the address of each GPU's copy is
+// looked up once per device and only that pointer is ever handed to a kernel.
+static __device__ __align__(256) unsigned char scratch[ZF_ARGMAX_NO_ALLOC_MAX_PARTIALS * 8];
+
+#define ZF_NO_ALLOC_MAX_DEVICES 64
+static void* scratch_ptr[ZF_NO_ALLOC_MAX_DEVICES];   // per device, null until looked up
+static std::mutex scratch_mutex;
+
+static int scratch_of_current_device(void** ptr) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= ZF_NO_ALLOC_MAX_DEVICES) return 1;
+  std::lock_guard<std::mutex> guard(scratch_mutex);
+  if (scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return 1;
+    scratch_ptr[dev] = p;
+  }
+  *ptr = scratch_ptr[dev];
+  return 0;
+}
+
+extern "C" int zf_argmax_no_alloc(const float* logits, int* out, int n, int V,
+                                  hipStream_t stream) {
+  if (logits == nullptr || out == nullptr || n < 0 || V < 1) {
+    fprintf(stderr, "zf_argmax_no_alloc: bad argument (logits %p, out %p, n %d, V %d)\n",
+            (const void*)logits, (void*)out, n, V);
+    return ZF_NO_ALLOC_BAD_ARGUMENT;
+  }
+  if (n == 0) return ZF_NO_ALLOC_OK;
+  const long long nchunks = ((long long)V + ARGMAX_CHUNK - 1) / ARGMAX_CHUNK;
+  if ((long long)n * nchunks > ZF_ARGMAX_NO_ALLOC_MAX_PARTIALS) {
+    fprintf(stderr, "zf_argmax_no_alloc: %d rows of %d logits need %lld partial results, the "
+            "fixed array holds %d\n", n, V, (long long)n * nchunks,
+            ZF_ARGMAX_NO_ALLOC_MAX_PARTIALS);
+    return ZF_NO_ALLOC_TOO_LARGE;
+  }
+  void* ws = nullptr;
+  if (scratch_of_current_device(&ws) != 0) {
+    fprintf(stderr, "zf_argmax_no_alloc: the address of the device array could not be had\n");
+    return ZF_NO_ALLOC_NO_SCRATCH;
+  }
+  float* pval = (float*)ws;
+  int* pidx = (int*)(pval + (size_t)n * nchunks);
+  hipLaunchKernelGGL(argmax_chunk_kernel, dim3(n, (int)nchunks), dim3(256), 0, stream, logits,
+                     pval, pidx, V, (int)nchunks);
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(n), dim3(256), 0, stream, pval, pidx, out,
+                     (int)nchunks);
   ZF_CHECK_LAUNCH();
 }
 

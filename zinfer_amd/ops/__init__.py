@@ -156,6 +156,25 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     _check(lib.zf_argmax(_ptr(logits), _ptr(out), _ptr(ws), n, V, _stream()), "argmax")
 
 
+ARGMAX_NO_ALLOC_MAX_PARTIALS = 32768    # ZF_ARGMAX_NO_ALLOC_MAX_PARTIALS in zf_no_alloc.h
+
+
+def argmax_no_alloc(logits: torch.Tensor, out: torch.Tensor) -> None:
+    """``argmax`` for callers that cannot allocate: the partial results live in a fixed device
+    array of the library (shared by all calls on a GPU: overlapping calls race), so at most
+    n * ceil(V / 4096) = 32768 of them."""
+    _need_gpu(logits, out)
+    _i32(out, "out")
+    n, V = logits.shape
+    if logits.dtype != torch.float32 or out.shape != (n,):
+        raise KernelUnavailable("argmax_no_alloc: float32 [n, V] -> int32 [n]")
+    if n * ((V + 4095) // 4096) > ARGMAX_NO_ALLOC_MAX_PARTIALS:
+        raise KernelUnavailable(f"argmax_no_alloc: {n} rows of {V} logits need more than "
+                                f"{ARGMAX_NO_ALLOC_MAX_PARTIALS} partial results")
+    lib = build.load("elementwise")
+    _check(lib.zf_argmax_no_alloc(_ptr(logits), _ptr(out), n, V, _stream()), "argmax_no_alloc")
+
+
 def advance_decode(token_ids: torch.Tensor, positions: torch.Tensor, ctx_len: torch.Tensor,
                    sampled: torch.Tensor, slot_mapping: torch.Tensor, block_table: torch.Tensor,
                    page_size: int, advance: bool) -> None:

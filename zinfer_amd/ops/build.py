@@ -23,7 +23,7 @@ from ..errors import KernelUnavailable
 
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 MODULES = ("elementwise", "gemm", "attention", "sampling")
-HEADERS = ("zf_common.h",)
+HEADERS = ("zf_common.h", "zf_no_alloc.h")
 # -packed-fp32-ops off: hipcc must not form packed 32-bit float instructions by itself
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
