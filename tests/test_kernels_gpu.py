@@ -641,3 +641,44 @@ def test_sample_topk_against_the_host_sampler(V):
         assert got[i] in pos and abs(pos[got[i]] - pos[want]) == 1, \
             f"case {i}: device {got[i]}, host {want}"
     assert exact >= n - 2
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind", ["normal", "gain", "zeros"])
+def test_randinit_is_the_numpy_draw_bit_for_bit(dtype, kind):
+    """The device's counter-based draw and its numpy twin: the same bits for every element,
+    from any starting index (2^20 + 77 elements: every octant of the cosine, both branches of
+    the logarithm's range reduction, mantissas next to the rounding boundary)."""
+    import numpy as np
+    from zinfer_amd.weights import counter_rng
+    key = counter_rng.tensor_key(12345, "model.layers.3.self_attn.o_proj.weight")
+    for start, n in ((0, (1 << 20) + 77), (3_000_000_019, 4099)):
+        got = torch.empty((n,), dtype=dtype, device=DEV)
+        _ops().randinit(got, key, start, kind, 0.02)
+        want = counter_rng.draw(key, start, n, kind, 0.02)
+        if dtype == torch.bfloat16:
+            want_bits = counter_rng.to_bfloat16_bits(want).astype(np.int32)
+            got_bits = got.cpu().view(torch.int16).numpy().astype(np.int32) & 0xFFFF
+        else:
+            want_bits = want.view(np.int32)
+            got_bits = got.cpu().numpy().view(np.int32)
+        assert np.array_equal(got_bits, want_bits), \
+            f"{int((got_bits != want_bits).sum())} of {n} elements differ"
+
+
+def test_random_model_on_the_device_is_the_folder_written_on_the_host(tmp_path):
+    """``random_model`` (drawn tensor by tensor on the GPU) binds the values that
+    ``write_model_dir`` stores from numpy's draw."""
+    import tiny
+    from zinfer_amd.models.build import load_model, random_model
+    from zinfer_amd.weights import write_model_dir
+    path = write_model_dir(str(tmp_path / "m"), tiny.config_of("C"), 9, torch.float32, device=None)
+    _, a = load_model(path, "float32", DEV)
+    _, b = random_model(tiny.config_of("C"), 9, "float32", DEV)
+    assert torch.equal(a.embedding, b.embedding)
+    assert torch.equal(a.head.weight, b.head.weight)
+    for x, y in zip(a.blocks, b.blocks):
+        assert torch.equal(x.mixer.qkv.weight, y.mixer.qkv.weight)
+        assert torch.equal(x.mixer.q_gain, y.mixer.q_gain)
+        assert torch.equal(x.feed_forward.down.weight, y.feed_forward.down.weight)
+        assert torch.equal(x.ff_norm.gain, y.ff_norm.gain)

@@ -143,3 +143,44 @@ def test_random_weights_mode(tmp_path):
     g = ta["model.layers.2.self_attn.k_norm.weight"].float()
     assert float(g.min()) >= 0.9 - 1e-2 and float(g.max()) <= 1.1 + 1e-2 and g.shape == (32,)
     assert json.load(open(tmp_path / "a" / "config.json"))["torch_dtype"] == "bfloat16"
+
+
+def test_counter_based_draws():
+    """An element's value is a function of (seed, tensor name, index): pieces, other tensors
+    and the order of drawing change nothing; the moments are those of the stated distributions."""
+    import numpy as np
+    from zinfer_amd.parts.base import TensorDecl
+    from zinfer_amd.weights import counter_rng, draw_tensor
+    key = counter_rng.tensor_key(7, "model.layers.0.mlp.up_proj.weight")
+    whole = counter_rng.draw(key, 0, 50000, "normal")
+    parts = np.concatenate([counter_rng.draw(key, 0, 1, "normal"),
+                            counter_rng.draw(key, 1, 16383, "normal"),
+                            counter_rng.draw(key, 16384, 33616, "normal")])
+    assert np.array_equal(whole, parts)
+    assert not np.array_equal(
+        whole, counter_rng.draw(counter_rng.tensor_key(7, "model.layers.1.mlp.up_proj.weight"),
+                                0, 50000, "normal"))
+    assert not np.array_equal(
+        whole, counter_rng.draw(counter_rng.tensor_key(8, "model.layers.0.mlp.up_proj.weight"),
+                                0, 50000, "normal"))
+    big = counter_rng.draw(key, 0, 400000, "normal").astype(np.float64)
+    assert abs(big.mean()) < 2e-4 and abs(big.std() - 0.02) < 1e-4
+    assert abs(((big / big.std()) ** 4).mean() - 3.0) < 0.05          # a normal's kurtosis
+    assert abs(np.mean(np.abs(big) > 0.04) - 0.0455) < 0.002          # mass beyond two sigma
+    gain = counter_rng.draw(key, 0, 100000, "gain").astype(np.float64)
+    assert gain.min() >= 0.9 and gain.max() <= 1.1 and abs(gain.mean() - 1.0) < 1e-3
+    assert abs(gain.std() - 0.2 / 12 ** 0.5) < 1e-3
+    # through draw_tensor: bfloat16 is the nearest-even rounding of the float32 draw
+    decl = TensorDecl((30, 41))
+    f = draw_tensor("t", decl, 7, torch.float32)
+    b = draw_tensor("t", decl, 7, torch.bfloat16)
+    assert torch.equal(b, f.to(torch.bfloat16))
+    assert torch.equal(f.flatten(), torch.from_numpy(
+        counter_rng.draw(counter_rng.tensor_key(7, "t"), 0, 30 * 41, "normal")))
+    # the library's logarithm and cosine give the same float32 values
+    k = np.array([counter_rng.mix64((key + (i + 1) * counter_rng.GOLDEN) & counter_rng.MASK)
+                  for i in range(3000)], dtype=np.uint64)
+    k1 = (k >> np.uint64(32)).astype(np.float64)
+    k2 = (k & np.uint64(0xFFFFFFFF)).astype(np.float64)
+    ref = np.sqrt(-2 * np.log((k1 + 1) / 2 ** 32)) * np.cos(2 * np.pi * k2 / 2 ** 32) * 0.02
+    assert np.abs(ref - whole[:3000]).max() < 1e-8

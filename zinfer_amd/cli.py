@@ -662,7 +662,8 @@ def cmd_random_model(args: List[str]) -> int:
         raw = json.load(f)
     cfg = entry_for(raw).config_type.from_dict(raw)
     dtype = torch.bfloat16 if opt.dtype in ("bfloat16", "bf16") else torch.float32
-    write_model_dir(pos[1], cfg, opt.seed, dtype)
+    device = "cuda:0" if torch.cuda.is_available() else None   # the same values either way
+    write_model_dir(pos[1], cfg, opt.seed, dtype, device=device)
     print(f"wrote {pos[1]} (seed {opt.seed}, {opt.dtype})")
     return 0
 

@@ -27,7 +27,7 @@ class Engine:
     """Owns a model, its cache and work buffers; ``step`` is the only way tokens run."""
 
     GRAPH_PAGE_BUCKET = 64      # decode graphs are captured for block tables this many pages wide
-    MAX_GRAPHS = 16
+    MAX_GRAPHS = 256            # the least recently replayed graph goes when there are more
 
     def __init__(self, model: DecoderModel, *, page_size: int = 16, num_pages: int = 256,
                  max_requests: int = 64, kv_dtype: Optional[torch.dtype] = None,
@@ -57,6 +57,10 @@ class Engine:
             and getattr(model, "graph_safe", False)
         self._graphs: Dict[tuple, tuple] = {}
         self.graph_replays = 0
+        # measurement: when a list, every step appends (tokens, sequences, seconds of host
+        # packing, seconds of host launching, event before, event after the step's kernels,
+        # whether a request brought more than one token)
+        self.step_trace: Optional[list] = None
 
     # ------------------------------------------------------------------ requests
     def has_request(self, rid) -> bool:
@@ -87,9 +91,23 @@ class Engine:
                     self.cache.add_request(rid)
                 self.cache.reserve(rid, new_len)
             decode_only = self.use_graphs and all(len(e.tokens) == 1 for e in entries)
+            traced = self.step_trace is not None and self.device.type == "cuda"
+            if traced:
+                import time
+                t0 = time.perf_counter()
             ctx = self._build_context(entries, bucket_pages=decode_only)
+            if traced:
+                t1 = time.perf_counter()
+                before = torch.cuda.Event(enable_timing=True)
+                after = torch.cuda.Event(enable_timing=True)
+                before.record()
             logits = self._forward_graphed(ctx) if decode_only \
                 else self.model.forward(ctx, self.views)
+            if traced:
+                after.record()
+                self.step_trace.append((ctx.n_tokens, ctx.n_seqs, t1 - t0,
+                                        time.perf_counter() - t1, before, after,
+                                        ctx.max_q_len > 1))
             for rid, new_len in wanted_len:
                 self.cache.commit(rid, new_len)
             self.steps_run += 1
@@ -155,7 +173,16 @@ class Engine:
             if not self.cache.has_request(rid):
                 self.cache.add_request(rid)
             self.cache.reserve(rid, new_len)
+        traced = self.step_trace is not None
+        if traced:
+            import time
+            t0 = time.perf_counter()
         ctx = self._build_context(entries, bucket_pages=True, extra_tokens=extra)
+        if traced:
+            t1 = time.perf_counter()
+            before = torch.cuda.Event(enable_timing=True)
+            after = torch.cuda.Event(enable_timing=True)
+            before.record()
         out = self._scratch.get("decoded", (n_steps, n), torch.int32)
         rec = None
         if records is not None:
@@ -172,6 +199,10 @@ class Engine:
                 ops.argmax(logits, out[s])
             else:
                 ops.sample_topk(logits, rec[s], out[s])
+        if traced:
+            after.record()
+            self.step_trace.append((n * n_steps, n, t1 - t0, time.perf_counter() - t1, before,
+                                    after, False))
         tokens = out.tolist()
         for rid, new_len in wanted_len:
             self.cache.commit(rid, new_len)
@@ -185,18 +216,25 @@ class Engine:
     def _forward_graphed(self, ctx: StepContext) -> torch.Tensor:
         """A decode-only step through a captured graph.  The graph holds the addresses of the
         metadata views, work buffers and pools: it is keyed by everything that fixes them
-        (sequences, wanted rows, width of the block tables) and dropped when a buffer moves."""
-        key = (ctx.n_seqs, ctx.n_want, tuple(t.max_pages for t in ctx.kv), ctx.meta_offset)
+        (sequences, wanted rows and whether they are simply all rows, which decides the kernels
+        of the head, width of the block tables) and dropped when a buffer moves."""
+        key = (ctx.n_seqs, ctx.n_want, ctx.wants_all_rows, tuple(t.max_pages for t in ctx.kv),
+               ctx.meta_offset)
         held = self._graphs.get(key)
         if held is not None and held[2] == self._generations():
+            self._graphs[key] = self._graphs.pop(key)      # most recently used last
             held[0].replay()
             self.graph_replays += 1
             return held[1]
         # first time: an eager run settles the sizes of every work buffer (it writes the same
         # keys and values the replay will write again), then capture and replay
         logits = self.model.forward(ctx, self.views)
-        if len(self._graphs) >= self.MAX_GRAPHS:
-            self._graphs.clear()
+        if held is not None or any(g[2] != self._generations() for g in self._graphs.values()):
+            # a work buffer has moved: every graph that holds its old address is dead
+            self._graphs = {k: g for k, g in self._graphs.items()
+                            if g[2] == self._generations() and k != key}
+        while len(self._graphs) >= self.MAX_GRAPHS:
+            self._graphs.pop(next(iter(self._graphs)))
         torch.cuda.current_stream(self.device).synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):

@@ -51,13 +51,15 @@ def load_model(model_dir: str, dtype="bfloat16", device="cuda:0"):
     return config, model
 
 
-def random_model(config, seed: int, dtype="bfloat16", device="cuda:0"):
+def random_model(config, seed: int, dtype="bfloat16", device="cuda:0", store_dtype=None):
     """(typed configuration, bound model) with weights drawn from ``seed``: the values that
-    ``write_model_dir(config, seed, dtype)`` stores, without the file.  ``config``: a typed
-    configuration, a dict of config.json keys, or the path of a config.json."""
+    ``write_model_dir(config, seed, store_dtype)`` stores, without the file, drawn on the
+    device one tensor at a time.  ``config``: a typed configuration, a dict of config.json
+    keys, or the path of a config.json.  ``store_dtype``: what the drawn values are rounded to
+    before the model takes them (default: the compute dtype)."""
     import json
     from ..config import entry_for
-    from ..weights.random_init import draw_tensors
+    from ..weights.random_init import DrawnTensors
     if isinstance(config, str):
         with open(config, "r", encoding="utf-8") as f:
             config = json.load(f)
@@ -66,7 +68,7 @@ def random_model(config, seed: int, dtype="bfloat16", device="cuda:0"):
     spec = config.model_spec()
     ctx = BuildContext(parse_dtype(dtype), torch.device(device))
     model = DecoderModel(spec, ctx)
-    tensors = draw_tensors(model.declare(), seed, ctx.compute_dtype,
-                           tied=spec.tie_word_embeddings, head_name=spec.head_name)
-    model.bind(tensors)
+    store = parse_dtype(store_dtype) if store_dtype is not None else ctx.compute_dtype
+    model.bind(DrawnTensors(model.declare(), seed, store, ctx.device,
+                            tied=spec.tie_word_embeddings, head_name=spec.head_name))
     return config, model

@@ -199,6 +199,19 @@ def advance_decode(token_ids: torch.Tensor, positions: torch.Tensor, ctx_len: to
            "advance_decode")
 
 
+def randinit(out: torch.Tensor, key: int, start: int, kind: str, std: float = 0.02) -> None:
+    """out[i] = element ``start + i`` of the random tensor with ``key``
+    (`weights/counter_rng.py`: 'normal' = N(0, std), 'gain' = 1 + U(-0.1, 0.1), 'zeros')."""
+    from ..weights.counter_rng import KIND
+    _need_gpu(out)
+    if out.dim() != 1 or kind not in KIND:
+        raise KernelUnavailable(f"randinit: a flat tensor and a kind of {sorted(KIND)}")
+    lib = build.load("randinit")
+    _check(lib.zf_randinit(_ptr(out), _dt(out), ctypes.c_ulonglong(key & ((1 << 64) - 1)),
+                           ctypes.c_ulonglong(start), ctypes.c_ulonglong(out.numel()),
+                           KIND[kind], ctypes.c_double(std), _stream()), "randinit")
+
+
 # ------------------------------------------------------------------------- work buffers
 _workspaces = {}
 _workspace_generation = 0

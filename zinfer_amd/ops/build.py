@@ -22,7 +22,7 @@ from typing import Dict, Iterable, List, Optional
 from ..errors import KernelUnavailable
 
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
-MODULES = ("elementwise", "gemm", "attention", "sampling")
+MODULES = ("elementwise", "gemm", "attention", "sampling", "randinit")
 HEADERS = ("zf_common.h", "zf_no_alloc.h")
 # -packed-fp32-ops off: hipcc must not form packed 32-bit float instructions by itself
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
