@@ -11,8 +11,17 @@ import torch
 F64 = torch.float64
 
 
-def embed(table, ids, out):
-    out.copy_(table[ids.long()].to(out.dtype))
+def embed(table, ids, out, scale=1.0):
+    out.copy_((table[ids.long()].to(F64) * float(torch.tensor(scale, dtype=torch.float32)))
+              .to(out.dtype))
+
+
+def scale_cap(x, scale=1.0, cap=0.0):
+    v = x.to(F64) * float(torch.tensor(scale, dtype=torch.float32))
+    if cap > 0:
+        c = float(torch.tensor(cap, dtype=torch.float32))
+        v = c * torch.tanh(v / c)
+    x.copy_(v.to(x.dtype))
 
 
 def rmsnorm(x, gain, eps, out):
@@ -128,7 +137,7 @@ def argmax(logits, out):
 
 
 ALL = ("embed", "rmsnorm", "gemm", "can_pretile", "can_fuse_swiglu", "gemm_swiglu", "qk_norm_rope_kv_write", "paged_attention", "swiglu",
-       "gather_rows", "argmax")
+       "gather_rows", "argmax", "scale_cap")
 
 
 def install(monkeypatch):

@@ -210,6 +210,59 @@ def test_step_errors_leave_cache_untouched(tmp_path_factory):
         eng.step([StepEntry("x", [1] * 5, [])])
     assert eng.length("x") == 60
     eng.cache.check()
+    # a failure inside the run (a kernel that refuses, a launch that fails): the step's new
+    # request goes again, the pages it reserved for the others go back
+    from zinfer_amd import KernelUnavailable
+    eng.release("x")
+    eng.step([StepEntry("y", [1] * 20, [])])
+    free = eng.cache.num_free_pages()
+    forward = eng.model.forward
+
+    def failing(ctx, views):
+        raise KernelUnavailable("a kernel refused")
+    eng.model.forward = failing
+    with pytest.raises(KernelUnavailable):
+        eng.step([StepEntry("y", [1] * 20, []), StepEntry("z", [2] * 9, [8])])
+    assert eng.length("y") == 20 and not eng.has_request("z")
+    assert eng.cache.num_free_pages() == free
+    eng.cache.check()
+    eng.model.forward = forward
+    assert eng.step([StepEntry("y", [1] * 20, [19]), StepEntry("z", [2] * 9, [8])]).shape[0] == 2
+    assert eng.length("y") == 40 and eng.length("z") == 9
+    eng.cache.check()
+
+
+def test_a_cache_of_another_dtype_is_refused(tmp_path_factory):
+    from zinfer_amd.engine import Engine
+    from zinfer_amd.errors import ConfigError
+    from zinfer_amd.models.build import load_model
+    path = tiny.model_dir_of("A", str(tmp_path_factory.getbasetemp()), torch.float32)
+    _, model = load_model(path, "float32", DEVICE[0])
+    with pytest.raises(ConfigError, match="compute dtype"):
+        Engine(model, page_size=16, num_pages=4, kv_dtype=torch.bfloat16)
+    Engine(model, page_size=16, num_pages=4, kv_dtype=torch.float32)
+
+
+def test_repeated_wants_beside_none_after_an_all_rows_graph(tmp_path_factory):
+    """Two decode-only steps with the same numbers of sequences and wanted rows, one wanting
+    every row once, one wanting the first row twice and the second not at all: the second
+    must not replay the first's graph, whose head reads all rows as they lie."""
+    from zinfer_amd.engine import StepEntry
+    from zinfer_amd.engine.replay import make_engine
+    path = tiny.model_dir_of("D", str(tmp_path_factory.getbasetemp()), torch.bfloat16)
+    V = tiny.CONFIGS["D"]["vocab_size"]
+    a = make_engine(path, "bfloat16", 256, DEVICE[0])
+    b = make_engine(path, "bfloat16", 256, DEVICE[0])
+    b.use_graphs = False
+    p, q = tiny.random_tokens(12, V, 71), tiny.random_tokens(9, V, 72)
+    for eng in (a, b):
+        eng.step([StepEntry("p", p[:8], []), StepEntry("q", q[:5], [])])
+    for k, (wp, wq) in enumerate((([0], [0]), ([0, 0], []), ([0], [0]), ([], [0, 0]))):
+        entries = [StepEntry("p", p[8 + k:9 + k], wp), StepEntry("q", q[5 + k:6 + k], wq)]
+        la, lb = a.step(entries), b.step(entries)
+        assert torch.equal(la, lb), f"step {k}: wants {wp} {wq}"
+        if len(wp) == 2 or len(wq) == 2:
+            assert torch.equal(la[0], la[1])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -34,6 +34,10 @@ def test_step_errors_host_logic(tmp_path_factory):
     G.test_step_errors_leave_cache_untouched(tmp_path_factory)
 
 
+def test_cache_dtype_host_logic(tmp_path_factory):
+    G.test_a_cache_of_another_dtype_is_refused(tmp_path_factory)
+
+
 def test_bfloat16_storage_host_logic(tmp_path_factory):
     """bfloat16 weights and cache through the same host code."""
     path, cfg, requests, ref = G._setup("B", "bfloat16", tmp_path_factory)

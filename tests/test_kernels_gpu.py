@@ -682,3 +682,115 @@ def test_random_model_on_the_device_is_the_folder_written_on_the_host(tmp_path):
         assert torch.equal(x.mixer.q_gain, y.mixer.q_gain)
         assert torch.equal(x.feed_forward.down.weight, y.feed_forward.down.weight)
         assert torch.equal(x.ff_norm.gain, y.ff_norm.gain)
+
+
+def test_embed_multiplier_and_logit_scale_cap():
+    table = _rand((50, 96), torch.bfloat16, 1)
+    ids = torch.tensor([3, 49, 0], dtype=torch.int32)
+    want = torch.empty((3, 96))
+    ref.embed(table, ids, want, 2.5)
+    got = torch.empty((3, 96), device=DEV)
+    _ops().embed(table.to(DEV), ids.to(DEV), got, 2.5)
+    assert torch.equal(got.cpu(), want)
+    x = _rand((5, 1003), torch.float32, 2, 4.0)
+    for scale, cap in ((0.25, 0.0), (1.0, 3.0), (30.0, 2.5)):
+        want = x.clone()
+        ref.scale_cap(want, scale, cap)
+        got = x.to(DEV)
+        _ops().scale_cap(got, scale, cap)
+        assert rel_err(got, want) <= 1e-6
+
+
+def test_device_sampler_order_vectors():
+    """The device's penalties and sampler on the cases in which the order of the reference's
+    operations decides the token."""
+    import numpy as np
+    import sampler_vectors as sv
+    import zinfer_amd.ops as ops
+    for logits, history, params, us, want, why in sv.ORDER_CASES:
+        V = 64                               # the cases' logits first, the rest far below
+        for u in us:
+            row = np.full((1, V), -1e4, np.float32)
+            row[0, :len(logits)] = logits
+            lg = torch.from_numpy(row).to(DEV)
+            counts = {}
+            for t in history:
+                counts[t] = counts.get(t, 0) + 1
+            if counts:
+                t32 = lambda a: torch.tensor(a, dtype=torch.int32, device=DEV)
+                pen = torch.tensor([[params.get("repetition_penalty", 1.0),
+                                     params.get("presence_penalty", 0.0),
+                                     params.get("frequency_penalty", 0.0)]], device=DEV)
+                ops.apply_penalties(lg, t32([0] * len(counts)), t32(list(counts)),
+                                    t32(list(counts.values())), pen)
+            rec = np.zeros((1,), dtype=ops.SAMPLE_ROW_DTYPE)
+            greedy = params["temperature"] <= 0.0
+            rec[0] = (1.0, 1.0, 0.0, 1, 0.0) if greedy else \
+                (params["temperature"], params.get("top_p", 1.0), params.get("min_p", 0.0),
+                 params["top_k"], u)
+            out = torch.empty((1,), dtype=torch.int32, device=DEV)
+            ops.sample_topk(lg, torch.from_numpy(rec.view(np.uint8).reshape(-1).copy()).to(DEV), out)
+            assert int(out[0]) == want, f"{why}: u = {u}: token {int(out[0])}, not {want}"
+
+
+def _stand_out(s, nKV, ps, hd, seq, position, query_row, q_head, dtype, nH):
+    """Makes the key at ``position`` of sequence ``seq`` take all the weight of query row
+    ``query_row``, head ``q_head``: aligned with that query and scaled up."""
+    G = nH // nKV
+    q = s["q"].view(-1, nH, hd).float()
+    kp = s["k_pool"].view(-1, nKV, ps, hd)
+    page = int(s["block_table"][seq, position // ps])
+    direction = q[query_row, q_head] / q[query_row, q_head].norm()
+    kp[page, q_head // G, position % ps] = (direction * 400.0).to(dtype)
+
+
+@pytest.mark.parametrize("hd", [64, 128])
+def test_mfma_decode_window_edge_and_far_key(hd):
+    """The MFMA decode kernel (bfloat16, pages of 16) with a key that stands out: just outside
+    the window it must have no influence, just inside it takes all the weight; the window's
+    first key is put at a page's edge, across a 64-key wave chunk and across a 256-key split."""
+    dtype, nH, nKV, ps = torch.bfloat16, 8, 2, 16
+    assert _ops().mfma_attention_covers(dtype, nH, nKV, hd, ps)
+    for ctx, window in ((700, 0), (700, 188), (700, 189), (700, 445), (1030, 262), (1030, 7),
+                        (300, 300), (300, 299), (513, 257)):
+        pos = ctx - 1
+        targets = [(0, True), (ctx - 1, True), (255, True), (256, True)] if window == 0 else \
+            [(pos - window, False), (pos - window + 1, True)]
+        for target, inside in targets:
+            if target < 0:
+                continue
+            s = _paged_setup(dtype, nH, nKV, hd, ps, [ctx, 40], [1, 1], seed=21)
+            _stand_out(s, nKV, ps, hd, 0, target, 0, 5, dtype, nH)
+            got, want = _run_attention(s, dtype, nH, nKV, hd, ps, window, [1, 1], [ctx, 40])
+            v_row = s["Vs"][0][target, 5 // (nH // nKV)].float()
+            close = torch.allclose(got.cpu().float()[0, 5 * hd:6 * hd], v_row, atol=3e-2)
+            assert close == inside, f"ctx {ctx}, window {window}, key {target}"
+            assert rel_err(got, want) <= 2 * tol(dtype), f"ctx {ctx}, window {window}, key {target}"
+
+
+@pytest.mark.parametrize("hd", [64, 128])
+def test_mfma_prefill_window_edge_and_far_key(hd):
+    """The MFMA prefill kernel on a portion that starts mid-context: for the first and the last
+    query of a 32-query tile, a key that stands out at p - window (no influence) and at
+    p - window + 1 (all the weight); windows whose first key falls on and beside the edges of a
+    32-key tile; without a window, a far key at the very start and at a tile's edge."""
+    dtype, nH, nKV, ps = torch.bfloat16, 4, 2, 16
+    ctx, q_len = 420, 100                       # the portion is positions 320 .. 419
+    start = ctx - q_len
+    for window in (0, 33, 64, 65, 97, 200, 330):
+        for row in (0, 31, 32, 63, 99):         # rows of the portion: tile edges and the last
+            p = start + row
+            cases = [(0, True), (31, True), (32, True), (p, True)] if window == 0 else \
+                [(p - window, False), (p - window + 1, True)]
+            for target, inside in cases:
+                if target < 0:
+                    continue
+                s = _paged_setup(dtype, nH, nKV, hd, ps, [ctx, 70], [q_len, 70], seed=23)
+                _stand_out(s, nKV, ps, hd, 0, target, row, 3, dtype, nH)
+                got, want = _run_attention(s, dtype, nH, nKV, hd, ps, window, [q_len, 70],
+                                           [ctx, 70])
+                v_row = s["Vs"][0][target, 3 // (nH // nKV)].float()
+                close = torch.allclose(got.cpu().float()[row, 3 * hd:4 * hd], v_row, atol=3e-2)
+                assert close == inside, f"window {window}, query {p}, key {target}"
+                assert rel_err(got, want) <= 2 * tol(dtype), \
+                    f"window {window}, query {p}, key {target}"

@@ -314,9 +314,32 @@ class ToyConfig:
             layers = (blk(full), blk(win))
             schedule = (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0),
                         ScheduleEntry(1, cache_of=1))
+        # the "state" kind also scales its embedding rows and scales and caps its logits
+        extra = dict(embedding_multiplier=3.0, logit_scale=40.0, logit_softcap=2.5) \
+            if self.kind == "state" else {}
         return ModelSpec(vocab_size=self.vocab_size, hidden_size=H, max_positions=512,
                          layers=layers, schedule=schedule, final_norm=norm,
-                         tie_word_embeddings=True)
+                         tie_word_embeddings=True, **extra)
+
+
+class ToyTokenizer:
+    """One id per byte; the text front end of the toy architecture."""
+
+    def encode(self, text):
+        return list(text.encode("utf-8"))
+
+    def decode(self, ids):
+        return bytes(int(i) % 256 for i in ids).decode("latin-1")
+
+
+def _toy_text_hooks():
+    from zinfer_amd.config import TextHooks
+    return TextHooks(
+        load_tokenizer=lambda model_dir: ToyTokenizer(),
+        render_messages=lambda messages, thinking: "".join(f"[{m.role}:{m.content}]" for m in messages),
+        render_single_user=lambda text, thinking, system=None:
+            (f"[system:{system}]" if system else "") + f"[user:{text}]" + ("?" if thinking else "!"),
+        assistant_history_content=lambda content: content)
 
 
 def _toy_plain(cfg: ToyConfig, w, toks):
@@ -327,7 +350,7 @@ def _toy_plain(cfg: ToyConfig, w, toks):
     states = [torch.zeros(cfg.state_size, dtype=F64) for _ in spec.schedule]
     rows = []
     for p, tok in enumerate(toks):
-        x = w["model.embed_tokens.weight"][tok].to(F64)
+        x = w["model.embed_tokens.weight"][tok].to(F64) * spec.embedding_multiplier
         for pos, e in enumerate(spec.schedule):
             pre = f"model.layers.{e.layer}."
             blk = spec.layers[e.layer]
@@ -354,9 +377,36 @@ def _toy_plain(cfg: ToyConfig, w, toks):
             x = x + plain.linear(plain.swiglu(plain.linear(mm, w[pre + "mlp.gate_proj.weight"]),
                                               plain.linear(mm, w[pre + "mlp.up_proj.weight"])),
                                  w[pre + "mlp.down_proj.weight"])
-        rows.append(plain.linear(plain.rms_norm(x, w["model.norm.weight"], 1e-5),
-                                 w["model.embed_tokens.weight"]))
+        logits = plain.linear(plain.rms_norm(x, w["model.norm.weight"], 1e-5),
+                              w["model.embed_tokens.weight"]) * spec.logit_scale
+        if spec.logit_softcap is not None:
+            logits = spec.logit_softcap * torch.tanh(logits / spec.logit_softcap)
+        rows.append(logits)
     return torch.stack(rows).numpy()
+
+
+def _toy_text_through_the_command_line(path, cfg):
+    """Text in and out with the toy architecture's own tokenizer and template, which the
+    command line takes from the registry entry of the folder's config.json."""
+    import contextlib
+    import io
+    from zinfer_amd import cli
+    from zinfer_amd.entrypoints import LLM, SamplingParams
+    prompt = "[system:be brief][user:hi]!"
+    ids = list(prompt.encode())
+    llm = LLM(path, dtype="float32", device=DEV, page_size=16, max_tokens=128)
+    want = llm.generate([ids], SamplingParams(temperature=0.0, max_new_tokens=5, ignore_eos=True))[0]
+    out = io.StringIO()
+    with contextlib.redirect_stdout(out):
+        rc = cli.main(["generate", path, "hi", "5", "no-think", "--system", "be brief",
+                       "--dtype", "float32", "--temperature", "0", "--repetition-penalty", "1",
+                       "--ignore-eos"])
+    assert rc == 0, out.getvalue()
+    assert "response: " + ToyTokenizer().decode(want) in out.getvalue()
+    out = io.StringIO()
+    with contextlib.redirect_stdout(out):
+        assert cli.main(["tokenize", path, "hi"]) == 0
+    assert "ids: [104, 105]" in out.getvalue()
 
 
 @pytest.mark.parametrize("kind", ["state", "mixed"])
@@ -370,11 +420,13 @@ def test_toy_architecture_registered_built_and_stepped(kind, tmp_path):
     from zinfer_amd.parts import unregister_part
     from zinfer_amd.weights import SafetensorsFile, write_model_dir
     _register_toy_state()
-    register_architecture("ToyForCausalLM", ToyConfig, model_type="toy")
+    register_architecture("ToyForCausalLM", ToyConfig, model_type="toy", text=_toy_text_hooks())
     try:
         cfg = ToyConfig(hidden_size=64, state_size=24, decay=0.9, window=19, vocab_size=300,
                         kind=kind)
         path = write_model_dir(str(tmp_path / "toy"), cfg, seed=5, dtype=torch.float32)
+        if kind == "state":
+            _toy_text_through_the_command_line(path, cfg)
         with SafetensorsFile(os.path.join(path, "model.safetensors")) as f:
             w = {n: f.tensor(n) for n in f.names()}
         requests = {f"q{i}": tiny.random_tokens(n, 300, 70 + i) for i, n in enumerate((50, 7, 90, 33))}

@@ -235,3 +235,57 @@ def test_rng_is_xoshiro256pp():
     r = plain.PlainRng(0)
     r.s = [1, 2, 3, 4]
     assert [r.next() for _ in range(3)] == [41943041, 58720359, 3588806011781223]
+
+
+def test_sampler_order_vectors():
+    """Where the order of the sampler's operations decides the token."""
+    import sampler_vectors as sv
+    for logits, history, params, us, want, why in sv.ORDER_CASES:
+        for u in us:
+            got = plain.sample_token(np.array(logits, np.float32), history, params, sv.FixedU(u))
+            assert got == want, f"{why}: u = {u}: token {got}, not {want}"
+
+
+def test_qk_norm_sits_before_the_rotation():
+    """Scores may depend on the distance between query and key only, so a block's output does
+    not change when all positions move by the same amount.  With per-head gains that differ
+    inside a rotated pair (i, i + hd/2), that holds only if the norm comes before the rotation
+    (`layer.zig:114-128`): a gain applied after it does not commute with the rotation."""
+    cfg, w = tiny.CONFIGS["B"], dict(tiny.weights_of("B"))
+    hd, nH, nKV, theta = cfg["head_dim"], cfg["num_attention_heads"], cfg["num_key_value_heads"], \
+        cfg["rope_theta"]
+    g = torch.Generator().manual_seed(9)
+    for l in range(cfg["num_hidden_layers"]):
+        for n in ("q_norm", "k_norm"):        # gains far from 1 and unequal inside every pair
+            w[plain.layer_name(l, f"self_attn.{n}.weight")] = 0.5 + 2.0 * torch.rand(hd, generator=g)
+    xs = torch.randn(6, cfg["hidden_size"], generator=g, dtype=torch.float32).to(F64)
+
+    def run(shift):
+        keys, values, out = [], [], []
+        # the cache is pre-filled with `shift` unreadable entries through a window, so the
+        # token at list index `shift + t` has position `shift + t` and sees only tokens >= shift
+        for _ in range(shift):
+            keys.append(torch.zeros(nKV, hd, dtype=F64)); values.append(torch.zeros(nKV, hd, dtype=F64))
+        for t in range(xs.shape[0]):
+            out.append(plain.block_token(cfg, w, 0, xs[t], shift + t, keys, values, window=t + 1))
+        return torch.stack(out)
+    base = run(0)
+    for shift in (1, 13, 200):
+        assert (run(shift) - base).abs().max() < 2e-4 * base.abs().max()
+    # the invariant notices the other order: gains applied after the rotation
+    q = torch.randn(hd, generator=g).to(F64); k = torch.randn(hd, generator=g).to(F64)
+    gq = w[plain.layer_name(0, "self_attn.q_norm.weight")].to(F64)
+    gk = w[plain.layer_name(0, "self_attn.k_norm.weight")].to(F64)
+    one = torch.ones(hd, dtype=F64)
+
+    def wrong(pq, pk):
+        a = plain.rope_head(plain.rms_norm(q, one, 1e-6), pq, theta) * gq
+        b = plain.rope_head(plain.rms_norm(k, one, 1e-6), pk, theta) * gk
+        return float((a * b).sum())
+
+    def right(pq, pk):
+        a = plain.rope_head(plain.rms_norm(q, gq, 1e-6), pq, theta)
+        b = plain.rope_head(plain.rms_norm(k, gk, 1e-6), pk, theta)
+        return float((a * b).sum())
+    assert abs(right(5, 2) - right(18, 15)) < 1e-4
+    assert abs(wrong(5, 2) - wrong(18, 15)) > 1e-2

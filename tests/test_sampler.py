@@ -63,3 +63,14 @@ def test_command_line_presets():
     a, b = thinking_defaults(False), thinking_defaults(True)
     assert (a.temperature, a.top_k, a.top_p, a.repetition_penalty) == (0.7, 20, 0.8, 1.1)
     assert (b.temperature, b.top_k, b.top_p, b.repetition_penalty) == (0.6, 20, 0.95, 1.1)
+
+
+def test_order_vectors():
+    """Where the order of the sampler's operations decides the token: the same cases that pin
+    the plain sampler."""
+    import sampler_vectors as sv
+    for logits, history, params, us, want, why in sv.ORDER_CASES:
+        for u in us:
+            got = sample_token(np.array(logits, np.float32), history, SamplingParams(**params),
+                               sv.FixedU(u))
+            assert got == want, f"{why}: u = {u}: token {got}, not {want}"

@@ -5,7 +5,6 @@ import numpy as np
 import pytest
 import torch
 
-from zinfer_amd import CacheFull
 from zinfer_amd.cache import CacheManager
 from zinfer_amd.engine.scheduler import Scheduler
 from zinfer_amd.parts import KVNeed
@@ -135,17 +134,64 @@ def test_out_of_pages_preempts_the_newest_and_recomputes():
     assert eng.cache.num_free_pages() == [4]
 
 
-def test_a_request_that_cannot_fit_alone_raises_cache_full():
+def test_a_request_that_cannot_fit_alone():
+    """A prompt larger than the whole pool is rejected when it is added; a request that is
+    alone and outgrows the pool while decoding ends with what it has."""
     eng = FakeEngine(num_pages=2, page_size=4)
     s = Scheduler(eng, max_step_tokens=64)
-    s.add_request(list(range(1, 12)), SamplingParams(max_new_tokens=2, **GREEDY))
-    with pytest.raises(CacheFull):
-        s.run()
+    rid = s.add_request(list(range(1, 12)), SamplingParams(max_new_tokens=2, **GREEDY))
+    out = s.run()
+    assert out[rid].finish_reason == "rejected" and "CacheFull" in out[rid].error
+    assert out[rid].generated == [] and eng.log == []
     eng2 = FakeEngine(num_pages=2, page_size=4)
     s2 = Scheduler(eng2, max_step_tokens=64)
-    s2.add_request([1, 2, 3, 4, 5, 6, 7], SamplingParams(max_new_tokens=5, **GREEDY))
-    with pytest.raises(CacheFull):
-        s2.run()                                    # grows beyond the pool while decoding
+    rid = s2.add_request([1, 2, 3, 4, 5, 6, 7], SamplingParams(max_new_tokens=5, **GREEDY))
+    out = s2.run()                                   # grows beyond the pool while decoding
+    assert out[rid].finish_reason == "cache" and out[rid].generated == [8, 9]
+    assert eng2.cache.num_free_pages() == [2] and not eng2.cache.requests
+    eng2.cache.check()
+
+
+def test_a_bad_request_among_good_ones_is_rejected_alone():
+    """A token id beyond the vocabulary, a prompt beyond the position table, an empty prompt:
+    each finishes as "rejected" when it is added, is handed back by the next step, and the
+    requests around it run as if it had never come."""
+    eng = FakeEngine(num_pages=64)
+    eng.model.spec.max_positions = 40
+    s = Scheduler(eng, max_step_tokens=16, chunk_size=8)
+    good1 = s.add_request([3, 4, 5], SamplingParams(max_new_tokens=3, **GREEDY))
+    bad_token = s.add_request([3, V, 5], SamplingParams(max_new_tokens=3, **GREEDY))
+    negative = s.add_request([3, -1], SamplingParams(max_new_tokens=3, **GREEDY))
+    too_long = s.add_request(list(range(1, 42)), SamplingParams(max_new_tokens=3, **GREEDY))
+    empty = s.add_request([], SamplingParams(max_new_tokens=3, **GREEDY))
+    good2 = s.add_request([20, 21], SamplingParams(max_new_tokens=2, **GREEDY))
+    first = s.step()
+    assert {r.id for r in first} >= {bad_token, negative, too_long, empty}
+    out = s.run()
+    assert out[good1].generated == [6, 7, 8] and out[good2].generated == [22, 23]
+    for rid, needle in ((bad_token, "TokenIdOutOfBounds"), (negative, "TokenIdOutOfBounds"),
+                        (too_long, "PositionOutOfBounds"), (empty, "EmptyPrompt")):
+        assert out[rid].finish_reason == "rejected" and needle in out[rid].error
+        assert out[rid].generated == []
+    seen = {rid for st in eng.log for rid, _, _ in st}
+    assert seen == {good1, good2}
+    assert eng.cache.num_free_pages() == [64] and not eng.cache.requests
+
+
+def test_a_request_id_in_use_is_refused():
+    from zinfer_amd.errors import StepError
+    eng = FakeEngine(num_pages=16)
+    s = Scheduler(eng, max_step_tokens=16)
+    s.add_request([1, 2], SamplingParams(max_new_tokens=2, **GREEDY), request_id="x")
+    with pytest.raises(StepError, match="already in use"):
+        s.add_request([3], request_id="x")                   # waiting
+    s.step()
+    with pytest.raises(StepError, match="already in use"):
+        s.add_request([3], request_id="x")                   # running
+    s.run()
+    with pytest.raises(StepError, match="already in use"):
+        s.add_request([3], request_id="x")                   # finished
+    assert s.finished["x"].generated == [3, 4]
 
 
 def test_sampled_output_does_not_depend_on_the_batch():

@@ -133,7 +133,11 @@ def test_stop_analysis_vectors():
 
 def test_tokenize_and_decode_ids_commands(tmp_path, capsys):
     """src/app/cli/tools/text.zig:5-75: the printed form."""
+    import json
+    import tiny
     text_fixture.write_tokenizer_json(str(tmp_path))
+    # the tokenizer is the one of the architecture that config.json names (text.zig:10-20)
+    (tmp_path / "config.json").write_text(json.dumps(tiny.TINY_A))
     vocab, _, specials = text_fixture.build()
     assert cli.main(["tokenize", str(tmp_path), "Hello<|im_end|>"]) == 0
     out = capsys.readouterr().out
@@ -141,4 +145,8 @@ def test_tokenize_and_decode_ids_commands(tmp_path, capsys):
     assert cli.main(["decode-ids", str(tmp_path), f"{vocab['Hi']},{vocab[chr(0x120) + 'world']}"]) == 0
     assert capsys.readouterr().out.endswith("text: Hi world\n")
     assert cli.main(["tokenize", str(tmp_path / "nothing"), "x"]) == 1
+    assert "no config.json" in capsys.readouterr().err
+    (tmp_path / "bare").mkdir()
+    (tmp_path / "bare" / "config.json").write_text(json.dumps(tiny.TINY_A))
+    assert cli.main(["tokenize", str(tmp_path / "bare"), "x"]) == 1
     assert "TokenizerNotFound" in capsys.readouterr().err

@@ -184,3 +184,58 @@ def test_counter_based_draws():
     k2 = (k & np.uint64(0xFFFFFFFF)).astype(np.float64)
     ref = np.sqrt(-2 * np.log((k1 + 1) / 2 ** 32)) * np.cos(2 * np.pi * k2 / 2 ** 32) * 0.02
     assert np.abs(ref - whole[:3000]).max() < 1e-8
+
+
+def _write_sharded(path, cfg_raw, tensors, n_shards=2):
+    """A model folder whose tensors lie in several files named by model.safetensors.index.json."""
+    import os
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg_raw, f)
+    names = list(tensors)
+    weight_map = {}
+    for s in range(n_shards):
+        part = names[s::n_shards]               # interleaved: a layer's tensors are split up
+        fname = f"model-{s + 1:05d}-of-{n_shards:05d}.safetensors"
+        write_safetensors(os.path.join(path, fname), {n: tensors[n] for n in part})
+        weight_map.update({n: fname for n in part})
+    with open(os.path.join(path, "model.safetensors.index.json"), "w") as f:
+        json.dump({"metadata": {}, "weight_map": weight_map}, f)
+    return path
+
+
+def test_sharded_folder_loads_the_same_tensors(tmp_path):
+    cfg = tiny.config_of("B")
+    decls = declare_tensors(cfg.model_spec())
+    tensors = draw_tensors(decls, 4, torch.bfloat16)
+    single = write_model_dir(str(tmp_path / "one"), cfg, 4, torch.bfloat16)
+    sharded = _write_sharded(str(tmp_path / "three"), tiny.TINY_B, tensors, 3)
+    a, b = load_tensors(single, decls), load_tensors(sharded, decls)
+    assert set(a) == set(b) == set(decls)
+    assert all(torch.equal(a[k], b[k]) for k in a)
+    # what is wrong is still reported in one error, whichever file it lies in
+    bad = dict(tensors)
+    del bad["model.layers.2.mlp.up_proj.weight"]
+    bad["extra.weight"] = torch.ones(2)
+    with pytest.raises(WeightError) as e:
+        load_tensors(_write_sharded(str(tmp_path / "bad"), tiny.TINY_B, bad, 2), decls)
+    assert "model.layers.2.mlp.up_proj.weight" in str(e.value) and "extra.weight" in str(e.value)
+
+
+def test_float16_weights_widen_exactly(tmp_path):
+    """A float16 tensor becomes float32 (exact), never bfloat16 (3 bits of mantissa fewer):
+    under a 32-bit build the model computes with the stored values."""
+    cfg = tiny.config_of("A")
+    decls = declare_tensors(cfg.model_spec())
+    tensors = {k: v.to(torch.float16) for k, v in draw_tensors(decls, 2, torch.float32, tied=True).items()}
+    (tmp_path / "config.json").write_text(json.dumps(tiny.TINY_A))
+    write_safetensors(str(tmp_path / "model.safetensors"), tensors)
+    got = load_tensors(str(tmp_path), decls)
+    for k, v in tensors.items():
+        assert got[k].dtype == torch.float32 and torch.equal(got[k], v.float()), k
+    assert not torch.equal(tensors["model.embed_tokens.weight"].float(),
+                           tensors["model.embed_tokens.weight"].to(torch.bfloat16).float())
+    model = build_model(cfg.model_spec(), got, "float32", "cpu")
+    assert torch.equal(model.embedding, tensors["model.embed_tokens.weight"].float())
+    assert torch.equal(model.blocks[0].ff_norm.gain,
+                       tensors["model.layers.0.post_attention_layernorm.weight"].float())

@@ -187,6 +187,31 @@ class CacheManager:
             for i in gone:
                 table[i] = NO_PAGE
 
+    def trim(self, rid) -> None:
+        """Gives back the pages reserved beyond the tokens the request holds (a step that
+        reserved them did not run)."""
+        req = self.requests[rid]
+        keep = (req["length"] + self.page_size - 1) // self.page_size
+        for grp in self.groups:
+            table = grp.tables[rid]
+            self._give_back(grp, [p for p in table[keep:] if p != NO_PAGE])
+            del table[keep:]
+
+    def pages_at_most(self, n_tokens: int, portion: int) -> List[int]:
+        """Upper bound, per group, of the pages a request of ``n_tokens`` tokens holds at any
+        one time when it runs in portions of at most ``portion`` tokens: a group with a window
+        keeps only the window and the portion being written."""
+        out = []
+        for grp in self.groups:
+            n = n_tokens
+            if grp.need.window is not None:
+                n = min(n, grp.need.window + portion + self.page_size)
+            out.append((n + self.page_size - 1) // self.page_size)
+        return out
+
+    def num_pages(self) -> List[int]:
+        return [g.pages.num_pages for g in self.groups]
+
     def release(self, rid) -> None:
         """Everything the request holds goes back: pages of every group and the state slot."""
         req = self.requests.pop(rid, None)

@@ -240,6 +240,17 @@ def _llm(model_dir: str, opt: Options, max_tokens: Optional[int] = None):
                multi_step=opt.multi_step)
 
 
+def _text_hooks(model_dir: str):
+    """The tokenizer and templates of the architecture that ``model_dir``'s config.json names
+    (`src/model/runtime/decoder_registry.zig:16-19`): the command line knows no family's."""
+    from .config import entry_for, read_config_json
+    entry = entry_for(read_config_json(model_dir))
+    if entry.text is None:
+        raise CliError(f"NoTextFrontEnd: the architecture {entry.name} brings no tokenizer and "
+                       "no prompt template; give token ids")
+    return entry.text
+
+
 # ------------------------------------------------------------------------- commands
 def cmd_inspect_config(args: List[str]) -> int:
     """`src/app/cli/inspect.zig:8-34`."""
@@ -250,22 +261,33 @@ def cmd_inspect_config(args: List[str]) -> int:
     print(f"model_dir: {model_dir}")
     print(f"model_type: {cfg.model_type}")
     print(f"architecture: {entry_for(read_config_json(model_dir)).name}")
-    for key in ("hidden_size", "intermediate_size", "num_hidden_layers", "num_attention_heads",
-                "num_key_value_heads", "head_dim", "vocab_size", "max_position_embeddings"):
-        print(f"{key}: {getattr(cfg, key)}")
-    print(f"rope_theta: {int(cfg.rope_theta)}")
-    print(f"rms_norm_eps: {cfg.rms_norm_eps:e}")
-    print(f"torch_dtype: {cfg.torch_dtype}")
-    print(f"tie_word_embeddings: {str(cfg.tie_word_embeddings).lower()}")
+    # every key of the typed configuration, whatever the architecture; numbers as the
+    # reference prints them (theta as an integer, eps in scientific notation)
+    for key, value in cfg.to_dict().items():
+        if key in ("model_type", "architectures"):
+            continue
+        if isinstance(value, bool):
+            value = str(value).lower()
+        elif isinstance(value, float):
+            value = int(value) if value >= 1.0 and value == int(value) else f"{value:e}"
+        print(f"{key}: {value}")
     return 0
 
 
 def cmd_inspect_weights(args: List[str]) -> int:
     """`src/app/cli/inspect.zig:36-72`."""
     import os
+    from .config import load_config
+    from .models.build import declare_tensors
     from .weights import SafetensorsFile
     model_dir = args[0] if args else DEFAULT_MODEL_DIR
     path = os.path.join(model_dir, "model.safetensors")
+    # what is shown: the tensors outside the layers and those of the first layer, by the
+    # names the architecture of config.json declares
+    spec = load_config(model_dir).model_spec()
+    first_layer, any_layer = spec.layer_prefix.format(0), spec.layer_prefix.split("{")[0]
+    shown = [n for n in declare_tensors(spec)
+             if n.startswith(first_layer) or not n.startswith(any_layer)]
     with SafetensorsFile(path) as f:
         print("Zinfer weights inspection")
         print(f"weights_path: {path}")
@@ -273,10 +295,7 @@ def cmd_inspect_weights(args: List[str]) -> int:
         print(f"tensor_count: {len(f.infos)}")
         for k, v in f.metadata.items():
             print(f"metadata.{k}: {v}")
-        for name in ("model.embed_tokens.weight", "model.layers.0.self_attn.q_proj.weight",
-                     "model.layers.0.self_attn.k_proj.weight",
-                     "model.layers.0.mlp.gate_proj.weight", "model.norm.weight",
-                     "lm_head.weight"):
+        for name in shown:
             if name in f.infos:
                 i = f.infos[name]
                 print(f"tensor {name}: dtype={i.dtype} shape={list(i.shape)} "
@@ -339,11 +358,12 @@ def cmd_generate(args: List[str]) -> int:
     and the answer is printed as ids."""
     model_dir, prompt, opt = parse_generate_text(args, 64)
     if not _looks_like_ids(prompt):
-        from .text import render_single_user
+        hooks = _text_hooks(model_dir)
         print("Zinfer generate")
         print(f"mode: {'think' if opt.think else 'no-think'}")
         print(f"prompt: {prompt}")
-        return _generate_text(model_dir, render_single_user(prompt, opt.think, opt.system), opt)
+        return _generate_text(model_dir, hooks.render_single_user(prompt, opt.think, opt.system),
+                              opt)
     ids = parse_token_ids(prompt)
     if not ids:
         raise CliError("EmptyPrompt")
@@ -371,8 +391,8 @@ def _generate_text(model_dir: str, prompt_text: str, opt: Options) -> int:
     a stop sequence (the family's defaults and ``--stop``), and prints the answer, piece by
     piece with ``--stream`` (`src/app/cli/runtime/generator.zig:60-140`,
     `runtime/streaming.zig:41-65`)."""
-    from .text import Tokenizer, analyze_generated_text, effective_stop_sequences
-    tok = Tokenizer.from_dir(model_dir)
+    from .text import analyze_generated_text, effective_stop_sequences
+    tok = _text_hooks(model_dir).load_tokenizer(model_dir)
     ids = tok.encode(prompt_text)
     if not ids:
         raise CliError("EmptyPrompt")
@@ -411,12 +431,13 @@ def _generate_text(model_dir: str, prompt_text: str, opt: Options) -> int:
 def cmd_generate_chat(args: List[str]) -> int:
     """`src/app/cli/generate.zig:39-75`: the prompt is a JSON file of messages."""
     model_dir, path, opt = parse_generate_text(args, 128)
-    from .text.chat import load_messages, render_messages, with_system
+    from .text.chat import load_messages, with_system
+    hooks = _text_hooks(model_dir)
     messages = with_system(load_messages(path), opt.system)
     print("Zinfer generate-chat")
     print(f"mode: {'think' if opt.think else 'no-think'}")
     print(f"messages_path: {path}")
-    return _generate_text(model_dir, render_messages(messages, opt.think), opt)
+    return _generate_text(model_dir, hooks.render_messages(messages, opt.think), opt)
 
 
 def _dir_and_one(args: List[str], what: str) -> Tuple[str, str]:
@@ -428,9 +449,8 @@ def _dir_and_one(args: List[str], what: str) -> Tuple[str, str]:
 
 def cmd_tokenize(args: List[str]) -> int:
     """`src/app/cli/tools/text.zig:5-36`."""
-    from .text import Tokenizer
     model_dir, text = _dir_and_one(args, "text")
-    ids = Tokenizer.from_dir(model_dir).encode(text)
+    ids = _text_hooks(model_dir).load_tokenizer(model_dir).encode(text)
     print("Zinfer tokenize")
     print(f"text: {text}")
     print("ids: [" + ", ".join(str(i) for i in ids) + "]")
@@ -439,12 +459,11 @@ def cmd_tokenize(args: List[str]) -> int:
 
 def cmd_decode_ids(args: List[str]) -> int:
     """`src/app/cli/tools/text.zig:38-75`."""
-    from .text import Tokenizer
     model_dir, csv = _dir_and_one(args, "ids_csv")
     ids = parse_token_ids(csv)
     print("Zinfer decode-ids")
     print("ids: [" + ", ".join(str(i) for i in ids) + "]")
-    print(f"text: {Tokenizer.from_dir(model_dir).decode(ids)}")
+    print(f"text: {_text_hooks(model_dir).load_tokenizer(model_dir).decode(ids)}")
     return 0
 
 
@@ -496,8 +515,7 @@ def cmd_serve_batch(args: List[str]) -> int:
                                f"than {sorted(allowed)} (found {sorted(extra)})")
             if "text" in raw:
                 if tok is None:
-                    from .text import Tokenizer
-                    tok = Tokenizer.from_dir(model_dir)
+                    tok = _text_hooks(model_dir).load_tokenizer(model_dir)
                 ids = tok.encode(raw["text"])
             else:
                 ids = [int(t) for t in raw["prompt"]]

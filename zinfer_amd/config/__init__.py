@@ -1,4 +1,4 @@
-from .registry import (ArchitectureEntry, entry_for, load_config, read_config_json,
+from .registry import (ArchitectureEntry, TextHooks, entry_for, load_config, read_config_json,
                        register_architecture, registered_architectures,
                        unregister_architecture)
 from .specs import (GqaAttentionSpec, ModelSpec, NoPositionSpec, PreNormBlockSpec, RmsNormSpec,

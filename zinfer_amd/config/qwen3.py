@@ -11,7 +11,7 @@ from dataclasses import dataclass, asdict, field
 from typing import List, Tuple
 
 from ..errors import ConfigError
-from .registry import register_architecture
+from .registry import TextHooks, register_architecture
 from .specs import (GqaAttentionSpec, ModelSpec, PreNormBlockSpec, RmsNormSpec,
                     RotaryHalfSplitSpec, ScheduleEntry, SwiGluSpec)
 
@@ -130,4 +130,29 @@ class Qwen3Config:
             eos_token_ids=QWEN3_EOS_TOKEN_IDS, default_stop_sequences=QWEN3_DEFAULT_STOPS)
 
 
-register_architecture("Qwen3ForCausalLM", Qwen3Config, model_type="qwen3")
+# `src/model/runtime/decoder_family.zig:249-265`: the family's tokenizer and templates; the
+# text front end is only imported when one of them is called
+def _load_tokenizer(model_dir: str):
+    from ..text import Tokenizer
+    return Tokenizer.from_dir(model_dir)
+
+
+def _render_messages(messages, thinking: bool) -> str:
+    from ..text.chat import render_messages
+    return render_messages(messages, thinking)
+
+
+def _render_single_user(user_text: str, thinking: bool, system=None) -> str:
+    from ..text.chat import render_single_user
+    return render_single_user(user_text, thinking, system)
+
+
+def _assistant_history_content(content: str) -> str:
+    from ..text.chat import strip_historical_thinking
+    return strip_historical_thinking(content)
+
+
+register_architecture(
+    "Qwen3ForCausalLM", Qwen3Config, model_type="qwen3",
+    text=TextHooks(_load_tokenizer, _render_messages, _render_single_user,
+                   _assistant_history_content))

@@ -17,18 +17,30 @@ from ..errors import ConfigError, UnsupportedModelType
 
 
 @dataclass
+class TextHooks:
+    """What an architecture brings for text in and out, as the reference's entry does
+    (`decoder_registry.zig:16-19`): the engine itself takes and returns token ids."""
+    load_tokenizer: Callable[[str], object]                  # model folder -> encode/decode
+    render_messages: Callable[..., str]                      # (messages, thinking) -> prompt
+    render_single_user: Callable[..., str]                   # (text, thinking, system) -> prompt
+    assistant_history_content: Callable[[str], str]          # an earlier answer as history
+
+
+@dataclass
 class ArchitectureEntry:
     name: str                      # e.g. "Qwen3ForCausalLM"
     model_type: Optional[str]      # e.g. "qwen3"
     config_type: type              # has from_dict(dict), to_dict(), model_spec()
+    text: Optional[TextHooks] = None
 
 
 _BY_NAME: Dict[str, ArchitectureEntry] = {}
 _BY_MODEL_TYPE: Dict[str, ArchitectureEntry] = {}
 
 
-def register_architecture(name: str, config_type: type, model_type: Optional[str] = None) -> None:
-    entry = ArchitectureEntry(name, model_type, config_type)
+def register_architecture(name: str, config_type: type, model_type: Optional[str] = None,
+                          text: Optional[TextHooks] = None) -> None:
+    entry = ArchitectureEntry(name, model_type, config_type, text)
     _BY_NAME[name] = entry
     if model_type is not None:
         _BY_MODEL_TYPE[model_type] = entry

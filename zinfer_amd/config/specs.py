@@ -93,3 +93,6 @@ class ModelSpec:
     layer_prefix: str = "model.layers.{}."
     eos_token_ids: Tuple[int, ...] = ()
     default_stop_sequences: Tuple[str, ...] = ()
+    embedding_multiplier: float = 1.0       # the embedding row times this enters the stream
+    logit_scale: float = 1.0                # logits = head(x) * logit_scale ...
+    logit_softcap: Optional[float] = None   # ... then cap * tanh(logits / cap) if given

@@ -7,24 +7,43 @@
 #include <stdio.h>
 
 // ---------------------------------------------------------------- embedding: x[t,:] = E[id[t],:]
+// times the architecture's multiplier (1 for most; the product with 1 is exact)
 template <typename TW>
 __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ ids,
-                             float* __restrict__ out, int H) {
+                             float* __restrict__ out, int H, float scale) {
   const int t = blockIdx.x;
   const TW* row = table + (size_t)ids[t] * H;
   float* o = out + (size_t)t * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = load_as_float<TW>(row + i);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = load_as_float<TW>(row + i) * scale;
 }
 
 extern "C" int zf_embed(const void* table, int table_dtype, const int* ids, float* out, int T,
-                        int H, hipStream_t stream) {
+                        int H, float scale, hipStream_t stream) {
   if (T <= 0) return 0;
   if (table_dtype == ZF_F32)
     hipLaunchKernelGGL(embed_kernel<float>, dim3(T), dim3(256), 0, stream, (const float*)table,
-                       ids, out, H);
+                       ids, out, H, scale);
   else
     hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(T), dim3(256), 0, stream,
-                       (const bf16_t*)table, ids, out, H);
+                       (const bf16_t*)table, ids, out, H, scale);
+  ZF_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------- logits after the head
+// x = x * scale, then, with cap > 0, x = cap * tanh(x / cap): what an architecture may ask for
+// between the head's product and the sampler
+__global__ void scale_cap_kernel(float* __restrict__ x, size_t n, float scale, float cap) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float v = x[i] * scale;
+  if (cap > 0.f) v = cap * tanhf(v / cap);
+  x[i] = v;
+}
+
+extern "C" int zf_scale_cap(float* x, long long n, float scale, float cap, hipStream_t stream) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(scale_cap_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
+                     x, (size_t)n, scale, cap);
   ZF_CHECK_LAUNCH();
 }
 

@@ -14,7 +14,8 @@ import numpy as np
 import torch
 
 from ..cache import NO_PAGE, CacheManager
-from ..errors import (CacheFull, PositionOutOfBounds, StepError, TokenIdOutOfBounds)
+from ..errors import (CacheFull, ConfigError, PositionOutOfBounds, StepError,
+                      TokenIdOutOfBounds)
 from ..models.decoder import DecoderModel
 from .batch import KVStepTables, Scratch, StepContext, StepEntry
 
@@ -39,6 +40,11 @@ class Engine:
             from ..ops import build
             build.prepare(getattr(model, "kernel_modules", ()))
         spec = model.spec
+        if kv_dtype is not None and kv_dtype != model.ctx.compute_dtype:
+            # the cache-write and attention kernels keep keys and values in the activations'
+            # dtype; there is no converting write
+            raise ConfigError(f"the cache is kept in the compute dtype ({model.ctx.compute_dtype}"
+                              f"): a cache of {kv_dtype} needs a model built with that dtype")
         needs = model.cache_needs()
         reads = [e.cache_of for e in spec.schedule]
         self.cache = CacheManager(needs, reads, page_size, num_pages, max_requests,
@@ -76,8 +82,9 @@ class Engine:
     def step(self, entries: Sequence[StepEntry], end: Sequence[object] = ()) -> torch.Tensor:
         """Runs the tokens of ``entries`` as one batch and returns float32 logits
         [number of wanted places, vocab] in the order of the entries and of their ``want``.
-        Requests in ``end`` give back what they hold after the step.  On an error nothing
-        has run and the cache is as before."""
+        Requests in ``end`` give back what they hold after the step.  On an error the cache
+        is as before: what can be refused is refused before anything runs, and a failure
+        inside the run gives back what the step had reserved."""
         seen, wanted_len = self._check_entries(entries)
         for rid in end:
             if rid not in seen and not self.cache.has_request(rid):
@@ -86,28 +93,29 @@ class Engine:
             raise CacheFull(f"CacheFull: the step needs more pages or request slots than are "
                             f"free (free pages per group: {self.cache.num_free_pages()})")
         if entries:
-            for rid, new_len in wanted_len:
-                if not self.cache.has_request(rid):
-                    self.cache.add_request(rid)
-                self.cache.reserve(rid, new_len)
-            decode_only = self.use_graphs and all(len(e.tokens) == 1 for e in entries)
-            traced = self.step_trace is not None and self.device.type == "cuda"
-            if traced:
-                import time
-                t0 = time.perf_counter()
-            ctx = self._build_context(entries, bucket_pages=decode_only)
-            if traced:
-                t1 = time.perf_counter()
-                before = torch.cuda.Event(enable_timing=True)
-                after = torch.cuda.Event(enable_timing=True)
-                before.record()
-            logits = self._forward_graphed(ctx) if decode_only \
-                else self.model.forward(ctx, self.views)
-            if traced:
-                after.record()
-                self.step_trace.append((ctx.n_tokens, ctx.n_seqs, t1 - t0,
-                                        time.perf_counter() - t1, before, after,
-                                        ctx.max_q_len > 1))
+            added = self._reserve(wanted_len)
+            try:
+                decode_only = self.use_graphs and all(len(e.tokens) == 1 for e in entries)
+                traced = self.step_trace is not None and self.device.type == "cuda"
+                if traced:
+                    import time
+                    t0 = time.perf_counter()
+                ctx = self._build_context(entries, bucket_pages=decode_only)
+                if traced:
+                    t1 = time.perf_counter()
+                    before = torch.cuda.Event(enable_timing=True)
+                    after = torch.cuda.Event(enable_timing=True)
+                    before.record()
+                logits = self._forward_graphed(ctx) if decode_only \
+                    else self.model.forward(ctx, self.views)
+                if traced:
+                    after.record()
+                    self.step_trace.append((ctx.n_tokens, ctx.n_seqs, t1 - t0,
+                                            time.perf_counter() - t1, before, after,
+                                            ctx.max_q_len > 1))
+            except BaseException:
+                self._roll_back(wanted_len, added)
+                raise
             for rid, new_len in wanted_len:
                 self.cache.commit(rid, new_len)
             self.steps_run += 1
@@ -117,6 +125,32 @@ class Engine:
         for rid in end:
             self.cache.release(rid)
         return logits
+
+    def _reserve(self, wanted_len) -> List[object]:
+        """Adds the requests that are new and reserves every request's pages; returns the
+        ids that were added."""
+        added = []
+        try:
+            for rid, new_len in wanted_len:
+                if not self.cache.has_request(rid):
+                    self.cache.add_request(rid)
+                    added.append(rid)
+                self.cache.reserve(rid, new_len)
+        except BaseException:
+            self._roll_back(wanted_len, added)
+            raise
+        return added
+
+    def _roll_back(self, wanted_len, added) -> None:
+        """A step failed after it had reserved: the requests it added go, the pages it
+        reserved beyond what the others hold go back.  (Keys and values that kernels may
+        already have written lie beyond the requests' lengths and are never read.)"""
+        for rid, _ in wanted_len:
+            if rid in added:
+                if self.cache.has_request(rid):
+                    self.cache.release(rid)
+            elif self.cache.has_request(rid):
+                self.cache.trim(rid)
 
     def _check_entries(self, entries: Sequence[StepEntry], extra: int = 0):
         """What can be refused before anything runs.  Returns the ids of the entries and
@@ -169,41 +203,42 @@ class Engine:
         if not self.cache.can_reserve(wanted_len):
             raise CacheFull(f"CacheFull: {n_steps} steps need more pages or request slots than "
                             f"are free (free pages per group: {self.cache.num_free_pages()})")
-        for rid, new_len in wanted_len:
-            if not self.cache.has_request(rid):
-                self.cache.add_request(rid)
-            self.cache.reserve(rid, new_len)
-        traced = self.step_trace is not None
-        if traced:
-            import time
-            t0 = time.perf_counter()
-        ctx = self._build_context(entries, bucket_pages=True, extra_tokens=extra)
-        if traced:
-            t1 = time.perf_counter()
-            before = torch.cuda.Event(enable_timing=True)
-            after = torch.cuda.Event(enable_timing=True)
-            before.record()
-        out = self._scratch.get("decoded", (n_steps, n), torch.int32)
-        rec = None
-        if records is not None:
-            rec = torch.from_numpy(records.view(np.uint8).reshape(n_steps, -1).copy()) \
-                .to(self.device)
-        for s in range(n_steps):
-            if s:
-                for g, tables in enumerate(ctx.kv):
-                    ops.advance_decode(ctx.token_ids, ctx.positions, ctx.ctx_len, out[s - 1],
-                                       tables.slot_mapping, tables.block_table, self.page_size,
-                                       advance=(g == 0))
-            logits = self._forward_graphed(ctx)
-            if rec is None:
-                ops.argmax(logits, out[s])
-            else:
-                ops.sample_topk(logits, rec[s], out[s])
-        if traced:
-            after.record()
-            self.step_trace.append((n * n_steps, n, t1 - t0, time.perf_counter() - t1, before,
-                                    after, False))
-        tokens = out.tolist()
+        added = self._reserve(wanted_len)
+        try:
+            traced = self.step_trace is not None
+            if traced:
+                import time
+                t0 = time.perf_counter()
+            ctx = self._build_context(entries, bucket_pages=True, extra_tokens=extra)
+            if traced:
+                t1 = time.perf_counter()
+                before = torch.cuda.Event(enable_timing=True)
+                after = torch.cuda.Event(enable_timing=True)
+                before.record()
+            out = self._scratch.get("decoded", (n_steps, n), torch.int32)
+            rec = None
+            if records is not None:
+                rec = torch.from_numpy(records.view(np.uint8).reshape(n_steps, -1).copy()) \
+                    .to(self.device)
+            for s in range(n_steps):
+                if s:
+                    for g, tables in enumerate(ctx.kv):
+                        ops.advance_decode(ctx.token_ids, ctx.positions, ctx.ctx_len, out[s - 1],
+                                           tables.slot_mapping, tables.block_table, self.page_size,
+                                           advance=(g == 0))
+                logits = self._forward_graphed(ctx)
+                if rec is None:
+                    ops.argmax(logits, out[s])
+                else:
+                    ops.sample_topk(logits, rec[s], out[s])
+            if traced:
+                after.record()
+                self.step_trace.append((n * n_steps, n, t1 - t0, time.perf_counter() - t1, before,
+                                        after, False))
+            tokens = out.tolist()
+        except BaseException:
+            self._roll_back(wanted_len, added)
+            raise
         for rid, new_len in wanted_len:
             self.cache.commit(rid, new_len)
         self.steps_run += n_steps

@@ -12,7 +12,12 @@ never run out; portions, the budget and what happens when pages run out are this
 * when a running request cannot get the page it needs, the most recently admitted running
   request is preempted: its pages are freed, it keeps its generated tokens and its random
   stream, goes to the front of the waiting queue and later recomputes prompt + generated;
-* a request that cannot fit even alone raises CacheFull.
+* a request that can never run (a token id beyond the vocabulary, a prompt longer than the
+  position table or than the whole pool, an empty prompt) is rejected when it is added: it
+  finishes at once with ``finish_reason`` "rejected" and the reason in ``error``, and the
+  next ``step()`` hands it back among the finished; the other requests never see it;
+* a request that is alone and still outgrows the pool while it decodes finishes with
+  ``finish_reason`` "cache" and keeps its tokens.
 
 When every running request decodes and nobody waits, up to ``multi_step`` decode steps run in
 a row on the device without the host between them; tokens that a request drew after its
@@ -43,6 +48,7 @@ class Request:
     finished: bool = False
     finish_reason: Optional[str] = None
     preemptions: int = 0
+    error: Optional[str] = None        # why the request was rejected
     counts: Optional[Dict[int, int]] = None    # occurrences of each token so far (penalties)
 
     @property
@@ -80,24 +86,52 @@ class Scheduler:
         self.n_steps = 0                    # engine steps so far
         self.last_steps = 0                 # engine steps the last call of step() ran
         self.n_preemptions = 0
+        self._rejected: List[Request] = []   # finished when added; handed back by step()
 
     # ------------------------------------------------------------------ requests
     def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None,
                     request_id=None) -> object:
+        """Queues a request and returns its id.  An id that is already in use is the caller's
+        mistake and raises; a request that can never run is rejected (see the module's text)."""
         prompt = [int(t) for t in prompt]
-        if not prompt:
-            raise StepError("a prompt must hold at least one token")
         params = params or SamplingParams()
         rid = request_id if request_id is not None else self._next_id
+        if rid in self.finished or self.cache.has_request(rid) or \
+                any(r.id == rid for r in self.running) or any(r.id == rid for r in self.waiting):
+            raise StepError(f"request id {rid!r} is already in use")
         index = self._next_id
         self._next_id += 1
         # every request has a stream of its own, so its output does not depend on the batch
         rng = Xoshiro256pp((params.seed ^ (index * 0x9E3779B97F4A7C15)) & ((1 << 64) - 1))
-        self.waiting.append(Request(rid, prompt, params, rng=rng))
+        req = Request(rid, prompt, params, rng=rng)
+        why = self._why_it_can_never_run(req)
+        if why is not None:
+            req.finished, req.finish_reason, req.error = True, "rejected", why
+            self.finished[rid] = req
+            self._rejected.append(req)
+        else:
+            self.waiting.append(req)
         return rid
 
+    def _why_it_can_never_run(self, req: Request) -> Optional[str]:
+        spec = self.engine.model.spec
+        if not req.prompt:
+            return "EmptyPrompt: a prompt must hold at least one token"
+        bad = next((t for t in req.prompt if not (0 <= t < spec.vocab_size)), None)
+        if bad is not None:
+            return f"TokenIdOutOfBounds: token {bad}, vocabulary {spec.vocab_size}"
+        if len(req.prompt) > spec.max_positions:
+            return (f"PositionOutOfBounds: a prompt of {len(req.prompt)} tokens, "
+                    f"max_position_embeddings is {spec.max_positions}")
+        # the prompt and the first generated token must fit into the pool when it is alone
+        need = self.cache.pages_at_most(len(req.prompt) + 1, self.chunk_size)
+        if any(n > total for n, total in zip(need, self.cache.num_pages())):
+            return (f"CacheFull: a prompt of {len(req.prompt)} tokens needs {need} pages, the "
+                    f"pool has {self.cache.num_pages()}")
+        return None
+
     def has_work(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self.waiting or self.running or self._rejected)
 
     def request(self, rid) -> Request:
         """The request with this id, wherever it is."""
@@ -127,6 +161,7 @@ class Scheduler:
     # ------------------------------------------------------------------ planning
     def plan(self) -> List[PlannedEntry]:
         """Decides what the next step runs.  May preempt; admits from the waiting queue."""
+        self._ended_by_plan: List[Request] = []
         while True:
             planned: List[PlannedEntry] = []
             budget = self.max_step_tokens
@@ -183,6 +218,11 @@ class Scheduler:
                 # a running request cannot get its pages: the newest running request yields
                 self._preempt(self.running[-1])
                 continue
+            if starved is not None and len(self.running) == 1 and starved.generated:
+                # alone, and its next token still does not fit: it ends here with what it has
+                self._finish(starved, "cache")
+                self._ended_by_plan.append(starved)
+                continue
             if not planned:
                 blocked = starved or (self.waiting[0] if self.waiting else None)
                 if blocked is not None and not self.running or \
@@ -205,13 +245,14 @@ class Scheduler:
     # ------------------------------------------------------------------ one iteration
     def step(self) -> List[Request]:
         """Plans, runs one step, samples, finishes.  Returns the requests finished by it."""
+        rejected, self._rejected = self._rejected, []
         k = self._multi_step_count()
         if k >= 2:
-            return self._decode_multi(k)
+            return rejected + self._decode_multi(k)
         planned = self.plan()
         self.last_steps = 1 if planned else 0
         if not planned:
-            return []
+            return rejected + self._ended_by_plan
         entries = []
         for p in planned:
             toks = p.request.tokens[p.request.n_computed:p.request.n_computed + p.n_tokens]
@@ -220,7 +261,7 @@ class Scheduler:
         self.n_steps += 1
         sampling = [p for p in planned if p.samples]
         next_tokens = self._sample(logits, sampling)
-        done: List[Request] = []
+        done: List[Request] = rejected + self._ended_by_plan
         for p in planned:
             p.request.n_computed += p.n_tokens
         for p, tok in zip(sampling, next_tokens):

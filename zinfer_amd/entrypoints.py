@@ -58,15 +58,21 @@ class LLM:
         return cls(None, config=config, random_seed=seed, **options)
 
     def _default_max_tokens(self, spec, page_size: int, max_seqs: int) -> int:
+        from .parts.base import KVNeed, StateNeed
         want = max_seqs * spec.max_positions
-        per_token = 0
+        elem = 2 if self.model.ctx.compute_dtype == torch.bfloat16 else 4   # the cache's dtype
+        per_token, state_bytes = 0, 0
         for need in self.model.cache_needs():
-            if need is not None and hasattr(need, "n_kv_heads"):
-                per_token += 2 * need.n_kv_heads * need.head_dim * \
-                    (2 if self.model.ctx.compute_dtype == torch.bfloat16 else 4)
+            if isinstance(need, KVNeed):
+                per_token += 2 * need.n_kv_heads * need.head_dim * elem
+            elif isinstance(need, StateNeed):
+                n = max_seqs
+                for d in need.shape:
+                    n *= d
+                state_bytes += n * torch.empty((), dtype=need.dtype).element_size()
         if self.model.ctx.device.type == "cuda" and per_token:
             free, _ = torch.cuda.mem_get_info(self.model.ctx.device)
-            want = min(want, int(free * 0.5) // per_token)
+            want = min(want, int(max(free - state_bytes, 0) * 0.5) // per_token)
         return max(page_size, want)
 
     def new_scheduler(self) -> Scheduler:

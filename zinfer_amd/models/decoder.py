@@ -58,8 +58,11 @@ class DecoderModel:
         self.final_norm.bind(tensors)
         if s.head_name in tensors:
             self.head = Linear(place_matrix(tensors[s.head_name], self.ctx))
-        else:  # tied: the embedding stands in for the head
-            self.head = Linear(self.embedding, pretile=False)
+        else:
+            # tied: the embedding stands in for the head.  Where the matrix pre-tiles, the
+            # head's product reads a second copy in the kernels' own order (the embedding
+            # itself stays in rows for the gather); elsewhere both are one tensor.
+            self.head = Linear(self.embedding)
 
     # ---------------------------------------------------------------- cache needs
     def cache_needs(self) -> List[Optional[object]]:
@@ -75,7 +78,7 @@ class DecoderModel:
         s = self.spec
         T = step.n_tokens
         x = step.scratch("residual", (T, s.hidden_size), torch.float32)
-        ops.embed(self.embedding, step.token_ids, x)
+        ops.embed(self.embedding, step.token_ids, x, float(s.embedding_multiplier))
         lazy_final = isinstance(self.final_norm, RmsNorm) and x.is_cuda \
             and self.ctx.compute_dtype == torch.bfloat16
         step.norm_ready = None
@@ -105,4 +108,6 @@ class DecoderModel:
             self.head.forward(LazyRmsNorm(self.final_norm, rows, make, given), logits)
         else:
             self.head.forward(self.final_norm.forward(rows, make()), logits)
+        if s.logit_scale != 1.0 or s.logit_softcap is not None:
+            ops.scale_cap(logits, float(s.logit_scale), float(s.logit_softcap or 0.0))
         return logits

@@ -61,8 +61,8 @@ def _i32(t: torch.Tensor, what: str) -> None:
 
 
 # ------------------------------------------------------------------------- elementwise
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
-    """out[t, :] = table[ids[t], :] widened to float32 (no scale factor)."""
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+    """out[t, :] = table[ids[t], :] widened to float32, times ``scale``."""
     _need_gpu(table, ids, out)
     _i32(ids, "ids")
     T, H = out.shape
@@ -70,7 +70,18 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
         raise KernelUnavailable(f"embed: table {tuple(table.shape)}, ids {tuple(ids.shape)}, "
                                 f"out {tuple(out.shape)} {out.dtype}")
     lib = build.load("elementwise")
-    _check(lib.zf_embed(_ptr(table), _dt(table), _ptr(ids), _ptr(out), T, H, _stream()), "embed")
+    _check(lib.zf_embed(_ptr(table), _dt(table), _ptr(ids), _ptr(out), T, H,
+                        ctypes.c_float(scale), _stream()), "embed")
+
+
+def scale_cap(x: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> None:
+    """In place on float32: x = x * scale, then with cap > 0: x = cap * tanh(x / cap)."""
+    _need_gpu(x)
+    if x.dtype != torch.float32 or cap < 0.0:
+        raise KernelUnavailable("scale_cap: a float32 tensor and a cap that is not negative")
+    lib = build.load("elementwise")
+    _check(lib.zf_scale_cap(_ptr(x), ctypes.c_longlong(x.numel()), ctypes.c_float(scale),
+                            ctypes.c_float(cap), _stream()), "scale_cap")
 
 
 def rmsnorm(x: torch.Tensor, gain: torch.Tensor, eps: float, out: torch.Tensor) -> None:
@@ -556,6 +567,7 @@ def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bo
 
 
 # ------------------------------------------------------------------------- attention
+MAX_HEAD_DIM = 512          # the wave kernel keeps a head in registers: 8 values a lane
 DECODE_SPLIT_KEYS = 256     # keys per split of the decode kernel (DEC_SPLIT in attention.hip)
 
 
@@ -589,8 +601,9 @@ def paged_attention(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index,
         _i32(t, name)
     if n_heads % n_kv_heads != 0:
         raise KernelUnavailable("paged_attention: InvalidGrouping")
-    if head_dim > 512:
-        raise KernelUnavailable(f"paged_attention: head_dim {head_dim} > 512 is not covered")
+    if head_dim > MAX_HEAD_DIM:
+        raise KernelUnavailable(f"paged_attention: head_dim {head_dim} > {MAX_HEAD_DIM} is not "
+                                "covered")
     if max_ctx_len > block_table.shape[1] * page_size:
         raise KernelUnavailable("paged_attention: block table shorter than the context")
     n_seqs = ctx_len.shape[0]

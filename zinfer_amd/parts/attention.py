@@ -30,6 +30,9 @@ class GqaAttention(Mixer):
             raise ConfigError("InvalidDimensions: heads and head_dim must not be 0")
         if s.n_heads % s.n_kv_heads != 0:
             raise ConfigError(f"InvalidGrouping: {s.n_heads} query heads, {s.n_kv_heads} kv heads")
+        if s.head_dim % 2 != 0 or s.head_dim > ops.MAX_HEAD_DIM:
+            raise ConfigError(f"InvalidHeadDim: head_dim={s.head_dim}: the attention kernels "
+                              f"take even head sizes up to {ops.MAX_HEAD_DIM}")
         if s.window is not None and s.window < 1:
             raise ConfigError(f"window={s.window} must be at least 1")
         self.q_width = s.n_heads * s.head_dim

@@ -9,8 +9,8 @@ from .. import ops
 
 class Linear:
     """``pretile``: a bfloat16 matrix on the GPU whose sizes allow it is re-laid once into the
-    MFMA kernels' own order (the plain copy is dropped); pass False for a matrix that is also
-    read by rows (a tied embedding)."""
+    MFMA kernels' own order; the copy in rows is not kept here (a caller that also reads the
+    matrix by rows, as a tied embedding is read, keeps its own)."""
 
     def __init__(self, weight: torch.Tensor, pretile: bool = True):
         assert weight.dim() == 2

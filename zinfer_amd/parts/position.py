@@ -24,6 +24,23 @@ def rotary_tables(head_dim: int, theta: float, max_positions: int):
             torch.from_numpy(np.sin(angle).astype(np.float32)))
 
 
+_device_tables = {}     # (specification, device) -> (cos, sin): layers with equal specs share
+
+
+def device_rotary_tables(spec, device):
+    """The tables of ``spec`` on ``device``, built and uploaded once however many layers ask."""
+    key = (spec, str(device))
+    held = _device_tables.get(key)
+    if held is None:
+        cos, sin = rotary_tables(spec.head_dim, spec.theta, spec.max_positions)
+        held = (cos.to(device), sin.to(device))
+        _device_tables[key] = held
+        for k in [k for k in _device_tables if k != key and k[1] == key[1]
+                  and len(_device_tables) > 8]:
+            del _device_tables[k]      # a process that builds many models keeps the newest
+    return held
+
+
 class RotaryHalfSplit(PositionEncoding):
     """Half-split rotation over the full head (`src/kernel/attention/rope.zig:92-109`); the
     attention kernel applies it from the tables."""
@@ -32,9 +49,7 @@ class RotaryHalfSplit(PositionEncoding):
 
     def __init__(self, spec, ctx, prefix):
         super().__init__(spec, ctx, prefix)
-        cos, sin = rotary_tables(spec.head_dim, spec.theta, spec.max_positions)
-        self.cos = cos.to(ctx.device)
-        self.sin = sin.to(ctx.device)
+        self.cos, self.sin = device_rotary_tables(spec, ctx.device)
 
     def rotation_tables(self):
         return self.cos, self.sin

@@ -5,8 +5,12 @@ Everything is checked at load, before anything runs: one error lists every missi
 every unexpected one and every wrong shape.  (The reference finds a missing name at
 `src/tensor/backends/backend.zig:98` and a wrong shape only at first use,
 `src/tensor/storage/store.zig:177-182`.)  Tensors keep the dtype they are stored in
-(bfloat16 or 32-bit float; integer tables become int32); what a compute dtype does with them
-is the parts' business.
+(bfloat16 or 32-bit float; float16 and float64 become 32-bit floats, integer tables int32);
+what a compute dtype does with them is the parts' business.
+
+Tensors the model does not declare are an error, not ignored: a folder that brings a bias, a
+second head or another architecture's layers would otherwise load and run with formulas that
+are not its own.
 """
 from __future__ import annotations
 
@@ -73,9 +77,10 @@ def load_tensors(model_dir: str, decls: Dict[str, TensorDecl]) -> Dict[str, torc
             info = where[n].infos[n]
             if info.dtype in _INT:
                 t = t.to(torch.int32)
-            elif info.dtype == "F16":
-                t = t.to(torch.bfloat16)
-            elif info.dtype == "F64":
+            elif info.dtype in ("F16", "F64"):
+                # float16 widens exactly; rounding it to bfloat16 here would take 3 bits of
+                # mantissa from a 32-bit build's weights.  What a bfloat16 build does with a
+                # 32-bit tensor is the parts' business.
                 t = t.to(torch.float32)
             out[n] = t
         return out
