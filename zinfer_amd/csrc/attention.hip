@@ -328,6 +328,19 @@ __global__ __launch_bounds__(64) void attn_decode_merge_kernel(
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int first = lo / DEC_SPLIT, last = pos / DEC_SPLIT;
   const size_t base = ((size_t)s * nH + head) * max_splits;
+  // the first eight splits' partial outputs are asked for together with the (max, sum)
+  // pairs, before the weights are known: one trip to memory less for contexts of up to
+  // 2048 keys, where this kernel is nothing but such trips
+  float v0[8][8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const float* src = ws_o + (base + min(first + u, last)) * hd;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int d = lane + 64 * i;
+      v0[u][i] = (d < hd) ? src[d] : 0.f;
+    }
+  }
   float mx = -INFINITY;
   for (int sp = first + lane; sp <= last; sp += 64) mx = fmaxf(mx, ws_ml[(base + sp) * 2]);
   mx = wave_max(mx);
@@ -347,14 +360,21 @@ __global__ __launch_bounds__(64) void attn_decode_merge_kernel(
     const int n = min(64, last - chunk + 1);
     for (int i0 = 0; i0 < n; i0 += 8) {
       float v[8][8];
+      if (chunk == first && i0 == 0) {
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int sp = min(chunk + i0 + u, last);
-        const float* src = ws_o + (base + sp) * hd;
+        for (int u = 0; u < 8; ++u)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const int d = lane + 64 * i;
-          v[u][i] = (d < hd) ? src[d] : 0.f;
+          for (int i = 0; i < 8; ++i) v[u][i] = v0[u][i];
+      } else {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int sp = min(chunk + i0 + u, last);
+          const float* src = ws_o + (base + sp) * hd;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const int d = lane + 64 * i;
+            v[u][i] = (d < hd) ? src[d] : 0.f;
+          }
         }
       }
 #pragma unroll

@@ -736,28 +736,61 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_skinny_kernel(
   const u32x4_t zero = u32x4_t{0, 0, 0, 0};
   const int kstride = NW * 64 * gridDim.y;
   int k0 = (blockIdx.y * NW + wave) * 64;
-  if (WT && NORM != NORM_FOLD && RG * MT == 1) {
-    // one row group and up to 16 tokens per wave: take 4 k-steps at once so that more loads
-    // are in flight (pre-tiled weights need no bounds checks; K % 64 == 0); measured to help
-    // only in this case
-    constexpr int UNR = 4;
-    for (; k0 + (UNR - 1) * kstride < K; k0 += UNR * kstride) {
-      u32x4_t w0[UNR][RG], w1[UNR][RG], a0[UNR][MT], a1[UNR][MT];
+  // What the epilogue reads from memory is asked for now, so that it has arrived when the
+  // last weights have: the residual and the next norm's gains (wave 0 writes the outputs of
+  // one row group and up to 16 tokens), and the producer's sums of squares.
+  constexpr bool PRE_EPI = EMIT && RG * MT == 1;
+  float4 pre_c = float4{0.f, 0.f, 0.f, 0.f}, pre_g = float4{0.f, 0.f, 0.f, 0.f};
+  if (PRE_EPI && wave == 0 && gridDim.y == 1) {
+    const int token = lane % 16, n = n0 + 4 * (lane / 16);
+    if (token < M && n + 3 < N) {
+      pre_c = *(const float4*)((const float*)Cv + (size_t)token * N + n);
+      pre_g = *(const float4*)(nrm.gain_out + n);
+    }
+  }
+  // the producer's sums of squares per 16 columns: thread (p, j) adds groups p, p + NSS, ...
+  // of token j; the first SQ_PRE of them are asked for here, before the weights
+  constexpr int SQ_PRE = NORM == NORM_GIVEN ? 16 : 1;
+  float sqv[SQ_PRE];
+  if (NORM == NORM_GIVEN) {
+    const int j = tid % 16, p = tid / 16;
+#pragma unroll
+    for (int i = 0; i < SQ_PRE; ++i) {
+      const int gidx = p + i * NSS;
+      sqv[i] = gidx < nrm.sq_groups ? nrm.sq_in[gidx * 16 + j] : 0.f;
+    }
+  }
+  if (WT && NORM != NORM_FOLD && (RG * MT == 1 || (RG * MT == 2 && EPI != EPI_SWIGLU))) {
+    // Pre-tiled weights (no bounds checks; K % 64 == 0), up to two MFMA tiles per k-step:
+    // batches of UNR k-steps in two register sets, the next batch asked for before the
+    // MFMAs of the one that has arrived, so that a wave always has loads in flight.  The
+    // paths below are laid out so that every wait has a known number of younger loads.
+    // (Measured in a replayed graph at 1 and 8 tokens, 4096 x 4096, 4096 x 12288 and
+    // 6144 x 4096: 0.1 to 1.0 us less than waiting for each batch before asking for the
+    // next; the gate/up product with its three workgroups to a CU loses by it and keeps the
+    // plain loop below.)
+    constexpr int UNR = RG * MT == 1 ? 4 : 2;
+    u32x4_t w0[2][UNR][RG], w1[2][UNR][RG], a0[2][UNR][MT], a1[2][UNR][MT];
+    auto load = [&](auto BUF, int kb) {
+      constexpr int B = decltype(BUF)::value;
 #pragma unroll
       for (int u = 0; u < UNR; ++u) {
-        const int kk = k0 + u * kstride;
+        const int kk = kb + u * kstride;
 #pragma unroll
         for (int r = 0; r < RG; ++r) {
           const bf16_t* tile = wrow[r] + (size_t)(kk / 64) * 1024;
-          w0[u][r] = __builtin_nontemporal_load((const u32x4_t*)tile);
-          w1[u][r] = __builtin_nontemporal_load((const u32x4_t*)(tile + 512));
+          w0[B][u][r] = __builtin_nontemporal_load((const u32x4_t*)tile);
+          w1[B][u][r] = __builtin_nontemporal_load((const u32x4_t*)(tile + 512));
         }
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
-          a0[u][t] = tok[t] ? *(const u32x4_t*)(arow[t] + kk + g * 16) : zero;
-          a1[u][t] = tok[t] ? *(const u32x4_t*)(arow[t] + kk + g * 16 + 8) : zero;
+          a0[B][u][t] = tok[t] ? *(const u32x4_t*)(arow[t] + kk + g * 16) : zero;
+          a1[B][u][t] = tok[t] ? *(const u32x4_t*)(arow[t] + kk + g * 16 + 8) : zero;
         }
       }
+    };
+    auto compute = [&](auto BUF) {
+      constexpr int B = decltype(BUF)::value;
 #pragma unroll
       for (int u = 0; u < UNR; ++u)
 #pragma unroll
@@ -765,10 +798,39 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_skinny_kernel(
 #pragma unroll
           for (int t = 0; t < MT; ++t) {
             acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                *(bf16x8_t*)&w0[u][r], *(bf16x8_t*)&a0[u][t], acc[r][t], 0, 0, 0);
+                *(bf16x8_t*)&w0[B][u][r], *(bf16x8_t*)&a0[B][u][t], acc[r][t], 0, 0, 0);
             acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                *(bf16x8_t*)&w1[u][r], *(bf16x8_t*)&a1[u][t], acc[r][t], 0, 0, 0);
+                *(bf16x8_t*)&w1[B][u][r], *(bf16x8_t*)&a1[B][u][t], acc[r][t], 0, 0, 0);
           }
+    };
+    using B0 = std::integral_constant<int, 0>;
+    using B1 = std::integral_constant<int, 1>;
+    const int bstride = UNR * kstride;
+    // whole batches of this wave: k0 + (nb * UNR - 1) * kstride < K
+    const int nb = k0 < K ? ((K - 1 - k0) / kstride + 1) / UNR : 0;
+    if (nb > 0) {
+      load(B0{}, k0);
+      int b = 0;
+      for (; b + 2 < nb; b += 2) {
+        load(B1{}, k0 + (b + 1) * bstride);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(B0{});
+        __builtin_amdgcn_sched_barrier(0);
+        load(B0{}, k0 + (b + 2) * bstride);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(B1{});
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (nb - b == 2) {
+        load(B1{}, k0 + (b + 1) * bstride);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(B0{});
+        __builtin_amdgcn_sched_barrier(0);
+        compute(B1{});
+      } else {
+        compute(B0{});
+      }
+      k0 += nb * bstride;
     }
   }
   for (; k0 < K; k0 += kstride) {
@@ -843,7 +905,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_skinny_kernel(
     // thread (p, j) adds groups p, p + NSS, ... of token j, the rest follows in order of p
     const int j = tid % 16, p = tid / 16;
     float v = 0.f;
-    for (int gidx = p; gidx < nrm.sq_groups; gidx += NSS) v += nrm.sq_in[gidx * 16 + j];
+#pragma unroll
+    for (int i = 0; i < SQ_PRE; ++i) v += sqv[i];
+    for (int gidx = p + SQ_PRE * NSS; gidx < nrm.sq_groups; gidx += NSS)
+      v += nrm.sq_in[gidx * 16 + j];
     ssum[p][0][j] = v;
   }
   __syncthreads();
@@ -910,10 +975,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_skinny_kernel(
             } else if (EPI == EPI_STORE_F32) {
               ((float*)Cv)[off] = s[e];
             } else {
-              const float v = ((float*)Cv)[off] + s[e];
+              const float old = PRE_EPI ? ((const float*)&pre_c)[e] : ((float*)Cv)[off];
+              const float v = old + s[e];
               ((float*)Cv)[off] = v;
               if (EMIT) {   // what the RMSNorm after this sum needs: v * gain, and v^2
-                nrm.xg_out[off] = float_to_bf16(v * nrm.gain_out[n]);
+                const float go = PRE_EPI ? ((const float*)&pre_g)[e] : nrm.gain_out[n];
+                nrm.xg_out[off] = float_to_bf16(v * go);
                 sq += v * v;
               }
             }
