@@ -264,8 +264,9 @@ def main_continuous(args) -> int:
         raw["num_hidden_layers"] = args.layers
     n, lo, hi, new = args.requests, args.prompt_min, args.prompt_max, args.new_tokens
     t_build = time.perf_counter()
+    step_tokens = args.step_tokens or args.chunk
     llm = build_llm(raw, args.dtype, args.seed, n * (hi + new + PAGE), n,
-                    max_step_tokens=args.chunk + n, chunk_size=args.chunk,
+                    max_step_tokens=step_tokens, chunk_size=args.chunk,
                     multi_step=args.multi_step)
     cfg = llm.config
     build_s = time.perf_counter() - t_build
@@ -280,7 +281,7 @@ def main_continuous(args) -> int:
             "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
             "config": config_of(cfg, args.shape or "14b", requests=n, prompt_min=lo,
                                 prompt_max=hi, new_tokens=new, chunk_size=args.chunk,
-                                max_step_tokens=args.chunk + n,
+                                max_step_tokens=step_tokens,
                                 steps_in_a_row=args.multi_step),
             "continuous": res, "build_s": round(build_s, 1)}
     print(json.dumps(line))
@@ -424,7 +425,7 @@ def main_decode(args) -> int:
         drop(llm)
         n = 32
         llm = build_llm(SHAPES["14b"], args.dtype, args.seed, n * (4096 + 256 + PAGE), n,
-                        max_step_tokens=512 + n, chunk_size=512, multi_step=args.multi_step)
+                        max_step_tokens=512, chunk_size=512, multi_step=args.multi_step)
         res = run_continuous(llm, llm.config, elem, n, 128, 4096, 256, args.seed + 7)
         points["continuous_14b_total"] = res["total_tok_s"]
         points["continuous_14b_decode"] = res["decode_tok_s"]
@@ -475,6 +476,9 @@ def main() -> int:
     ap.add_argument("--prompt-max", type=int, default=4096)
     ap.add_argument("--new-tokens", type=int, default=256)
     ap.add_argument("--chunk", type=int, default=512, help="continuous: tokens of a prompt per step")
+    ap.add_argument("--step-tokens", type=int, default=None,
+                    help="continuous: token budget of a step (default: the chunk, so that a "
+                         "prompt's portion and the decode tokens beside it fill whole tiles)")
     ap.add_argument("--context", type=int, default=8192, help="long-context: context decoded at")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()

@@ -33,7 +33,10 @@ def test_tiled_products(N, K):
         if ks > 1:
             assert K // 64 // ks >= 8, "every workgroup keeps at least 8 k-tiles"
             tiles = ((M + 127) // 128) * ((N + 127) // 128)
-            assert tiles < 192 and tiles * ks <= 256
+            # a split fills the chip's places (256, or 512 with two workgroups to a CU) more
+            # evenly than the tiles alone do
+            places = lambda n: 256 if n <= 256 else (n + 511) // 512 * 512
+            assert tiles < 384 and places(tiles * ks) / (tiles * ks) < places(tiles) / tiles
         assert ops._tile_variant(M, N, True, False, K) in (6, 10, 16)
         if ops._tile_variant(M, N, True, False, K) == 16:
             assert K % 128 == 0
@@ -42,6 +45,13 @@ def test_tiled_products(N, K):
     # one and a half times
     assert ops._tile_variant(2048, 24576, True) == 10 and ops._tile_variant(2048, 4096, True) == 10
     assert ops._tile_variant(2048, 6144, True) == 6
+    # measured choices at a few hundred tokens (Qwen3-8B and 14B widths)
+    for (M, n, k), want in {(512, 5120, 5120): 3, (512, 5120, 17408): 3, (512, 7168, 5120): 1,
+                            (512, 4096, 4096): 2, (512, 4096, 12288): 2, (512, 6144, 4096): 1,
+                            (256, 4096, 4096): 4, (256, 6144, 4096): 2, (1024, 5120, 17408): 3,
+                            (1024, 4096, 12288): 1}.items():
+        assert ops._tile_ksplit(M, n, k) == want, (M, n, k)
+    assert ops._tile_variant(512, 24576, True, False, 4096) == 10
 
 
 def test_weight_streaming_plans():
@@ -50,3 +60,26 @@ def test_weight_streaming_plans():
             for tiled in (True, False):
                 rg, ks = ops._skinny_plan(M, N, K, tiled)
                 assert rg in (1, 2, 4) and 1 <= ks <= 16
+
+
+def test_the_flat_kernel_table_is_complete_and_its_references_exist():
+    """Every function of `zinfer_amd.ops` that launches a kernel is in the table once, its
+    module is one the build knows, and the reference it names exists."""
+    import importlib
+    import inspect
+    import os
+    import re
+    from zinfer_amd.ops import build, table
+    launchers = {name for name, fn in vars(ops).items()
+                 if inspect.isfunction(fn) and fn.__module__ == "zinfer_amd.ops"
+                 and not name.startswith("_") and "build.load(" in inspect.getsource(fn)}
+    assert launchers == set(table.KERNELS), launchers ^ set(table.KERNELS)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for name, entry in table.KERNELS.items():
+        assert entry.launch is getattr(ops, name)
+        assert entry.module in build.MODULES
+        path, fn = entry.reference.split(":")
+        with open(os.path.join(root, path)) as f:
+            assert re.search(rf"^def {fn}\(", f.read(), re.M), entry.reference
+        source = inspect.getsource(entry.launch)
+        assert f'build.load("{entry.module}")' in source, name

@@ -794,3 +794,18 @@ def test_mfma_prefill_window_edge_and_far_key(hd):
                 assert close == inside, f"window {window}, query {p}, key {target}"
                 assert rel_err(got, want) <= 2 * tol(dtype), \
                     f"window {window}, query {p}, key {target}"
+
+
+def test_cast_and_poison_pages():
+    x = _rand((37, 101), torch.float32, 5, 3.0)
+    out = torch.empty((37, 101), dtype=torch.bfloat16, device=DEV)
+    _ops().cast(x.to(DEV), out)
+    assert torch.equal(out.cpu(), x.to(torch.bfloat16))           # nearest even, as torch rounds
+    back = torch.empty((37, 101), dtype=torch.float32, device=DEV)
+    _ops().cast(out, back)
+    assert torch.equal(back.cpu(), x.to(torch.bfloat16).float())  # widening is exact
+    for dtype in DTYPES:
+        pool = torch.ones((3, 9, 50), dtype=dtype, device=DEV)
+        _ops().poison_pages(pool, torch.tensor([7, 0, 4], dtype=torch.int32, device=DEV))
+        bad = torch.isnan(pool.float()).cpu()
+        assert bad[:, [0, 4, 7]].all() and not bad[:, [1, 2, 3, 5, 6, 8]].any()

@@ -143,3 +143,31 @@ def test_a_tied_head_reads_a_copy_in_the_kernels_order(tmp_path):
     got = np.concatenate(got)
     err = np.abs(got - ref).max(axis=1) / np.abs(ref).max()
     assert err.max() <= 2e-2, f"first wrong position {int(np.argmax(err > 2e-2))}: {err.max():.3g}"
+
+
+@pytest.mark.parametrize("dtype,tolerance", [("float32", 2e-5), ("bfloat16", 2e-2)])
+def test_thirty_six_layers_against_the_plain_model(dtype, tolerance, tmp_path):
+    """The depth of the served models at tiny widths: a whole prompt, then decode steps, with
+    the tolerances of the shallow configurations (rounding must not pile up layer by layer)."""
+    from zinfer_amd.config import Qwen3Config
+    from zinfer_amd.engine import StepEntry
+    from zinfer_amd.engine.replay import make_engine
+    from zinfer_amd.models.build import declare_tensors
+    from zinfer_amd.weights import draw_tensors, write_model_dir
+    raw = dict(tiny.TINY_D, num_hidden_layers=36, hidden_size=256, num_attention_heads=4,
+               num_key_value_heads=2, head_dim=64, intermediate_size=768, vocab_size=1024,
+               tie_word_embeddings=False)
+    cfg = Qwen3Config.from_dict(raw)
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    path = write_model_dir(str(tmp_path / "deep"), cfg, 5, store, device=DEV)
+    w = {k: v.cpu() for k, v in draw_tensors(declare_tensors(cfg.model_spec()), 5, store,
+                                             device=DEV).items()}
+    toks = tiny.random_tokens(96, raw["vocab_size"], 3)
+    ref = plain.model_forward_batched(raw, w, toks).numpy()
+    eng = make_engine(path, dtype, 128, DEV)
+    got = [eng.step([StepEntry("r", toks[:80], list(range(80)))]).cpu().numpy()]
+    for t in range(80, 96):
+        got.append(eng.step([StepEntry("r", toks[t:t + 1], [0])]).cpu().numpy())
+    got = np.concatenate(got)
+    err = np.abs(got - ref).max(axis=1) / np.abs(ref).max()
+    assert err.max() <= tolerance, f"position {int(err.argmax())}: {err.max():.3g}"

@@ -226,9 +226,15 @@ class CacheManager:
         if not pages:
             return
         if self.poison_freed:
-            idx = torch.tensor(pages, dtype=torch.long, device=self.device)
-            grp.k[:, idx] = float("nan")
-            grp.v[:, idx] = float("nan")
+            if grp.k.is_cuda:
+                from .. import ops
+                idx = torch.tensor(pages, dtype=torch.int32, device=self.device)
+                ops.poison_pages(grp.k, idx)
+                ops.poison_pages(grp.v, idx)
+            else:
+                idx = torch.tensor(pages, dtype=torch.long, device=self.device)
+                grp.k[:, idx] = float("nan")
+                grp.v[:, idx] = float("nan")
         grp.pages.free(reversed(pages))
 
     def table(self, group: int, rid) -> List[int]:

@@ -407,6 +407,56 @@ extern "C" int zf_swiglu(const void* gu, void* out, int dtype, int T, int I,
   ZF_CHECK_LAUNCH();
 }
 
+// ---------------------------------------------------------------- cast and poison
+// out[i] = in[i] in the other storage type (bfloat16 -> float32 is exact, float32 -> bfloat16
+// rounds to nearest even): weights stored in one type for a build in the other are converted
+// on the device after the upload.
+template <typename TI, typename TO>
+__global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, size_t n) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+    store_from_float<TO>(out + i, load_as_float<TI>(in + i));
+}
+
+extern "C" int zf_cast(const void* in, int in_dtype, void* out, int out_dtype, long long n,
+                       hipStream_t stream) {
+  if (n <= 0) return 0;
+  long long blocks = (n + 256 * 8 - 1) / (256 * 8);
+  if (blocks > 65536) blocks = 65536;
+  const dim3 grid((unsigned)blocks), block(256);
+  if (in_dtype == ZF_BF16 && out_dtype == ZF_F32)
+    hipLaunchKernelGGL((cast_kernel<bf16_t, float>), grid, block, 0, stream, (const bf16_t*)in,
+                       (float*)out, (size_t)n);
+  else if (in_dtype == ZF_F32 && out_dtype == ZF_BF16)
+    hipLaunchKernelGGL((cast_kernel<float, bf16_t>), grid, block, 0, stream, (const float*)in,
+                       (bf16_t*)out, (size_t)n);
+  else
+    return 1;
+  ZF_CHECK_LAUNCH();
+}
+
+// pool[run, pages[i], :] = NaN for every run and listed page: pages that were given back hold
+// nothing that may be read again, and a test that poisons them finds a kernel that does.
+template <typename T>
+__global__ void poison_pages_kernel(T* __restrict__ pool, const int* __restrict__ pages,
+                                    size_t row, size_t pages_in_pool) {
+  T* dst = pool + ((size_t)blockIdx.y * pages_in_pool + pages[blockIdx.x]) * row;
+  for (size_t i = threadIdx.x; i < row; i += blockDim.x) store_from_float<T>(dst + i, NAN);
+}
+
+extern "C" int zf_poison_pages(void* pool, int dtype, const int* pages, int n_pages, int runs,
+                               long long pages_in_pool, long long row, hipStream_t stream) {
+  if (n_pages <= 0 || runs <= 0 || row <= 0) return 0;
+  const dim3 grid(n_pages, runs), block(256);
+  if (dtype == ZF_F32)
+    hipLaunchKernelGGL(poison_pages_kernel<float>, grid, block, 0, stream, (float*)pool, pages,
+                       (size_t)row, (size_t)pages_in_pool);
+  else
+    hipLaunchKernelGGL(poison_pages_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)pool, pages,
+                       (size_t)row, (size_t)pages_in_pool);
+  ZF_CHECK_LAUNCH();
+}
+
 // ---------------------------------------------------------------- out[r,:] = x[idx[r],:]
 __global__ void gather_rows_kernel(const float* __restrict__ x, const int* __restrict__ idx,
                                    float* __restrict__ out, int H) {

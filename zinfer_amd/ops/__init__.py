@@ -145,6 +145,29 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     _check(lib.zf_swiglu(_ptr(gate_up), _ptr(out), _dt(out), T, I, _stream()), "swiglu")
 
 
+def cast(src: torch.Tensor, out: torch.Tensor) -> None:
+    """out = src in the other storage type (bfloat16 <-> float32), element by element."""
+    _need_gpu(src, out)
+    if src.shape != out.shape or src.dtype == out.dtype:
+        raise KernelUnavailable(f"cast: {tuple(src.shape)} {src.dtype} -> {tuple(out.shape)} "
+                                f"{out.dtype}")
+    lib = build.load("elementwise")
+    _check(lib.zf_cast(_ptr(src), _dt(src), _ptr(out), _dt(out), ctypes.c_longlong(src.numel()),
+                       _stream()), "cast")
+
+
+def poison_pages(pool: torch.Tensor, pages: torch.Tensor) -> None:
+    """pool[:, pages, :] = NaN: ``pool`` [runs, pages, row] float32 or bfloat16, ``pages`` int32."""
+    _need_gpu(pool, pages)
+    _i32(pages, "pages")
+    if pool.dim() != 3 or pages.dim() != 1:
+        raise KernelUnavailable("poison_pages: a pool [runs, pages, row] and a list of pages")
+    lib = build.load("elementwise")
+    _check(lib.zf_poison_pages(_ptr(pool), _dt(pool), _ptr(pages), pages.shape[0], pool.shape[0],
+                               ctypes.c_longlong(pool.shape[1]), ctypes.c_longlong(pool.shape[2]),
+                               _stream()), "poison_pages")
+
+
 def gather_rows(x: torch.Tensor, idx: torch.Tensor, out: torch.Tensor) -> None:
     _need_gpu(x, idx, out)
     _i32(idx, "idx")
@@ -300,31 +323,43 @@ def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = Fals
                   K: int = 0) -> int:
     """Which tiled kernel: with pre-tiled weights the kernels that take W straight from
     memory (10: 128 x 256 tiles, two workgroups to a CU, when they fill the chip; else 128 x
-    128 tiles, 16: with the waves side by side and k-tiles of 128 when there are few of them,
-    6: with 2 x 2 waves); otherwise the kernels that stage both operands through LDS (4: 256
-    x 256 when they still fill the chip, else 0: 128 x 128).  Measured on MI355X at the
-    Qwen3-8B sizes."""
+    128 tiles, 16: with the waves side by side and k-tiles of 128 for a long K, 6: with
+    2 x 2 waves); otherwise the kernels that stage both operands through LDS (4: 256 x 256
+    when they still fill the chip, else 0: 128 x 128).  Measured on MI355X at the Qwen3-8B and
+    Qwen3-14B sizes."""
     if w_tiled:
-        tiles = ((M + 127) // 128) * ((N + 255) // 256)
+        tiles_m = (M + 127) // 128
+        tiles = tiles_m * ((N + 255) // 256)
         # between one and two 128 x 256 tiles per CU half the CUs hold two workgroups and half
-        # one, and the smaller tiles finish sooner (2048 tokens into 6144 outputs)
-        if tiles >= 192 and not 256 < tiles < 512:
+        # one, and the smaller tiles finish sooner (2048 tokens into 6144 outputs); with few
+        # tiles along the tokens (512 tokens into 24576 outputs) the large tiles still win
+        if tiles >= 160 and not (256 < tiles < 512 and tiles_m > 4):
             return 10
-        small = ((M + 127) // 128) * ((N + 127) // 128)
-        return 16 if small < 256 and K > 0 and K % 128 == 0 else 6
+        return 16 if K >= 8192 and K % 128 == 0 else 6
     tiles = ((M + 255) // 256) * ((N + 255) // 256)
     return 4 if tiles >= 160 else 0
 
 
 def _tile_ksplit(M: int, N: int, K: int) -> int:
     """Workgroups per 128 x 128 tile along K: products of a few hundred tokens on a narrow
-    output have too few tiles for 256 CUs; split them until about 256 workgroups run, each
-    keeping at least 8 k-tiles of 64.  The partials cost ksplit * M * N floats of traffic."""
+    output have too few tiles for 256 CUs, or a number that fills them unevenly (160 tiles:
+    96 CUs idle; 320: a second round for a quarter of them).  Two workgroups fit a CU, so the
+    split is chosen to fill 256 or a multiple of 512 places as evenly as it can, each
+    workgroup keeping at least 8 k-tiles of 64.  Every split costs partials of M * N floats,
+    written and read again (against the product's own time that is about 400 / K a split),
+    and the first one a second launch.  Measured on MI355X at the Qwen3-8B and Qwen3-14B
+    sizes, 256 to 1024 tokens."""
     tiles = ((M + 127) // 128) * ((N + 127) // 128)
-    if tiles >= 192:
+    if tiles >= 384:
         return 1
-    ksplit = min(256 // tiles, K // 64 // 8, 16)
-    return ksplit if ksplit >= 2 else 1
+    best, best_cost = 1, None
+    for ks in range(1, min(8, K // 64 // 8) + 1):
+        wgs = tiles * ks
+        places = 256 if wgs <= 256 else (wgs + 511) // 512 * 512
+        cost = places / wgs + (ks * 400.0 / K + 0.05 if ks > 1 else 0.0)
+        if best_cost is None or cost < best_cost - 1e-9:
+            best, best_cost = ks, cost
+    return best
 
 
 def can_pretile(w: torch.Tensor) -> bool:

@@ -59,6 +59,14 @@ class Linear:
 def place_matrix(t: torch.Tensor, ctx) -> torch.Tensor:
     """A matrix on the device: bfloat16 stays bfloat16 under a bfloat16 build, a tensor
     stored in 32-bit stays so; a float32 build widens everything."""
+    if ctx.compute_dtype == torch.float32 and t.dtype == torch.bfloat16 \
+            and torch.device(ctx.device).type == "cuda":
+        # half the bytes go over the bus; the widening (exact) runs on the device
+        from .. import ops
+        src = t.to(ctx.device).contiguous()
+        out = torch.empty(src.shape, dtype=torch.float32, device=src.device)
+        ops.cast(src, out)
+        return out
     if ctx.compute_dtype == torch.float32:
         t = t.to(torch.float32)
     elif t.dtype not in (torch.bfloat16, torch.float32):
