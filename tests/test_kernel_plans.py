@@ -83,3 +83,42 @@ def test_the_flat_kernel_table_is_complete_and_its_references_exist():
             assert re.search(rf"^def {fn}\(", f.read(), re.M), entry.reference
         source = inspect.getsource(entry.launch)
         assert f'build.load("{entry.module}")' in source, name
+
+
+def test_measured_plans_are_plans_the_kernels_take():
+    """Every entry of the measured table names a kernel configuration that exists: row groups
+    of 1, 2 or 4 that divide the outputs, splits that leave each workgroup k-tiles, the
+    SwiGLU products unsplit and with whole gate/up pairs."""
+    plans = ops._measured_plans()
+    for key, entry in plans["plans"].items():
+        shape, _, kind = key.partition(":")
+        N, K = (int(x) for x in shape.split("x"))
+        for bucket, plan in entry.items():
+            M = int(bucket)
+            assert 16 < M <= 64
+            if plan[0] == "mid":
+                ks = plan[1]
+                assert K % ((256 if M <= 32 else 128) * ks) == 0 and N % 16 == 0
+            else:
+                assert plan[0] == "skinny"
+                rg, ks = plan[1:]
+                assert rg in (1, 2, 4) and N % (16 * rg) == 0 and 1 <= ks <= 16 and K % 64 == 0
+            if kind == "swiglu":
+                assert plan[-1] == 1 and (plan[0] == "mid" or plan[1] >= 2) and N % 32 == 0
+            for m in range(17, 65):
+                got = ops._small_plan(m, N, K, True, swiglu=(kind == "swiglu"))
+                assert got is not None and got[0] in ("mid", "skinny")
+                if got[0] == "mid":
+                    assert K % ((256 if m <= 32 else 128) * got[1]) == 0
+    for key, plan in plans["decode_acc"].items():
+        if key == "_":
+            continue
+        N, K = (int(x) for x in key.split("x"))
+        assert plan[0] == "skinny" and plan[1] in (1, 2, 4) and N % (16 * plan[1]) == 0
+        assert 2 <= plan[2] <= 16 and N <= 8192
+        assert ops._decode_acc_plan(8, N, K) == tuple(plan) and ops._decode_acc_plan(17, N, K) is None
+    # widths without an entry follow the rules
+    assert ops._small_plan(40, 4160, 1088, True) is not None
+    assert ops._skinny_plan(8, 5120, 5120, True) == (2, 1) and ops._skinny_plan(8, 4096, 4096, True) == (1, 1)
+    assert ops._skinny_plan(8, 10240, 5120, True) == (4, 1) and ops._skinny_plan(8, 6144, 4096, True) == (2, 1)
+    assert ops._skinny_plan(1, 151936, 4096, True) == (2, 1)

@@ -1110,7 +1110,8 @@ extern "C" int zf_gemm_bf16_splitk_sum_norm(const void* A, const void* W, void* 
 
 template <int MT, int RG, bool WT, int NORM = NORM_NONE, bool EMIT = false>
 static int launch_skinny(const void* A, const void* W, void* C, void* ws, int M, int N, int K,
-                         int epi, int ksplit, hipStream_t stream, SkinnyNorm nrm = SkinnyNorm{}) {
+                         int epi, int ksplit, hipStream_t stream, SkinnyNorm nrm = SkinnyNorm{},
+                         bool reduce = true) {
   constexpr int NW = 8;
   const dim3 grid((N + 16 * RG - 1) / (16 * RG), ksplit), block(NW * 64);
   void* dst = ksplit > 1 ? ws : C;
@@ -1136,7 +1137,35 @@ static int launch_skinny(const void* A, const void* W, void* C, void* ws, int M,
   else
     hipLaunchKernelGGL((gemm_bf16_skinny_kernel<MT, RG, EPI_ACC_F32, WT, NORM_NONE, NW>), grid, block, 0,
                        stream, (const bf16_t*)A, (const bf16_t*)W, dst, M, N, K, nrm);
-  if (ksplit > 1) return launch_reduce(ws, C, M, N, ksplit, epi, stream);
+  if (ksplit > 1 && reduce) return launch_reduce(ws, C, M, N, ksplit, epi, stream);
+  return (int)hipGetLastError();
+}
+
+// C += A W^T in 32-bit by the weight-streaming kernel with ksplit >= 2 workgroups along K, and
+// normed = bfloat16 RMSNorm of the sum's rows from the kernel that adds the partials: for
+// narrow outputs whose row groups alone leave CUs idle (320 of them on 256 CUs).  M <= 64,
+// W pre-tiled, N a multiple of 16 * rg; ws: float32 [ksplit, M, N].
+extern "C" int zf_gemm_bf16_skinny_sum_norm(const void* A, const void* W, void* C, void* ws,
+                                            const float* gain, float eps, void* normed, int M,
+                                            int N, int K, int rg, int ksplit,
+                                            hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || ksplit < 2 || ksplit > 16 || K % 64 != 0 || N % (16 * rg) != 0 || N > 8192 ||
+      ws == nullptr)
+    return -3;
+  const int mt = (M + 15) / 16;
+  int rc = -4;
+#define ZF_SKS(MT, RG)                                                                         \
+  rc = launch_skinny<MT, RG, true>(A, W, C, ws, M, N, K, EPI_ACC_F32, ksplit, stream,          \
+                                   SkinnyNorm{}, false)
+  if (rg == 1) { if (mt == 1) ZF_SKS(1, 1); else if (mt == 2) ZF_SKS(2, 1); else if (mt == 3) ZF_SKS(3, 1); else ZF_SKS(4, 1); }
+  if (rg == 2) { if (mt == 1) ZF_SKS(1, 2); else if (mt == 2) ZF_SKS(2, 2); else if (mt == 3) ZF_SKS(3, 2); else ZF_SKS(4, 2); }
+  if (rg == 4) { if (mt == 1) ZF_SKS(1, 4); else if (mt == 2) ZF_SKS(2, 4); else if (mt == 3) ZF_SKS(3, 4); else ZF_SKS(4, 4); }
+#undef ZF_SKS
+  if (rc != 0) return rc;
+  const int threads = N / 4 >= 1024 ? 1024 : (N / 4 > 256 ? 512 : 256);
+  hipLaunchKernelGGL(reduce_sum_norm_kernel, dim3(M), dim3(threads), 0, stream, (const float*)ws,
+                     (float*)C, gain, (bf16_t*)normed, M, N, ksplit, eps);
   return (int)hipGetLastError();
 }
 

@@ -53,7 +53,7 @@ class Engine:
         self.views = [self.cache.view(pos) for pos in range(len(spec.schedule))]
         self.page_size = page_size
         self._scratch = Scratch(self.device)
-        self._meta_host: Optional[torch.Tensor] = None
+        self._meta_host = None          # two pinned buffers that take turns
         self._meta_dev: Optional[torch.Tensor] = None
         self._meta_generation = 0
         self.steps_run = 0
@@ -400,16 +400,29 @@ class Engine:
             _scratch=self._scratch)
 
     def _upload(self, host: np.ndarray) -> torch.Tensor:
+        """The packed metadata on the device.  Two pinned host buffers take turns, each with an
+        event that says when its last copy has left it, so that packing a step never waits
+        for the stream: the copy of the step before last is long done.  (The device buffer is
+        one: its copy is queued on the stream behind the kernels that read the old contents.)"""
         n = host.shape[0]
         if self.device.type == "cpu":
             return torch.from_numpy(host.copy())
-        if self._meta_host is None or self._meta_host.numel() < n:
+        if self._meta_dev is None or self._meta_dev.numel() < n:
             cap = max(n * 2, 1 << 18)
-            self._meta_host = torch.empty((cap,), dtype=torch.int32, pin_memory=True)
+            self._meta_host = [torch.empty((cap,), dtype=torch.int32, pin_memory=True)
+                               for _ in range(2)]
+            self._meta_events = [None, None]
+            self._meta_turn = 0
             self._meta_dev = torch.empty((cap,), dtype=torch.int32, device=self.device)
             self._meta_generation += 1
-        # the previous step's copy must have left the pinned buffer before it is rewritten
-        torch.cuda.current_stream(self.device).synchronize()
-        self._meta_host[:n].numpy()[:] = host
-        self._meta_dev[:n].copy_(self._meta_host[:n], non_blocking=True)
+        turn = self._meta_turn
+        self._meta_turn = 1 - turn
+        if self._meta_events[turn] is not None:
+            self._meta_events[turn].synchronize()
+        pinned = self._meta_host[turn]
+        pinned[:n].numpy()[:] = host
+        self._meta_dev[:n].copy_(pinned[:n], non_blocking=True)
+        event = torch.cuda.Event()
+        event.record(torch.cuda.current_stream(self.device))
+        self._meta_events[turn] = event
         return self._meta_dev[:n]

@@ -282,6 +282,12 @@ def _skinny_plan(M: int, N: int, K: int, tiled: bool):
     are re-read once per workgroup).  Measured on MI355X at the Qwen3-8B sizes."""
     if tiled:
         if M <= 16:
+            # one workgroup per CU streams best: the fewest row groups per workgroup that
+            # still leave at most 256 workgroups, if that keeps half the CUs busy (384 row
+            # groups: 192 workgroups of 2; 320: 160 of 2; 640: 160 of 4); a wide output takes 2
+            for rg in (1, 2, 4):
+                if N % (16 * rg) == 0 and 128 <= N // (16 * rg) <= 256:
+                    return rg, 1
             return (2 if N >= 6144 else 1), 1
         if N >= 16384:
             return 4, 1
@@ -317,6 +323,54 @@ def _mid_plan(M: int, N: int, K: int, w_tiled: bool, swiglu: bool = False):
         return 1
     tiles = (N + 127) // 128
     return max(1, min(256 // tiles, K // 1024))
+
+
+_measured = None
+
+
+def _measured_plans() -> dict:
+    global _measured
+    if _measured is None:
+        import json
+        import os
+        with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "plans_mi355x.json")) as f:
+            _measured = json.load(f)
+    return _measured
+
+
+def _small_plan(M: int, N: int, K: int, w_tiled: bool, swiglu: bool = False):
+    """Which kernel takes a product of 17 to 128 tokens (None: the tiled kernels):
+    ('mid', workgroups along K) or ('skinny', row groups per workgroup, workgroups along K).
+    The widths of the served models have measured entries in ``plans_mi355x.json``; other
+    widths follow the rules of ``_mid_plan`` and ``_skinny_plan``."""
+    if w_tiled and 16 < M <= SKINNY_MAX_M:
+        bucket = 17 if M <= 20 else 24 if M <= 28 else 32 if M <= 32 else 48 if M <= 56 else 64
+        entry = _measured_plans()["plans"].get(f"{N}x{K}" + (":swiglu" if swiglu else ""))
+        if entry is not None:
+            # a width measured at fewer numbers of tokens: the nearest one on the same side of
+            # 32 tokens (the kernels change there)
+            same = [int(b) for b in entry if (int(b) <= 32) == (bucket <= 32)]
+            if same:
+                plan = entry[str(min(same, key=lambda b: abs(b - bucket)))]
+                return tuple(plan)
+    mid = _mid_plan(M, N, K, w_tiled, swiglu)
+    if mid is not None:
+        return ("mid", mid)
+    if M <= SKINNY_MAX_M:
+        if swiglu:
+            return ("skinny", 4 if (M > 16 and N >= 16384) else 2, 1)
+        return ("skinny",) + tuple(_skinny_plan(M, N, K, w_tiled))
+    return None
+
+
+def _decode_acc_plan(M: int, N: int, K: int):
+    """('skinny', row groups, workgroups along K) if, at 1 to 16 tokens, a residual sum that an
+    RMSNorm follows is measured to run faster split along K (the reduce adds the residual and
+    norms) than with the one-launch epilogue; else None."""
+    if not 0 < M <= NORM_FOLD_MAX_M:
+        return None
+    plan = _measured_plans()["decode_acc"].get(f"{N}x{K}")
+    return tuple(plan) if plan is not None else None
 
 
 def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = False,
@@ -403,13 +457,14 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and K % 8 == 0 and M > 0:
         epi = _EPI_ACC_F32 if accumulate else \
             (_EPI_STORE_BF16 if out.dtype == torch.bfloat16 else _EPI_STORE_F32)
-        mid = _mid_plan(M, N, K, w_tiled)
-        if mid is not None:
+        plan = _small_plan(M, N, K, w_tiled) if M > 16 else None
+        if plan is not None and plan[0] == "mid":
+            mid = plan[1]
             ws = _workspace("gemm_splitk", mid * M * N, torch.float32, a.device) if mid > 1 else None
             _check(lib.zf_gemm_bf16_mid(_ptr(a), _ptr(w), _ptr(out), _ptr(ws), M, N, K, epi, mid,
                                         _stream()), "gemm (17 to 128 tokens)")
         elif M <= SKINNY_MAX_M:
-            rg, ks = _skinny_plan(M, N, K, w_tiled)
+            rg, ks = plan[1:] if plan is not None else _skinny_plan(M, N, K, w_tiled)
             ws = _workspace("gemm_splitk", ks * M * N, torch.float32, a.device) if ks > 1 else None
             _check(lib.zf_gemm_bf16_skinny(_ptr(a), _ptr(w), _ptr(out), _ptr(ws), M, N, K, epi,
                                            rg, ks, 1 if w_tiled else 0, _stream()),
@@ -468,15 +523,19 @@ def norm_gemm(x: torch.Tensor, gain: torch.Tensor, eps: float, w: torch.Tensor,
 
 
 def sum_norm_plan(M: int, N: int, K: int, w: torch.Tensor, w_tiled: bool):
-    """Workgroups along K if ``gemm_sum_norm`` covers residual += a w^T: a product that is
-    split along K anyway (17 to 128 tokens, or a few hundred tokens on a narrow output), whose
-    partials one kernel can add, sum into the residual and norm; else None."""
+    """The plan if ``gemm_sum_norm`` covers residual += a w^T: a product that is split along K
+    anyway (by measurement at 1 to 64 tokens, by rule at 17 to 128, or a few hundred tokens on
+    a narrow output), whose partials one kernel can add, sum into the residual and norm; else
+    None.  ('mid' | 'tile' | 'skinny', [row groups per workgroup,] workgroups along K)."""
     if not (w_tiled and w.dtype == torch.bfloat16 and w.is_cuda and N % 16 == 0 and N <= 8192):
         return None
-    ks = _mid_plan(M, N, K, True) if M <= MID_MAX_M else None
-    if ks is None and M > SKINNY_MAX_M:
-        ks = _tile_ksplit(M, N, K)
-    return ks if ks is not None and ks >= 2 else None
+    if M <= NORM_FOLD_MAX_M:
+        return _decode_acc_plan(M, N, K)
+    if M <= MID_MAX_M:
+        plan = _small_plan(M, N, K, True)
+        return plan if plan is not None and plan[-1] >= 2 else None
+    ks = _tile_ksplit(M, N, K)
+    return ("tile", ks) if ks >= 2 else None
 
 
 def gemm_sum_norm(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, gain: torch.Tensor,
@@ -486,8 +545,8 @@ def gemm_sum_norm(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, gain
     _need_gpu(a, w, residual, gain, normed)
     M, K = a.shape
     N = w.shape[0]
-    ks = sum_norm_plan(M, N, K, w, True)
-    if ks is None or a.dtype != torch.bfloat16 or w.shape[1] != K or not can_pretile(w) \
+    plan = sum_norm_plan(M, N, K, w, True)
+    if plan is None or a.dtype != torch.bfloat16 or w.shape[1] != K or not can_pretile(w) \
             or residual.shape != (M, N) or residual.dtype != torch.float32 \
             or gain.shape != (N,) or gain.dtype != torch.float32 \
             or normed.shape != (M, N) or normed.dtype != torch.bfloat16 \
@@ -495,11 +554,18 @@ def gemm_sum_norm(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, gain
         raise KernelUnavailable(f"gemm_sum_norm: a {tuple(a.shape)} {a.dtype}, w "
                                 f"{tuple(w.shape)}, residual {tuple(residual.shape)} "
                                 f"{residual.dtype}")
+    ks = plan[-1]
     ws = _workspace("gemm_splitk", ks * M * N, torch.float32, a.device)
     lib = build.load("gemm")
-    _check(lib.zf_gemm_bf16_splitk_sum_norm(_ptr(a), _ptr(w), _ptr(residual), _ptr(ws), _ptr(gain),
-                                            ctypes.c_float(eps), _ptr(normed), M, N, K, ks,
-                                            _stream()), "gemm_sum_norm")
+    if plan[0] == "skinny":
+        _check(lib.zf_gemm_bf16_skinny_sum_norm(_ptr(a), _ptr(w), _ptr(residual), _ptr(ws),
+                                                _ptr(gain), ctypes.c_float(eps), _ptr(normed), M, N,
+                                                K, plan[1], ks, _stream()),
+               "gemm_sum_norm (weight streaming)")
+    else:
+        _check(lib.zf_gemm_bf16_splitk_sum_norm(_ptr(a), _ptr(w), _ptr(residual), _ptr(ws),
+                                                _ptr(gain), ctypes.c_float(eps), _ptr(normed), M, N,
+                                                K, ks, _stream()), "gemm_sum_norm")
 
 
 def norm_emit_plan(M: int, N: int, K: int, w: torch.Tensor, w_tiled: bool):
@@ -507,6 +573,8 @@ def norm_emit_plan(M: int, N: int, K: int, w: torch.Tensor, w_tiled: bool):
     up to 16 tokens, pre-tiled bfloat16 weight, no split over workgroups), else None."""
     if not (w_tiled and 0 < M <= NORM_FOLD_MAX_M and w.dtype == torch.bfloat16 and w.is_cuda):
         return None
+    if N <= 8192 and _decode_acc_plan(M, N, K) is not None:
+        return None             # measured: the split along K with the norm in its reduce is faster
     rg, ks = _skinny_plan(M, N, K, True)
     return rg if (ks == 1 and rg <= 2) else None
 
@@ -586,11 +654,12 @@ def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bo
     if M == 0:
         return
     lib = build.load("gemm")
-    if _mid_plan(M, N, K, w_tiled, swiglu=True) is not None:
+    plan = _small_plan(M, N, K, w_tiled, swiglu=True) if M > 16 else None
+    if plan is not None and plan[0] == "mid":
         _check(lib.zf_gemm_bf16_mid(_ptr(a), _ptr(w), _ptr(out), _ptr(None), M, N, K, _EPI_SWIGLU,
                                     1, _stream()), "gemm_swiglu (17 to 128 tokens)")
     elif M <= SKINNY_MAX_M:
-        rg = 4 if (M > 16 and N >= 16384) else 2
+        rg = plan[1] if plan is not None else 2
         _check(lib.zf_gemm_bf16_skinny(_ptr(a), _ptr(w), _ptr(out), _ptr(None), M, N, K,
                                        _EPI_SWIGLU, rg, 1, 1 if w_tiled else 0, _stream()),
                "gemm_swiglu (weight streaming)")
