@@ -396,7 +396,7 @@ def _paged_setup(dtype, nH, nKV, hd, page_size, ctx_lens, q_lens, seed, num_page
                 seq_index=seq_index.int(), Ks=Ks, Vs=Vs)
 
 
-def _run_attention(s, dtype, nH, nKV, hd, page_size, window, q_lens, ctx_lens):
+def _run_attention(s, dtype, nH, nKV, hd, page_size, window, q_lens, ctx_lens, tiles_hint=False):
     scale = 1.0 / math.sqrt(hd)
     T = s["q"].shape[0]
     want = torch.empty((T, nH * hd), dtype=dtype)
@@ -412,8 +412,22 @@ def _run_attention(s, dtype, nH, nKV, hd, page_size, window, q_lens, ctx_lens):
     _ops().paged_attention(d["q"], d["k_pool"], d["v_pool"], d["block_table"], d["q_start"],
                            d["ctx_len"], d["seq_index"], got, scale, window, nH, nKV, hd,
                            page_size, max(q_lens), max(ctx_lens),
-                           n_single=sum(1 for n in q_lens if n == 1))
+                           n_single=sum(1 for n in q_lens if n == 1),
+                           **_tile_hints(q_lens, ctx_lens, tiles_hint))
     return got, want
+
+
+def _tile_hints(q_lens, ctx_lens, on):
+    """What the engine passes with a step: the query tiles of the sequences with more than one
+    token (heaviest first) and those sequences' longest context."""
+    if not on:
+        return {}
+    tiles = [(c - n + min(32 * (t + 1), n), i, t) for i, (n, c) in enumerate(zip(q_lens, ctx_lens))
+             if n > 1 for t in range((n + 31) // 32)]
+    tiles.sort(key=lambda x: -x[0])
+    tmap = torch.tensor([(i, t) for _, i, t in tiles], dtype=torch.int32, device=DEV).view(-1, 2)
+    return dict(n_query_tiles=len(tiles), q_tile_map=tmap if tiles else None,
+                prefill_max_ctx=max((c for c, n in zip(ctx_lens, q_lens) if n > 1), default=None))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -457,6 +471,11 @@ def test_paged_attention_mfma(nH, nKV, hd, page_size, window, kind):
     got, want = _run_attention(s, dtype, nH, nKV, hd, page_size, window, q_lens, ctx_lens)
     assert not torch.isnan(got.float()).any(), "a slot outside the context was read"
     assert rel_err(got, want) <= 2 * tol(dtype)     # probabilities are rounded once more
+    # with the engine's hints (the list of query tiles that exist, heaviest first)
+    got, want = _run_attention(s, dtype, nH, nKV, hd, page_size, window, q_lens, ctx_lens,
+                               tiles_hint=True)
+    assert not torch.isnan(got.float()).any(), "a slot outside the context was read"
+    assert rel_err(got, want) <= 2 * tol(dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -818,3 +837,37 @@ def test_cast_and_poison_pages():
         _ops().poison_pages(pool, torch.tensor([7, 0, 4], dtype=torch.int32, device=DEV))
         bad = torch.isnan(pool.float()).cpu()
         assert bad[:, [0, 4, 7]].all() and not bad[:, [1, 2, 3, 5, 6, 8]].any()
+
+
+@pytest.mark.parametrize("nH,nKV,hd,window", [(10, 2, 128, 0), (8, 1, 64, 0), (4, 1, 128, 0),
+                                              (10, 2, 128, 700), (6, 2, 64, 33)])
+def test_prefill_attention_splits_keys_over_workgroups(nH, nKV, hd, window):
+    """Portions behind long contexts, few query tiles: the keys are split over workgroups and
+    a second kernel merges the partials.  Portions that start at 0, mid-page and at a split's
+    edge, a short prompt whose keys lie in one split, single tokens beside them; and a key
+    that stands out at a split's last and first position."""
+    dtype, ps = torch.bfloat16, 16
+    ops = _ops()
+    ctx_lens = [2300, 1024 + 40, 70, 1500, 1]
+    q_lens = [100, 40, 70, 33, 1]
+    tiles = sum((n + 31) // 32 for n in q_lens if n > 1)
+    split = ops._prefill_key_split(tiles, nKV, max(ctx_lens))
+    assert split is not None and split[1] >= 2
+    s = _paged_setup(dtype, nH, nKV, hd, ps, ctx_lens, q_lens, seed=31)
+    got, want = _run_attention(s, dtype, nH, nKV, hd, ps, window, q_lens, ctx_lens, tiles_hint=True)
+    assert not torch.isnan(got.float()).any(), "a slot outside the context was read"
+    assert rel_err(got, want) <= 2 * tol(dtype)
+    # the same without the hint (one workgroup walks all keys): equal up to rounding
+    plain, _ = _run_attention(s, dtype, nH, nKV, hd, ps, window, q_lens, ctx_lens)
+    assert rel_err(got, plain) <= 2 * tol(dtype)
+    if window == 0:
+        keys = split[0]
+        for target in (keys - 1, keys, 2 * keys - 1, 0):
+            s = _paged_setup(dtype, nH, nKV, hd, ps, ctx_lens, q_lens, seed=32)
+            row = 57                     # a query of the first sequence (position 2257)
+            _stand_out(s, nKV, ps, hd, 0, target, row, nH - 1, dtype, nH)
+            got, want = _run_attention(s, dtype, nH, nKV, hd, ps, 0, q_lens, ctx_lens,
+                                       tiles_hint=True)
+            v_row = s["Vs"][0][target, (nH - 1) // (nH // nKV)].float()
+            assert torch.allclose(got.cpu().float()[row, (nH - 1) * hd:nH * hd], v_row, atol=3e-2), target
+            assert rel_err(got, want) <= 2 * tol(dtype)

@@ -437,16 +437,20 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
     const bf16_t* __restrict__ v_pool, const int* __restrict__ block_table,
     const int* __restrict__ q_start, const int* __restrict__ ctx_len, bf16_t* __restrict__ out,
     float scale_log2e, int window, int nH, int nKV, int ps, int max_pages, int skip_single,
-    int q_tiles, int nsplit, int ps_shift) {
+    int q_tiles, int nsplit, int ps_shift, float* __restrict__ ws_o, float* __restrict__ ws_ml,
+    int split_keys, int max_splits, const int* __restrict__ tile_map) {
   auto page_of = [&](int key) { return POW2 ? key >> ps_shift : key / ps; };
   auto row_of = [&](int key) { return POW2 ? key & (ps - 1) : key % ps; };
   extern __shared__ float xch[];      // partials of the waves that took other key tiles
   // workgroups are handed out in the order of blockIdx.x: kv heads vary fastest and the
   // last query tiles (the longest key ranges under the causal bound) come first, so the
   // heavy tiles do not end up as the tail
+  // (tile_map: the host lists the (sequence, query tile) pairs that exist, heaviest first,
+  // and the grid holds no workgroup for a single token or beyond a short portion's end)
   const int kvh = blockIdx.x % nKV;
-  const int qt = q_tiles - 1 - (blockIdx.x / nKV) % q_tiles;
-  const int s = blockIdx.x / (nKV * q_tiles);
+  const int qt = tile_map ? tile_map[2 * (blockIdx.x / nKV) + 1]
+                          : q_tiles - 1 - (blockIdx.x / nKV) % q_tiles;
+  const int s = tile_map ? tile_map[2 * (blockIdx.x / nKV)] : blockIdx.x / (nKV * q_tiles);
   const int q_len = q_start[s + 1] - q_start[s];
   if (q_len == 1 && skip_single) return;
   const int qbase = qt * 32;
@@ -467,6 +471,13 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
   const int lo_top = (window > 0 && p_max - window + 1 > 0) ? p_max - window + 1 : 0;
   const int* table = block_table + (size_t)s * max_pages;
   const int t_row = q_start[s] + qbase + min(j, nq - 1);
+  // gridDim.y > 1: the keys are also split over workgroups, blockIdx.y taking the keys
+  // [split_keys * y, split_keys * (y + 1)) (a multiple of 32, so no tile lies across an edge);
+  // each writes un-normalised partials that attn_prefill_merge_kernel combines.  For portions
+  // behind a long context, whose few query tiles would otherwise walk thousands of keys each.
+  const int k_lo = gridDim.y > 1 ? max(lo_min, (int)blockIdx.y * split_keys) : lo_min;
+  const int k_hi = gridDim.y > 1 ? min(p_max, ((int)blockIdx.y + 1) * split_keys - 1) : p_max;
+  if (k_lo > k_hi) return;
 
   // With few query heads per kv head the waves also split the key tiles of a head between
   // them (wave `split` takes tiles split, split + nsplit, ...): under the causal bound the
@@ -505,7 +516,7 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
       for (int stp = 0; stp < HD / 16; ++stp)
         dst[stp] = *(const u32x4_t*)(kblk + (stp / 2) * 512 + (stp % 2) * 256);
     };
-    const int kb0 = (lo_min / 32) * 32 + 32 * split, kstep = 32 * nsplit;
+    const int kb0 = (k_lo / 32) * 32 + 32 * split, kstep = 32 * nsplit;
     u32x4_t kf[HD / 16];
     load_keys(kb0, kf);
     // values of a tile: keys kb + 16 u .. + 15 (one page) for u = 0, 1, into one of two
@@ -617,9 +628,9 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
       }
     };
     load_vals(kb0, Buf0{});
-    for (int kb = kb0; kb <= p_max; kb += 2 * kstep) {
+    for (int kb = kb0; kb <= k_hi; kb += 2 * kstep) {
       tile(kb, Buf0{}, Buf1{});
-      if (kb + kstep <= p_max) tile(kb + kstep, Buf1{}, Buf0{});
+      if (kb + kstep <= k_hi) tile(kb + kstep, Buf1{}, Buf0{});
       else load_vals(kb + 2 * kstep, Buf0{});     // keeps the register sets in step (unused)
     }
     if (nsplit > 1) {     // one pass over g here: every wave comes by exactly once
@@ -649,6 +660,24 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
           for (int r = 0; r < 16; ++r) o[dt][r] = o[dt][r] * ca + src[(dt * 16 + r) * 64] * cb;
       }
     }
+    if (gridDim.y > 1) {
+      // this split's partial for (token, head): O^T un-normalised, running maximum and sum
+      if (q_valid) {
+        const size_t slot = ((size_t)t_row * nH + head) * max_splits + blockIdx.y;
+        float* dst = ws_o + slot * HD;
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+          for (int r4 = 0; r4 < 4; ++r4)
+            *(f32x4_t*)(dst + dt * 32 + 8 * r4 + 4 * hf) =
+                f32x4_t{o[dt][r4 * 4 + 0], o[dt][r4 * 4 + 1], o[dt][r4 * 4 + 2], o[dt][r4 * 4 + 3]};
+        if (hf == 0) {
+          ws_ml[slot * 2] = m;
+          ws_ml[slot * 2 + 1] = l;
+        }
+      }
+      continue;
+    }
     if (q_valid) {
       const float inv = 1.0f / l;
       bf16_t* orow = out + ((size_t)t_row * nH + head) * HD;
@@ -665,23 +694,75 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
   }
 }
 
+// Combines the key splits of one (token, head) of a prompt portion in split order and writes
+// bfloat16: token t of sequence s = seq_index[t] sits at position ctx_len[s] - q_len + (t -
+// q_start[s]) and has partials from the splits that hold its keys lo .. position.
+__global__ __launch_bounds__(64) void attn_prefill_merge_kernel(
+    const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+    const int* __restrict__ q_start, const int* __restrict__ ctx_len,
+    const int* __restrict__ seq_index, bf16_t* __restrict__ out, int window, int nH, int hd,
+    int split_keys, int max_splits, int skip_single) {
+  const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const int s = seq_index[t];
+  const int q_len = q_start[s + 1] - q_start[s];
+  if (q_len == 1 && skip_single) return;
+  const int pos = ctx_len[s] - q_len + (t - q_start[s]);
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int first = lo / split_keys, last = pos / split_keys;
+  const size_t base = ((size_t)t * nH + head) * max_splits;
+  float mx = -INFINITY;
+  for (int sp = first; sp <= last; ++sp) mx = fmaxf(mx, ws_ml[(base + sp) * 2]);
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  float denom = 0.f;
+  for (int sp = first; sp <= last; ++sp) {
+    const float w = exp2f(ws_ml[(base + sp) * 2] - mx);
+    denom += w * ws_ml[(base + sp) * 2 + 1];
+    const float* src = ws_o + (base + sp) * hd;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int d = lane + 64 * i;
+      if (d < hd) acc[i] = fmaf(w, src[d], acc[i]);
+    }
+  }
+  const float inv = 1.0f / denom;
+  bf16_t* orow = out + ((size_t)t * nH + head) * hd;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int d = lane + 64 * i;
+    if (d < hd) orow[d] = float_to_bf16(acc[i] * inv);
+  }
+}
+
+// tile_map (or null): int32 pairs (sequence, query tile), n_tiles of them: the workgroups that
+// exist.  split_keys > 0 (a multiple of 32; ws_o: n_tokens * nH * max_splits * hd floats, ws_ml:
+// n_tokens * nH * max_splits * 2, max_splits >= ceil(longest context / split_keys)): the keys
+// are split over workgroups and merged by a second kernel.
 extern "C" int zf_attn_prefill_bf16(const void* q, const void* k_pool, const void* v_pool,
                                     const int* block_table, const int* q_start,
                                     const int* ctx_len, void* out, float scale, int window,
                                     int n_seqs, int max_q_len, int nH, int nKV, int hd,
                                     int page_size, int max_pages, int skip_single,
-                                    int allow_split, hipStream_t stream) {
+                                    int allow_split, const int* seq_index, int n_tokens,
+                                    float* ws_o, float* ws_ml, int split_keys, int max_splits,
+                                    const int* tile_map, int n_tiles, hipStream_t stream) {
   if (n_seqs <= 0 || max_q_len <= 0) return 0;
   if (page_size % 16 != 0 || nKV <= 0 || nH % nKV != 0) return -2;
+  if (split_keys > 0 && (split_keys % 32 != 0 || max_splits < 1 || ws_o == nullptr ||
+                         ws_ml == nullptr || seq_index == nullptr))
+    return -2;
   const float scale_log2e = scale * 1.4426950408889634f;
   const int G = nH / nKV;
   const int q_tiles = (max_q_len + 31) / 32;
-  dim3 grid((unsigned)n_seqs * q_tiles * nKV);
+  if (tile_map != nullptr && n_tiles <= 0) return 0;
+  dim3 grid((unsigned)(tile_map != nullptr ? n_tiles : n_seqs * q_tiles) * nKV,
+            split_keys > 0 ? max_splits : 1);
   // up to 8 waves: one per query head of the kv head, and with 4 heads or fewer several
   // waves per head that split its key tiles, as far as the partials fit into LDS
   // (allow_split: the caller expects short contexts before the portions, where the causal
   // bound leaves the tiles most unequal, and a grid that does not fill the chip many times)
-  int nsplit = (allow_split && G <= 4 && grid.x <= 1024) ? 8 / G : 1;
+  int nsplit = (allow_split && split_keys == 0 && G <= 4 && grid.x <= 1024) ? 8 / G : 1;
   const size_t per_wave = (size_t)(hd / 2 + 2) * 64 * sizeof(float);
   while (nsplit > 1 && (size_t)(nsplit - 1) * G * per_wave > 144 * 1024) --nsplit;
   const int head_waves = G < 8 ? G : 8;
@@ -700,7 +781,8 @@ extern "C" int zf_attn_prefill_bf16(const void* q, const void* k_pool, const voi
     hipLaunchKernelGGL(KERN, grid, block, smem, stream, (const bf16_t*)q,                       \
                        (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, q_start,      \
                        ctx_len, (bf16_t*)out, scale_log2e, window, nH, nKV, page_size,          \
-                       max_pages, skip_single, q_tiles, nsplit, ps_shift);                      \
+                       max_pages, skip_single, q_tiles, nsplit, ps_shift, ws_o, ws_ml,          \
+                       split_keys, max_splits, tile_map);                                       \
   } while (0)
 #define ZF_PRE(HD)                                                                              \
   do {                                                                                          \
@@ -714,5 +796,9 @@ extern "C" int zf_attn_prefill_bf16(const void* q, const void* k_pool, const voi
   else return -2;
 #undef ZF_PRE
 #undef ZF_PRE_K
+  if (split_keys > 0)
+    hipLaunchKernelGGL(attn_prefill_merge_kernel, dim3(n_tokens, nH), dim3(64), 0, stream, ws_o,
+                       ws_ml, q_start, ctx_len, seq_index, (bf16_t*)out, window, nH, hd, split_keys,
+                       max_splits, skip_single);
   ZF_CHECK_LAUNCH();
 }

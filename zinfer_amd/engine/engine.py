@@ -334,8 +334,15 @@ class Engine:
             max_ctx = max_pages * ps
 
         # one packed int32 buffer, one copy to the device
+        # the 32-token query tiles of the sequences that bring more than one token, those that
+        # read the most keys first
+        tiles = [(starts[i] + min(32 * (t + 1), q_lens[i]), i, t) for i in range(n_seqs)
+                 if q_lens[i] > 1 for t in range((q_lens[i] + 31) // 32)]
+        tiles.sort(key=lambda x: -x[0])
+        n_tiles = len(tiles)
         sizes = [("token_ids", T), ("positions", T), ("seq_index", T), ("q_start", n_seqs + 1),
-                 ("ctx_len", n_seqs), ("state_slots", n_seqs), ("want_rows", max(n_want, 1))]
+                 ("ctx_len", n_seqs), ("state_slots", n_seqs), ("want_rows", max(n_want, 1)),
+                 ("q_tile_map", 2 * n_tiles)]
         for g in range(n_groups):
             sizes += [(f"slot_mapping{g}", T), (f"block_table{g}", n_seqs * max_pages)]
         offs, total = {}, 0
@@ -363,6 +370,8 @@ class Engine:
         put("ctx_len", np.asarray(ctx_lens, dtype=np.int32))
         put("state_slots", np.asarray(slots, dtype=np.int32))
         put("want_rows", np.asarray(want_rows, dtype=np.int32))
+        if n_tiles:
+            put("q_tile_map", np.asarray([(i, t) for _, i, t in tiles], dtype=np.int32).reshape(-1))
         for g in range(n_groups):
             bt = np.full((n_seqs, max_pages), NO_PAGE, dtype=np.int32)
             sm = np.empty((T,), dtype=np.int32)
@@ -396,6 +405,9 @@ class Engine:
             max_ctx_len=max_ctx, q_lens=q_lens, ctx_lens=ctx_lens, slots=slots,
             meta_offset=self._meta_dev.data_ptr() if self._meta_dev is not None else 0,
             n_single=sum(1 for n in q_lens if n == 1),
+            n_query_tiles=n_tiles,
+            q_tile_map=view("q_tile_map").view(n_tiles, 2) if n_tiles else None,
+            prefill_max_ctx=max((c for c, n in zip(ctx_lens, q_lens) if n > 1), default=None),
             wants_all_rows=want_rows == list(range(T)),
             _scratch=self._scratch)
 

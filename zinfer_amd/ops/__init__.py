@@ -684,13 +684,33 @@ def mfma_attention_covers(dtype, n_heads, n_kv_heads, head_dim, page_size) -> bo
         and n_heads // n_kv_heads <= 16
 
 
+def _prefill_key_split(n_query_tiles: int, n_kv_heads: int, max_ctx_len: int):
+    """(keys per split, splits) if a prompt portion's attention should also split its keys over
+    workgroups: few query tiles behind a long context (a 512-token portion at context 4096: 128
+    workgroups that walk up to 128 key tiles each) leave half the chip idle and the rest
+    waiting on one chain of tiles.  Splits of at least 512 keys, about 512 workgroups; from
+    2048 keys on (measured, 481 queries of 40 heads on 8: 4096 keys 223 -> 151 us, 8192 keys
+    443 -> 259 us; at 1024 keys the partials cost what the split gains)."""
+    wgs = n_query_tiles * n_kv_heads
+    if wgs <= 0 or wgs >= 384 or max_ctx_len < 2048:
+        return None
+    want = (512 + wgs - 1) // wgs
+    keys = max(512, ((max_ctx_len + want - 1) // want + 31) // 32 * 32)
+    splits = (max_ctx_len + keys - 1) // keys
+    return (keys, splits) if splits >= 2 else None
+
+
 def paged_attention(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index, out, scale,
                     window, n_heads, n_kv_heads, head_dim, page_size, max_q_len,
-                    max_ctx_len, n_single=None) -> None:
+                    max_ctx_len, n_single=None, n_query_tiles=None, q_tile_map=None,
+                    prefill_max_ctx=None) -> None:
     """Causal grouped-query attention of the step's tokens over the paged cache.  Token t of
     sequence s = seq_index[t] has position ctx_len[s] - q_len[s] + (t - q_start[s]) and reads
     the positions up to its own (the last ``window`` of them if window > 0).  ``n_single`` is
-    the number of sequences with exactly one token in this step (None: unknown).
+    the number of sequences with exactly one token in this step (None: unknown),
+    ``n_query_tiles`` the number of 32-query tiles of the others, ``q_tile_map`` their int32
+    (sequence, tile) pairs [n_query_tiles, 2] and ``prefill_max_ctx`` the longest context among
+    those sequences (None: unknown): they only decide how the work is cut.
 
     bfloat16 with head_dim 32/64/128/256 and a page size that is a multiple of 16 runs the
     MFMA kernels: split-context decode for single tokens, the tiled kernel for portions.
@@ -730,11 +750,32 @@ def paged_attention(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index,
                 int(window), n_seqs, n_heads, n_kv_heads, head_dim, page_size, max_pages,
                 max_splits, _stream()), "paged_attention (decode)")
         if n_single != n_seqs and max_q_len > 1:
+            if q_tile_map is not None:
+                _i32(q_tile_map, "q_tile_map")
+                if n_query_tiles is None or q_tile_map.shape != (n_query_tiles, 2) \
+                        or not q_tile_map.is_cuda or not q_tile_map.is_contiguous():
+                    raise KernelUnavailable("paged_attention: q_tile_map must be int32 "
+                                            "[n_query_tiles, 2] on the device")
+            split = _prefill_key_split(n_query_tiles, n_kv_heads,
+                                       prefill_max_ctx if prefill_max_ctx is not None
+                                       else max_ctx_len) \
+                if n_query_tiles is not None else None
+            if split is not None and T * n_heads * split[1] * (head_dim + 2) * 4 > (1 << 28):
+                split = None
+            ws_o = ws_ml = None
+            if split is not None:
+                ws_o = _workspace("attn_pre_o", T * n_heads * split[1] * head_dim, torch.float32,
+                                  q.device)
+                ws_ml = _workspace("attn_pre_ml", T * n_heads * split[1] * 2, torch.float32,
+                                   q.device)
             _check(lib.zf_attn_prefill_bf16(
                 _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), _ptr(q_start),
                 _ptr(ctx_len), _ptr(out), ctypes.c_float(scale), int(window), n_seqs,
                 max_q_len, n_heads, n_kv_heads, head_dim, page_size, max_pages,
                 1 if n_single != 0 else 0, 1 if max_ctx_len <= 2 * max_q_len else 0,
+                _ptr(seq_index), T, _ptr(ws_o), _ptr(ws_ml),
+                split[0] if split is not None else 0, split[1] if split is not None else 0,
+                _ptr(q_tile_map), n_query_tiles if q_tile_map is not None else 0,
                 _stream()), "paged_attention (prefill)")
         return
     _check(lib.zf_paged_attention_wave(

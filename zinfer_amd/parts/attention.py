@@ -105,7 +105,9 @@ class GqaAttention(Mixer):
                             step.ctx_len, step.seq_index, attn, float(self.scale),
                             0 if s.window is None else int(s.window),
                             s.n_heads, s.n_kv_heads, s.head_dim, cache.page_size,
-                            step.max_q_len, step.max_ctx_len, n_single=step.n_single)
+                            step.max_q_len, step.max_ctx_len, n_single=step.n_single,
+                            n_query_tiles=step.n_query_tiles, q_tile_map=step.q_tile_map,
+                            prefill_max_ctx=step.prefill_max_ctx)
         self.o.forward(attn, residual, accumulate=True, step=step)
 
 
