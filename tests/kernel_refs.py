@@ -96,7 +96,8 @@ def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, cos, sin, positions, slot_ma
 
 def paged_attention(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index, out, scale,
                     window, n_heads, n_kv_heads, head_dim, page_size, max_q_len, max_ctx_len,
-                    n_single=None, n_query_tiles=None, q_tile_map=None, prefill_max_ctx=None):
+                    n_single=None, n_query_tiles=None, q_tile_map=None, prefill_max_ctx=None,
+                    prefill_variant=0):
     T = q.shape[0]
     hd = head_dim
     G = n_heads // n_kv_heads

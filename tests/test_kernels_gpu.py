@@ -396,7 +396,8 @@ def _paged_setup(dtype, nH, nKV, hd, page_size, ctx_lens, q_lens, seed, num_page
                 seq_index=seq_index.int(), Ks=Ks, Vs=Vs)
 
 
-def _run_attention(s, dtype, nH, nKV, hd, page_size, window, q_lens, ctx_lens, tiles_hint=False):
+def _run_attention(s, dtype, nH, nKV, hd, page_size, window, q_lens, ctx_lens, tiles_hint=False,
+                   variant=0):
     scale = 1.0 / math.sqrt(hd)
     T = s["q"].shape[0]
     want = torch.empty((T, nH * hd), dtype=dtype)
@@ -412,7 +413,7 @@ def _run_attention(s, dtype, nH, nKV, hd, page_size, window, q_lens, ctx_lens, t
     _ops().paged_attention(d["q"], d["k_pool"], d["v_pool"], d["block_table"], d["q_start"],
                            d["ctx_len"], d["seq_index"], got, scale, window, nH, nKV, hd,
                            page_size, max(q_lens), max(ctx_lens),
-                           n_single=sum(1 for n in q_lens if n == 1),
+                           n_single=sum(1 for n in q_lens if n == 1), prefill_variant=variant,
                            **_tile_hints(q_lens, ctx_lens, tiles_hint))
     return got, want
 
@@ -448,7 +449,8 @@ def test_paged_attention_mixed_batch(dtype, nH, nKV, hd, page_size, window):
 @pytest.mark.parametrize("nH,nKV,hd,page_size,window", [
     (8, 2, 32, 16, 0), (32, 8, 128, 16, 0), (6, 6, 64, 32, 0), (16, 1, 64, 16, 0),
     (9, 3, 256, 16, 0), (8, 2, 64, 16, 37), (4, 4, 128, 48, 300), (36, 4, 32, 16, 0),
-    (16, 2, 128, 16, 0), (8, 2, 128, 32, 100), (16, 2, 128, 16, 45)])
+    (16, 2, 128, 16, 0), (8, 2, 128, 32, 100), (16, 2, 128, 16, 45), (10, 2, 128, 16, 0),
+    (6, 2, 64, 48, 20), (4, 2, 128, 64, 0), (24, 2, 64, 16, 0)])
 @pytest.mark.parametrize("kind", ["decode", "prefill", "mixed", "whole"])
 def test_paged_attention_mfma(nH, nKV, hd, page_size, window, kind):
     """The bfloat16 MFMA kernels: decode tokens over contexts that end at, before and after a
@@ -796,19 +798,24 @@ def test_mfma_decode_window_edge_and_far_key(hd):
             assert rel_err(got, want) <= 2 * tol(dtype), f"ctx {ctx}, window {window}, key {target}"
 
 
+@pytest.mark.parametrize("variant", [1, 2])
 @pytest.mark.parametrize("hd", [64, 128])
-def test_mfma_prefill_window_edge_and_far_key(hd):
-    """The MFMA prefill kernel on a portion that starts mid-context: for the first and the last
+def test_mfma_prefill_window_edge_and_far_key(hd, variant):
+    """Both MFMA prefill kernels (1: every wave fetches its keys and values, 2: they are staged
+    in LDS in tiles of 64 keys) on a portion that starts mid-context: for the first and the last
     query of a 32-query tile, a key that stands out at p - window (no influence) and at
     p - window + 1 (all the weight); windows whose first key falls on and beside the edges of a
-    32-key tile; without a window, a far key at the very start and at a tile's edge."""
+    32- and a 64-key tile; without a window, a far key at the very start, at the tiles' edges
+    and in a later tile that needs no mask (where the exponent the sums are held against has
+    to move)."""
     dtype, nH, nKV, ps = torch.bfloat16, 4, 2, 16
     ctx, q_len = 420, 100                       # the portion is positions 320 .. 419
     start = ctx - q_len
-    for window in (0, 33, 64, 65, 97, 200, 330):
+    for window in (0, 33, 64, 65, 97, 129, 200, 330):
         for row in (0, 31, 32, 63, 99):         # rows of the portion: tile edges and the last
             p = start + row
-            cases = [(0, True), (31, True), (32, True), (p, True)] if window == 0 else \
+            cases = [(0, True), (31, True), (32, True), (63, True), (64, True), (127, True),
+                     (200, True), (p, True)] if window == 0 else \
                 [(p - window, False), (p - window + 1, True)]
             for target, inside in cases:
                 if target < 0:
@@ -816,7 +823,7 @@ def test_mfma_prefill_window_edge_and_far_key(hd):
                 s = _paged_setup(dtype, nH, nKV, hd, ps, [ctx, 70], [q_len, 70], seed=23)
                 _stand_out(s, nKV, ps, hd, 0, target, row, 3, dtype, nH)
                 got, want = _run_attention(s, dtype, nH, nKV, hd, ps, window, [q_len, 70],
-                                           [ctx, 70])
+                                           [ctx, 70], variant=variant)
                 v_row = s["Vs"][0][target, 3 // (nH // nKV)].float()
                 close = torch.allclose(got.cpu().float()[row, 3 * hd:4 * hd], v_row, atol=3e-2)
                 assert close == inside, f"window {window}, query {p}, key {target}"
@@ -839,9 +846,30 @@ def test_cast_and_poison_pages():
         assert bad[:, [0, 4, 7]].all() and not bad[:, [1, 2, 3, 5, 6, 8]].any()
 
 
+@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("nH,nKV,hd,ps,window", [
+    (8, 2, 128, 16, 0), (10, 2, 128, 16, 0), (16, 2, 64, 32, 0), (3, 1, 128, 48, 0),
+    (2, 2, 64, 16, 0), (18, 2, 128, 16, 0), (8, 2, 128, 16, 150), (5, 1, 64, 16, 64)])
+def test_both_prefill_kernels_on_portions_and_whole_prompts(nH, nKV, hd, ps, window, variant):
+    """Each of the two MFMA prefill kernels, chosen by hand, over groups of 1, 3, 4, 5, 8 and 9
+    query heads (9: two blocks of heads per kv head), whole prompts and portions whose keys
+    end at, before and after the edges of 64-key tiles, pages of 16, 32 and 48 rows in a
+    shuffled pool whose unwritten rows are NaN, with and without the engine's list of tiles."""
+    dtype = torch.bfloat16
+    ctx_lens = [64, 65, 127, 128, 129, 300, 1000, 40, 2]
+    q_lens = [64, 65, 127, 64, 2, 237, 130, 7, 2]
+    s = _paged_setup(dtype, nH, nKV, hd, ps, ctx_lens, q_lens, seed=41)
+    for hint in (False, True):
+        got, want = _run_attention(s, dtype, nH, nKV, hd, ps, window, q_lens, ctx_lens,
+                                   tiles_hint=hint, variant=variant)
+        assert not torch.isnan(got.float()).any(), "a row outside the context was read"
+        assert rel_err(got, want) <= 2 * tol(dtype)
+
+
 @pytest.mark.parametrize("nH,nKV,hd,window", [(10, 2, 128, 0), (8, 1, 64, 0), (4, 1, 128, 0),
                                               (10, 2, 128, 700), (6, 2, 64, 33)])
-def test_prefill_attention_splits_keys_over_workgroups(nH, nKV, hd, window):
+@pytest.mark.parametrize("variant", [1, 2])
+def test_prefill_attention_splits_keys_over_workgroups(nH, nKV, hd, window, variant):
     """Portions behind long contexts, few query tiles: the keys are split over workgroups and
     a second kernel merges the partials.  Portions that start at 0, mid-page and at a split's
     edge, a short prompt whose keys lie in one split, single tokens beside them; and a key
@@ -854,11 +882,12 @@ def test_prefill_attention_splits_keys_over_workgroups(nH, nKV, hd, window):
     split = ops._prefill_key_split(tiles, nKV, max(ctx_lens))
     assert split is not None and split[1] >= 2
     s = _paged_setup(dtype, nH, nKV, hd, ps, ctx_lens, q_lens, seed=31)
-    got, want = _run_attention(s, dtype, nH, nKV, hd, ps, window, q_lens, ctx_lens, tiles_hint=True)
+    got, want = _run_attention(s, dtype, nH, nKV, hd, ps, window, q_lens, ctx_lens, tiles_hint=True,
+                               variant=variant)
     assert not torch.isnan(got.float()).any(), "a slot outside the context was read"
     assert rel_err(got, want) <= 2 * tol(dtype)
     # the same without the hint (one workgroup walks all keys): equal up to rounding
-    plain, _ = _run_attention(s, dtype, nH, nKV, hd, ps, window, q_lens, ctx_lens)
+    plain, _ = _run_attention(s, dtype, nH, nKV, hd, ps, window, q_lens, ctx_lens, variant=variant)
     assert rel_err(got, plain) <= 2 * tol(dtype)
     if window == 0:
         keys = split[0]
@@ -867,7 +896,7 @@ def test_prefill_attention_splits_keys_over_workgroups(nH, nKV, hd, window):
             row = 57                     # a query of the first sequence (position 2257)
             _stand_out(s, nKV, ps, hd, 0, target, row, nH - 1, dtype, nH)
             got, want = _run_attention(s, dtype, nH, nKV, hd, ps, 0, q_lens, ctx_lens,
-                                       tiles_hint=True)
+                                       tiles_hint=True, variant=variant)
             v_row = s["Vs"][0][target, (nH - 1) // (nH // nKV)].float()
             assert torch.allclose(got.cpu().float()[row, (nH - 1) * hd:nH * hd], v_row, atol=3e-2), target
             assert rel_err(got, want) <= 2 * tol(dtype)

@@ -135,6 +135,18 @@ typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
 // which a soft-max term does not need.
 __device__ __forceinline__ float exp2_raw(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// maximum and sum of a value over the two lanes 32 places apart, the same in both
+// (v_permlane32_swap leaves the low half's values in one register and the high half's in
+// the other: no trip through LDS)
+__device__ __forceinline__ float max_of_halves(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_of_halves(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   return pack_bf16x2(lo, hi);
 }
@@ -694,6 +706,356 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
   }
 }
 
+// The same work with the keys and values of a tile staged once per workgroup: one workgroup
+// per (sequence, tile of 32 queries, kv head, block of up to 8 of its query heads), wave w
+// takes head w of the block.  Tiles of 64 keys go from the tiled pools into LDS with
+// direct-to-LDS loads (no registers in between; a wave instruction copies 1 KB, 64 lanes x 16
+// bytes, to one uniform LDS address + 16 bytes a lane, which is the pools' own order), two
+// stages: the next tile is in flight while the waves compute this one out of LDS, each reading
+// the operands at the offsets it would have read in the pool.  Against attn_prefill_kernel,
+// where every wave fetches its own copy of a tile from L2 and looks up its pages lane by
+// lane, the loads of a tile and their address arithmetic are shared by the heads of the group.
+// The stages are two arrays, not one indexed array: the compiler then knows that reads of one
+// stage do not wait for the loads into the other.
+template <int HD, bool POW2>
+__global__ __launch_bounds__(512) void attn_prefill_shared_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool,
+    const bf16_t* __restrict__ v_pool, const int* __restrict__ block_table,
+    const int* __restrict__ q_start, const int* __restrict__ ctx_len, bf16_t* __restrict__ out,
+    float scale_log2e, int window, int nH, int nKV, int ps, int max_pages, int skip_single,
+    int q_tiles, int head_blocks, int ps_shift, float* __restrict__ ws_o,
+    float* __restrict__ ws_ml, int split_keys, int max_splits,
+    const int* __restrict__ tile_map) {
+  constexpr int GROUP_CHUNKS = 2 * HD;          // 16-byte pieces of 16 rows of one kv head
+  constexpr int TILE_CHUNKS = 4 * GROUP_CHUNKS;  // of 64 rows: keys first, then values
+  __shared__ u32x4_t stage0[2 * TILE_CHUNKS];
+  __shared__ u32x4_t stage1[2 * TILE_CHUNKS];
+  auto page_of = [&](int key) { return POW2 ? key >> ps_shift : key / ps; };
+  auto row_of = [&](int key) { return POW2 ? key & (ps - 1) : key % ps; };
+  const int kvh = blockIdx.x % nKV;
+  const int hb = (blockIdx.x / nKV) % head_blocks;
+  const int entry = blockIdx.x / (nKV * head_blocks);
+  const int qt = tile_map ? tile_map[2 * entry + 1] : q_tiles - 1 - entry % q_tiles;
+  const int s = tile_map ? tile_map[2 * entry] : entry / q_tiles;
+  const int q_len = q_start[s + 1] - q_start[s];
+  if (q_len == 1 && skip_single) return;
+  const int qbase = qt * 32;
+  if (qbase >= q_len) return;
+  const int ctx = ctx_len[s];
+  const int pos0 = ctx - q_len + qbase;
+  const int nq = min(32, q_len - qbase);
+  const int p_max = pos0 + nq - 1;
+  const int G = nH / nKV;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64), nwaves = blockDim.x / 64;
+  const int lane = threadIdx.x % 64, j = lane % 32, hf = lane / 32;
+  const bool q_valid = j < nq;
+  const int p_j = pos0 + min(j, nq - 1);
+  const int lo_j = (window > 0 && p_j - window + 1 > 0) ? p_j - window + 1 : 0;
+  const int lo_min = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int lo_top = (window > 0 && p_max - window + 1 > 0) ? p_max - window + 1 : 0;
+  const int* table = block_table + (size_t)s * max_pages;
+  const int t_row = q_start[s] + qbase + min(j, nq - 1);
+  const int k_lo = gridDim.y > 1 ? max(lo_min, (int)blockIdx.y * split_keys) : lo_min;
+  const int k_hi = gridDim.y > 1 ? min(p_max, ((int)blockIdx.y + 1) * split_keys - 1) : p_max;
+  if (k_lo > k_hi) return;      // uniform over the workgroup: before any barrier
+  const int g = hb * nwaves + wave;
+  const bool active = g < G;
+  const int head = kvh * G + min(g, G - 1);
+
+  // groups of 16 rows that hold live keys of this request: every load is clamped into them
+  const int lo_grp = (lo_min / 16) * 16, hi_grp = (p_max / 16) * 16;
+  auto source_of = [&](int base) { return min(max(base, lo_grp), hi_grp); };
+  // pool offsets in 16-byte pieces: a page holds nKV * ps * HD / 8 of them
+  const int gpp = ps / 16;                       // groups of 16 rows in a page
+  const uint32_t page_chunks = (uint32_t)nKV * ps * (HD / 8);
+  const uint32_t head_chunks = (uint32_t)kvh * ps * (HD / 8);
+  const u32x4_t* k_chunks = (const u32x4_t*)k_pool;
+  const u32x4_t* v_chunks = (const u32x4_t*)v_pool;
+  auto issue = [&](int kb, u32x4_t* stage) {
+    // where the tile's four groups of 16 rows lie in the pools: four scalar look-ups in flight
+    // together, then the copies
+    int gi[4], pg[4];
+#pragma unroll
+    for (int grp = 0; grp < 4; ++grp) gi[grp] = source_of(kb + 16 * grp) / 16;
+#pragma unroll
+    for (int grp = 0; grp < 4; ++grp) pg[grp] = table[POW2 ? gi[grp] >> (ps_shift - 4) : gi[grp] / gpp];
+    uint64_t at[4];
+#pragma unroll
+    for (int grp = 0; grp < 4; ++grp)
+      at[grp] = (uint64_t)(uint32_t)pg[grp] * page_chunks + head_chunks +
+                (uint32_t)(POW2 ? gi[grp] & (gpp - 1) : gi[grp] % gpp) * GROUP_CHUNKS;
+    for (int c0 = wave * 64; c0 < TILE_CHUNKS; c0 += 64 * nwaves) {
+      const int grp = c0 / GROUP_CHUNKS;
+      const uint64_t base = grp == 0 ? at[0] : grp == 1 ? at[1] : grp == 2 ? at[2] : at[3];
+      const uint64_t from = base + (uint32_t)(c0 % GROUP_CHUNKS + lane);
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(k_chunks + from),
+          (__attribute__((address_space(3))) void*)(stage + c0), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(v_chunks + from),
+          (__attribute__((address_space(3))) void*)(stage + TILE_CHUNKS + c0), 16, 0, 0);
+    }
+  };
+  // the loads into LDS count as vector-memory operations: all of this wave's have landed,
+  // then all waves meet
+  auto landed = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0)
+    __syncthreads();
+  };
+
+  bf16x8_t qf[HD / 16];
+  {
+    const bf16_t* qrow = q + ((size_t)t_row * nH + head) * HD + 8 * hf;
+#pragma unroll
+    for (int st = 0; st < HD / 16; ++st) {
+      u32x4_t v = *(const u32x4_t*)(qrow + st * 16);
+      if (!q_valid) v = u32x4_t{0, 0, 0, 0};
+      qf[st] = *(bf16x8_t*)&v;
+    }
+  }
+  f32x16_t o[HD / 32];
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
+  float m = -INFINITY, l = 0.f;
+  // the lane's places inside a stage: keys in 16-byte pieces, values in 8-byte pieces
+  const int k_at = (j / 16) * GROUP_CHUNKS + hf * 16 + j % 16;
+  const int v_at = (j / 16) * 64 + hf * 16 + j % 16;
+
+  // one tile out of `stage`; the next one is requested into `next` once this tile's first
+  // products are under way (every wave has left `next` behind at the barrier before)
+  auto tile = [&](int kb, const u32x4_t* stage, u32x4_t* next) {
+    if (!active) {
+      if (kb + 64 <= k_hi) issue(kb + 64, next);
+      return;
+    }
+    if (kb + 64 <= k_hi) issue(kb + 64, next);
+    const u32x4_t* sk = stage + k_at;
+    const u32x2_t* sv = (const u32x2_t*)(stage + TILE_CHUNKS) + v_at;
+    f32x16_t st[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) st[h][r] = 0.f;
+    bool have_scores = false;
+    if (__builtin_expect(kb + 63 <= pos0 && kb >= lo_top, 1)) {
+      // Every key of the tile is visible to every query of the wave (so all its rows hold
+      // keys of this request and were loaded from their own places): no masks.
+      u32x4_t kf[2][HD / 16];
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int stp = 0; stp < HD / 16; ++stp)
+          kf[h][stp] = sk[2 * h * GROUP_CHUNKS + (stp / 2) * 64 + (stp % 2) * 32];
+      // the two halves' products alternate: neither waits for its own last result
+#pragma unroll
+      for (int stp = 0; stp < HD / 16; ++stp) {
+        st[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&kf[0][stp], qf[stp], st[0], 0, 0, 0);
+        st[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&kf[1][stp], qf[stp], st[1], 0, 0, 0);
+      }
+      have_scores = true;
+      float tmax = st[0][0];
+#pragma unroll
+      for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, st[0][r]);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, st[1][r]);
+      tmax = max_of_halves(tmax) * scale_log2e;
+      // m is the exponent the running sums are held against, not always the maximum: here it
+      // stays where it is unless a score exceeds it by more than 2^20 (after a query's first
+      // keys that is rare; the tile then takes the path below, which moves it and rescales
+      // the sums).  The terms stay far inside the range of 32-bit and bfloat16 numbers,
+      // whose relative precision does not depend on their size.
+      const float m_ref = (m == -INFINITY) ? tmax : m;      // nothing summed yet
+      if (__builtin_expect(!__any(tmax > m_ref + 20.f), 1)) {
+        m = m_ref;
+        float psum = 0.f;
+        auto terms = [&](int h) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            st[h][r] = exp2_raw(fmaf(st[h][r], scale_log2e, -m_ref));
+            psum += st[h][r];
+          }
+        };
+        auto values = [&](int h) {
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            u32x4_t pk = u32x4_t{pack_bf16(st[h][8 * u + 0], st[h][8 * u + 1]),
+                                 pack_bf16(st[h][8 * u + 2], st[h][8 * u + 3]),
+                                 pack_bf16(st[h][8 * u + 4], st[h][8 * u + 5]),
+                                 pack_bf16(st[h][8 * u + 6], st[h][8 * u + 7])};
+            const bf16x8_t pf = *(bf16x8_t*)&pk;
+            const u32x2_t* svg = sv + (2 * h + u) * 4 * HD;
+#pragma unroll
+            for (int dt = 0; dt < HD / 32; ++dt) {
+              const u32x2_t v0 = svg[dt * 128], v1 = svg[dt * 128 + 32];
+              u32x4_t vv = u32x4_t{v0[0], v0[1], v1[0], v1[1]};
+              o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8_t*)&vv, pf, o[dt], 0, 0, 0);
+            }
+          }
+        };
+        // the second half's terms (vector ALU) are issued between the products of the first
+        // half's values (matrix cores)
+        terms(0);
+        values(0);
+        terms(1);
+        l += sum_of_halves(psum);
+        values(1);
+        return;
+      }
+    }
+    asm volatile("");      // a real branch: the tiles at the diagonal and at the ends
+    // the second 32 keys of the tile: beyond the last key any query here reads?
+    const bool two = kb + 32 <= k_hi;
+    if (!have_scores) {
+#pragma unroll
+      for (int stp = 0; stp < HD / 16; ++stp) {
+        const u32x4_t kf = sk[(stp / 2) * 64 + (stp % 2) * 32];
+        st[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&kf, qf[stp], st[0], 0, 0, 0);
+      }
+      if (two) {
+#pragma unroll
+        for (int stp = 0; stp < HD / 16; ++stp) {
+          const u32x4_t kf = sk[2 * GROUP_CHUNKS + (stp / 2) * 64 + (stp % 2) * 32];
+          st[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&kf, qf[stp], st[1], 0, 0, 0);
+        }
+      }
+    }
+    // st[h][r]: key kb + 32 h + 8 (r / 4) + 4 hf + r % 4, query column j
+    float tmax = -INFINITY;
+    if (kb + 63 <= pos0 && kb >= lo_top) {
+      // every key of the tile is visible to every query of the wave: nothing to mask
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, st[h][r]);
+    } else {
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = kb + 32 * h + 8 * (r / 4) + 4 * hf + r % 4;
+          const float v = (key <= p_j && key >= lo_j && (h == 0 || two)) ? st[h][r] : -INFINITY;
+          st[h][r] = v;
+          tmax = fmaxf(tmax, v);
+        }
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * scale_log2e;
+    const float m_new = fmaxf(m, tmax);
+    // a query whose window lies wholly beyond this tile has no key here yet
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float corr = exp2_raw(m - m_use);
+    float psum = 0.f;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        st[h][r] = exp2_raw(fmaf(st[h][r], scale_log2e, -m_use));
+        psum += st[h][r];
+      }
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * corr + psum;
+    m = m_new;
+    if (__any(corr != 1.0f)) {      // after the first tiles the maxima rarely move
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[dt][r] *= corr;
+    }
+    auto packed = [&](int h, int u) {
+      // slots e = 0..7 <-> st[h][8 u + e]: keys base + 4 hf + e (e < 4) and
+      // base + 8 + 4 hf + (e - 4), base = kb + 32 h + 16 u
+      u32x4_t pk = u32x4_t{pack_bf16(st[h][8 * u + 0], st[h][8 * u + 1]),
+                           pack_bf16(st[h][8 * u + 2], st[h][8 * u + 3]),
+                           pack_bf16(st[h][8 * u + 4], st[h][8 * u + 5]),
+                           pack_bf16(st[h][8 * u + 6], st[h][8 * u + 7])};
+      return *(bf16x8_t*)&pk;
+    };
+    // every group of the tile was loaded from its own place and all its rows hold keys of
+    // this request: nothing to look at group by group
+    if (kb >= lo_min && kb + 64 <= ctx && kb + 48 <= hi_grp) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const bf16x8_t pf = packed(h, u);
+          const u32x2_t* svg = sv + (2 * h + u) * 4 * HD;
+#pragma unroll
+          for (int dt = 0; dt < HD / 32; ++dt) {
+            const u32x2_t v0 = svg[dt * 128], v1 = svg[dt * 128 + 32];
+            u32x4_t vv = u32x4_t{v0[0], v0[1], v1[0], v1[1]};
+            o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8_t*)&vv, pf, o[dt], 0, 0, 0);
+          }
+        }
+      return;
+    }
+    asm volatile("");      // a real branch: the tiles at the ends of the key range
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      if (h == 1 && !two) break;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const bf16x8_t pf = packed(h, u);
+        // the rows that were loaded for this group (clamped into the live groups) and which
+        // of them hold a key of this request: rows at or beyond ctx were never written, rows
+        // below lo_min may be stale; both are zeroed (0 * NaN would poison the sum)
+        const int src = source_of(kb + 32 * h + 16 * u);
+        const int a0 = src + 4 * hf, a1 = a0 + 8;
+        const u32x2_t all = u32x2_t{~0u, ~0u};
+        const u32x2_t keep0 = keep_range4(all, lo_min - a0, ctx - a0);
+        const u32x2_t keep1 = keep_range4(all, lo_min - a1, ctx - a1);
+        const u32x2_t* svg = sv + (2 * h + u) * 4 * HD;
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt) {
+          const u32x2_t v0 = svg[dt * 128], v1 = svg[dt * 128 + 32];
+          u32x4_t vv = u32x4_t{v0[0] & keep0[0], v0[1] & keep0[1], v1[0] & keep1[0],
+                               v1[1] & keep1[1]};
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8_t*)&vv, pf, o[dt], 0, 0, 0);
+        }
+      }
+    }
+  };
+
+  const int kb0 = (k_lo / 64) * 64;
+  issue(kb0, stage0);
+  landed();
+  for (int kb = kb0; kb <= k_hi; kb += 128) {
+    tile(kb, stage0, stage1);
+    landed();
+    if (kb + 64 > k_hi) break;
+    tile(kb + 64, stage1, stage0);
+    landed();
+  }
+  if (!active || !q_valid) return;
+  if (gridDim.y > 1) {
+    // this split's partial for (token, head): O^T un-normalised, running maximum and sum
+    const size_t slot = ((size_t)t_row * nH + head) * max_splits + blockIdx.y;
+    float* dst = ws_o + slot * HD;
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4)
+        *(f32x4_t*)(dst + dt * 32 + 8 * r4 + 4 * hf) =
+            f32x4_t{o[dt][r4 * 4 + 0], o[dt][r4 * 4 + 1], o[dt][r4 * 4 + 2], o[dt][r4 * 4 + 3]};
+    if (hf == 0) {
+      ws_ml[slot * 2] = m;
+      ws_ml[slot * 2 + 1] = l;
+    }
+    return;
+  }
+  const float inv = 1.0f / l;
+  bf16_t* orow = out + ((size_t)t_row * nH + head) * HD;
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+      const int d = dt * 32 + 8 * r4 + 4 * hf;
+      u32x2_t w = u32x2_t{pack_bf16(o[dt][r4 * 4 + 0] * inv, o[dt][r4 * 4 + 1] * inv),
+                          pack_bf16(o[dt][r4 * 4 + 2] * inv, o[dt][r4 * 4 + 3] * inv)};
+      *(u32x2_t*)(orow + d) = w;
+    }
+}
+
 // Combines the key splits of one (token, head) of a prompt portion in split order and writes
 // bfloat16: token t of sequence s = seq_index[t] sits at position ctx_len[s] - q_len + (t -
 // q_start[s]) and has partials from the splits that hold its keys lo .. position.
@@ -739,6 +1101,9 @@ __global__ __launch_bounds__(64) void attn_prefill_merge_kernel(
 // exist.  split_keys > 0 (a multiple of 32; ws_o: n_tokens * nH * max_splits * hd floats, ws_ml:
 // n_tokens * nH * max_splits * 2, max_splits >= ceil(longest context / split_keys)): the keys
 // are split over workgroups and merged by a second kernel.
+// variant: 0 chooses; 1 the kernel whose waves fetch their own keys and values; 2 the kernel
+// that stages them in LDS for the heads of a group (head sizes 64 and 128, splits of a
+// multiple of 64 keys), -2 where it does not apply.
 extern "C" int zf_attn_prefill_bf16(const void* q, const void* k_pool, const void* v_pool,
                                     const int* block_table, const int* q_start,
                                     const int* ctx_len, void* out, float scale, int window,
@@ -746,9 +1111,11 @@ extern "C" int zf_attn_prefill_bf16(const void* q, const void* k_pool, const voi
                                     int page_size, int max_pages, int skip_single,
                                     int allow_split, const int* seq_index, int n_tokens,
                                     float* ws_o, float* ws_ml, int split_keys, int max_splits,
-                                    const int* tile_map, int n_tiles, hipStream_t stream) {
+                                    const int* tile_map, int n_tiles, int variant,
+                                    hipStream_t stream) {
   if (n_seqs <= 0 || max_q_len <= 0) return 0;
   if (page_size % 16 != 0 || nKV <= 0 || nH % nKV != 0) return -2;
+  if (variant < 0 || variant > 2) return -2;
   if (split_keys > 0 && (split_keys % 32 != 0 || max_splits < 1 || ws_o == nullptr ||
                          ws_ml == nullptr || seq_index == nullptr))
     return -2;
@@ -756,8 +1123,36 @@ extern "C" int zf_attn_prefill_bf16(const void* q, const void* k_pool, const voi
   const int G = nH / nKV;
   const int q_tiles = (max_q_len + 31) / 32;
   if (tile_map != nullptr && n_tiles <= 0) return 0;
-  dim3 grid((unsigned)(tile_map != nullptr ? n_tiles : n_seqs * q_tiles) * nKV,
-            split_keys > 0 ? max_splits : 1);
+  int ps_shift = -1;
+  for (int b = 4; b < 31; ++b)
+    if (page_size == (1 << b)) ps_shift = b;
+  const unsigned entries = (unsigned)(tile_map != nullptr ? n_tiles : n_seqs * q_tiles);
+  // from two query heads per kv head on, the tiles staged in LDS are shared (measured: faster
+  // at every length from 512 tokens to 16 K, 1.1 to 1.9 times); a lone head would be one wave
+  // per workgroup and stays with the first kernel, whose waves split its key tiles
+  const bool shared_ok = (hd == 64 || hd == 128) && split_keys % 64 == 0;
+  if (variant == 2 && !shared_ok) return -2;
+  if (variant == 2 || (variant == 0 && shared_ok && G >= 2)) {
+    const int waves = G < 8 ? G : 8, head_blocks = (G + waves - 1) / waves;
+    dim3 sgrid(entries * head_blocks * nKV, split_keys > 0 ? max_splits : 1);
+#define ZF_PRE_S(HD, POW2)                                                                      \
+  hipLaunchKernelGGL((attn_prefill_shared_kernel<HD, POW2>), sgrid, dim3(64 * waves), 0, stream, \
+                     (const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool,            \
+                     block_table, q_start, ctx_len, (bf16_t*)out, scale_log2e, window, nH, nKV, \
+                     page_size, max_pages, skip_single, q_tiles, head_blocks, ps_shift, ws_o,   \
+                     ws_ml, split_keys, max_splits, tile_map)
+    if (hd == 64 && ps_shift >= 0) ZF_PRE_S(64, true);
+    else if (hd == 64) ZF_PRE_S(64, false);
+    else if (ps_shift >= 0) ZF_PRE_S(128, true);
+    else ZF_PRE_S(128, false);
+#undef ZF_PRE_S
+    if (split_keys > 0)
+      hipLaunchKernelGGL(attn_prefill_merge_kernel, dim3(n_tokens, nH), dim3(64), 0, stream,
+                         ws_o, ws_ml, q_start, ctx_len, seq_index, (bf16_t*)out, window, nH, hd,
+                         split_keys, max_splits, skip_single);
+    ZF_CHECK_LAUNCH();
+  }
+  dim3 grid(entries * nKV, split_keys > 0 ? max_splits : 1);
   // up to 8 waves: one per query head of the kv head, and with 4 heads or fewer several
   // waves per head that split its key tiles, as far as the partials fit into LDS
   // (allow_split: the caller expects short contexts before the portions, where the causal
@@ -768,9 +1163,6 @@ extern "C" int zf_attn_prefill_bf16(const void* q, const void* k_pool, const voi
   const int head_waves = G < 8 ? G : 8;
   dim3 block(64 * head_waves * nsplit);
   const size_t smem = nsplit > 1 ? (size_t)(nsplit - 1) * G * per_wave : 0;
-  int ps_shift = -1;
-  for (int b = 4; b < 31; ++b)
-    if (page_size == (1 << b)) ps_shift = b;
 #define ZF_PRE_K(KERN)                                                                          \
   do {                                                                                          \
     if (smem > 64 * 1024) {                                                                     \

@@ -695,7 +695,7 @@ def _prefill_key_split(n_query_tiles: int, n_kv_heads: int, max_ctx_len: int):
     if wgs <= 0 or wgs >= 384 or max_ctx_len < 2048:
         return None
     want = (512 + wgs - 1) // wgs
-    keys = max(512, ((max_ctx_len + want - 1) // want + 31) // 32 * 32)
+    keys = max(512, ((max_ctx_len + want - 1) // want + 63) // 64 * 64)
     splits = (max_ctx_len + keys - 1) // keys
     return (keys, splits) if splits >= 2 else None
 
@@ -703,7 +703,7 @@ def _prefill_key_split(n_query_tiles: int, n_kv_heads: int, max_ctx_len: int):
 def paged_attention(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index, out, scale,
                     window, n_heads, n_kv_heads, head_dim, page_size, max_q_len,
                     max_ctx_len, n_single=None, n_query_tiles=None, q_tile_map=None,
-                    prefill_max_ctx=None) -> None:
+                    prefill_max_ctx=None, prefill_variant=0) -> None:
     """Causal grouped-query attention of the step's tokens over the paged cache.  Token t of
     sequence s = seq_index[t] has position ctx_len[s] - q_len[s] + (t - q_start[s]) and reads
     the positions up to its own (the last ``window`` of them if window > 0).  ``n_single`` is
@@ -711,6 +711,9 @@ def paged_attention(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index,
     ``n_query_tiles`` the number of 32-query tiles of the others, ``q_tile_map`` their int32
     (sequence, tile) pairs [n_query_tiles, 2] and ``prefill_max_ctx`` the longest context among
     those sequences (None: unknown): they only decide how the work is cut.
+    ``prefill_variant`` picks the kernel for the portions (0: by size; 1: every wave fetches
+    its keys and values; 2: they are staged in LDS for a group's heads), for measurements and
+    tests.
 
     bfloat16 with head_dim 32/64/128/256 and a page size that is a multiple of 16 runs the
     MFMA kernels: split-context decode for single tokens, the tiled kernel for portions.
@@ -776,7 +779,7 @@ def paged_attention(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index,
                 _ptr(seq_index), T, _ptr(ws_o), _ptr(ws_ml),
                 split[0] if split is not None else 0, split[1] if split is not None else 0,
                 _ptr(q_tile_map), n_query_tiles if q_tile_map is not None else 0,
-                _stream()), "paged_attention (prefill)")
+                int(prefill_variant), _stream()), "paged_attention (prefill)")
         return
     _check(lib.zf_paged_attention_wave(
         _ptr(q), _ptr(k_pool), _ptr(v_pool), _dt(q), _ptr(block_table), _ptr(q_start),
