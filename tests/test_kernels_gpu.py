@@ -203,12 +203,15 @@ def test_gemm_sum_norm(M, N, K):
 
 @pytest.mark.parametrize("kind", ["store", "accumulate", "swiglu"])
 @pytest.mark.parametrize("K", [192, 256, 64])
-def test_gemm_many_large_tiles(kind, K):
-    """Enough 128 x 256 tiles to fill the chip more than once (the kernel that takes
-    pre-tiled W straight into its operands), with edges in M and N that are no multiple of
-    the tile; an odd and an even number of k-tiles (W one or two k-tiles ahead) and one."""
+@pytest.mark.parametrize("M,N,variant", [(4100, 4160, 10), (2100, 6208, 6)])
+def test_gemm_many_large_tiles(kind, K, M, N, variant):
+    """Enough 128 x 256 tiles (and, at the second size, 128 x 128 tiles) to fill the chip more
+    than once: the kernels that take pre-tiled W straight into their operands and copy the
+    tokens straight into LDS, with edges in M and N that are no multiple of the tile; an odd
+    and an even number of k-tiles (W one or two k-tiles ahead) and one."""
     ops = _ops()
-    M, N = 4100, 4160
+    assert ops._tile_variant(M, N, True, kind == "accumulate", K) == variant
+    assert variant == 10 or ((M + 127) // 128) * ((N + 127) // 128) >= 512
     a = _rand((M, K), torch.bfloat16, 35)
     w = _rand((N, K), torch.bfloat16, 36, 0.05)
     if kind == "swiglu":

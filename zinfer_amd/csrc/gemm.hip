@@ -310,7 +310,17 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_ker
 // 256 bytes), one k-tile ahead in registers.  That halves the LDS traffic per MFMA against
 // the kernel above, whose LDS is as busy as its MFMAs.  With the waves side by side along the
 // outputs (WM == BM) no two of them load the same part of W.
-template <int BM, int BN, int WM, int WN, int EPI, int TKM = TK, bool W2 = false>
+// ADMA: the tokens' k-tiles go from memory into LDS by direct-to-LDS loads (a wave instruction
+// copies 64 x 16 bytes to one LDS address + 16 bytes a lane), not through registers: no
+// registers hold them on the way, and the stores into LDS and their waits are gone (1 to 2 %
+// at 2048 and 8192 tokens).  Such a copy lands as consecutive bytes, so instead of padded rows
+// the 16-byte pieces of a row are permuted (piece c of row r lies at place c ^ ((r >> 1) & 7)
+// of its 128 bytes): the 16 rows a quarter wave reads then fall into 16 different groups of
+// banks.  Two stages in two arrays, so that the compiler knows which reads wait for which
+// copies; the barrier is a bare s_barrier behind a wait that lets the W loads issued since
+// (younger than the copies) stay in flight.
+template <int BM, int BN, int WM, int WN, int EPI, int TKM = TK, bool W2 = false,
+          bool ADMA = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdirect_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
     int N, int K, int tiles_m, int tiles_n) {
@@ -360,9 +370,112 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
     const int grp = min(n / 16, N / 16 - 1);
     wbase[j] = W + (size_t)grp * (K / 64) * 1024 + ((lane / 32) * 64 + n % 16) * 8;
   }
-  u32x4_t areg[A_CHUNKS];
   u32x4_t wreg[W2 ? 2 : 1][TKM / 16][FN];
+  auto gload_w = [&](auto BUF, int kt, int ks) {
+    constexpr int B = decltype(BUF)::value;
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+      wreg[B][ks][j] = *(const u32x4_t*)(wbase[j] + ((size_t)kt * (TKM / 64) + ks / 4) * 1024 +
+                                      (ks % 4) * 128);
+  };
+  // gridDim.y workgroups share a tile's k-tiles (split-K for products with few tiles); each
+  // then leaves a float32 partial [gridDim.y, M, N] in Cv for skinny_reduce_kernel
+  const int kt_all = K / TKM;
+  const int kt0 = (int)((long long)blockIdx.y * kt_all / gridDim.y);
+  const int ktiles = (int)((long long)(blockIdx.y + 1) * kt_all / gridDim.y);
+  if (gridDim.y > 1) Cv = (float*)Cv + (size_t)blockIdx.y * M * N;
+  using Buf0 = std::integral_constant<int, 0>;
+  using Buf1 = std::integral_constant<int, 1>;
 
+  if constexpr (ADMA) {
+    static_assert(TKM == 64, "direct-to-LDS tokens: k-tiles of 64 (rows of 8 pieces)");
+    __shared__ u32x4_t a_stage0[BM * 8];
+    __shared__ u32x4_t a_stage1[BM * 8];
+    // the places this thread fills: place p = tid + c NT is row p / 8, slot p % 8, and takes
+    // piece slot ^ ((row >> 1) & 7) of the row's 128 bytes (rows beyond M: the last row)
+    uint32_t asrc[A_CHUNKS];
+#pragma unroll
+    for (int c = 0; c < A_CHUNKS; ++c) {
+      const int p = tid + c * NT, row = p / 8, piece = (p % 8) ^ ((row >> 1) & 7);
+      asrc[c] = (uint32_t)(min(m0 + row, M - 1) - m0) * (uint32_t)K + piece * 8;
+    }
+    const bf16_t* a_tile = A + (size_t)m0 * K;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);      // the LDS address is a scalar
+    auto dma_a = [&](int k0, u32x4_t* stage) {
+#pragma unroll
+      for (int c = 0; c < A_CHUNKS; ++c)
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(a_tile + k0 + asrc[c]),
+            (__attribute__((address_space(3))) void*)(stage + (wave_u * 64 + c * NT)), 16, 0, 0);
+    };
+    // the operand of MFMA row block i, k-step ks: row 32 i + lane % 32, piece 2 ks + lane / 32
+    int a_at[TKM / 16];
+#pragma unroll
+    for (int ks = 0; ks < TKM / 16; ++ks)
+      a_at[ks] = (wm * WM + lane % 32) * 8 + ((2 * ks + lane / 32) ^ (((lane % 32) >> 1) & 7));
+    // (in this order, kept by the scheduling barriers: the first step's wait counts on it)
+    dma_a(kt0 * TKM, a_stage0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < TKM / 16; ++ks) gload_w(Buf0{}, kt0, ks);
+    __builtin_amdgcn_sched_barrier(0);
+    if (W2) {
+#pragma unroll
+      for (int ks = 0; ks < TKM / 16; ++ks) gload_w(Buf1{}, min(kt0 + 1, ktiles - 1), ks);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // Before a step: its tokens' copies have landed (they are older than the (TKM / 16) * FN
+    // = 8 W loads issued since, which may stay in flight), then all waves meet: every wave
+    // has also read its last operands out of the other stage.
+    static_assert((TKM / 16) * FN == 8, "the wait counts a step's W loads");
+    auto meet = [&]() {
+      __builtin_amdgcn_s_waitcnt(0x0f78);     // vmcnt(8)
+      __builtin_amdgcn_s_barrier();
+    };
+    auto step = [&](int kt, const u32x4_t* cur, u32x4_t* other, auto BUF) {
+      constexpr int B = decltype(BUF)::value;
+      meet();
+      dma_a(min(kt + 1, ktiles - 1) * TKM, other);
+      const int wnxt = min(kt + (W2 ? 2 : 1), ktiles - 1);
+      __builtin_amdgcn_sched_barrier(0);
+      u32x4_t af[2][FM];
+#pragma unroll
+      for (int i = 0; i < FM; ++i) af[0][i] = cur[a_at[0] + i * 256];
+#pragma unroll
+      for (int ks = 0; ks < TKM / 16; ++ks) {
+        if (ks + 1 < TKM / 16) {
+#pragma unroll
+          for (int i = 0; i < FM; ++i) af[(ks + 1) % 2][i] = cur[a_at[ks + 1] + i * 256];
+        }
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                *(const bf16x8_t*)&af[ks % 2][i], *(const bf16x8_t*)&wreg[B][ks][j], acc[i][j],
+                0, 0, 0);
+        gload_w(BUF, wnxt, ks);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    if (W2) {       // an even number of k-tiles (the launch sees to it)
+      for (int kt = kt0; kt < ktiles; kt += 2) {
+        step(kt, a_stage0, a_stage1, Buf0{});
+        step(kt + 1, a_stage1, a_stage0, Buf1{});
+      }
+    } else {
+      int kt = kt0;
+      for (; kt + 1 < ktiles; kt += 2) {
+        step(kt, a_stage0, a_stage1, Buf0{});
+        step(kt + 1, a_stage1, a_stage0, Buf0{});
+      }
+      if (kt < ktiles) step(kt, a_stage0, a_stage1, Buf0{});
+    }
+    // the last step copied its own tile once more: nothing may still be on its way into LDS
+    // when the workgroup ends
+    __builtin_amdgcn_s_waitcnt(0x0f70);       // vmcnt(0)
+  } else {
+  u32x4_t areg[A_CHUNKS];
   auto gload_a = [&](int k0) {
 #pragma unroll
     for (int c = 0; c < A_CHUNKS; ++c) {
@@ -371,13 +484,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
       const int m = min(m0 + row, M - 1);
       areg[c] = *(const u32x4_t*)(A + (size_t)m * K + k0 + kc);
     }
-  };
-  auto gload_w = [&](auto BUF, int kt, int ks) {
-    constexpr int B = decltype(BUF)::value;
-#pragma unroll
-    for (int j = 0; j < FN; ++j)
-      wreg[B][ks][j] = *(const u32x4_t*)(wbase[j] + ((size_t)kt * (TKM / 64) + ks / 4) * 1024 +
-                                      (ks % 4) * 128);
   };
   auto lstore = [&](int stage) {
     bf16_t* a_s = lds + stage * BM * LROW;
@@ -389,14 +495,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
     }
   };
 
-  // gridDim.y workgroups share a tile's k-tiles (split-K for products with few tiles); each
-  // then leaves a float32 partial [gridDim.y, M, N] in Cv for skinny_reduce_kernel
-  const int kt_all = K / TKM;
-  const int kt0 = (int)((long long)blockIdx.y * kt_all / gridDim.y);
-  const int ktiles = (int)((long long)(blockIdx.y + 1) * kt_all / gridDim.y);
-  if (gridDim.y > 1) Cv = (float*)Cv + (size_t)blockIdx.y * M * N;
-  using Buf0 = std::integral_constant<int, 0>;
-  using Buf1 = std::integral_constant<int, 1>;
   gload_a(kt0 * TKM);
 #pragma unroll
   for (int ks = 0; ks < TKM / 16; ++ks) gload_w(Buf0{}, kt0, ks);
@@ -453,6 +551,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
     }
   } else {
     for (int kt = kt0; kt < ktiles; ++kt) step(kt, (kt - kt0) & 1, Buf0{});
+  }
   }
 
   // Epilogue through LDS: a 32x32 MFMA result has a lane's 16 values in 16 different rows,
@@ -531,7 +630,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
 static int launch_reduce(const void* ws, void* C, int M, int N, int ksplit, int epi,
                          hipStream_t stream);
 
-template <int BM, int BN, int WM, int WN, int TKM = TK, bool W2 = false>
+template <int BM, int BN, int WM, int WN, int TKM = TK, bool W2 = false, bool ADMA = false>
 static int launch_tile_wdirect(const void* A, const void* W, void* C, int M, int N, int K, int epi,
                                hipStream_t stream, void* ws = nullptr, int ksplit = 1,
                                bool reduce = true) {
@@ -544,10 +643,11 @@ static int launch_tile_wdirect(const void* A, const void* W, void* C, int M, int
   const int final_epi = epi;
   constexpr size_t stages = (size_t)2 * BM * (TKM + 8) * sizeof(bf16_t);
   constexpr size_t slabs = (size_t)(BM / WM) * (BN / WN) * 32 * (WN + 4) * sizeof(float);
-  const size_t smem = stages > slabs ? stages : slabs;
+  // (with the tokens copied straight into LDS the stages are arrays of the kernel's own)
+  const size_t smem = ADMA ? slabs : stages > slabs ? stages : slabs;
 #define ZF_WD(E)                                                                              \
   do {                                                                                        \
-    auto kern = gemm_bf16_tile_wdirect_kernel<BM, BN, WM, WN, E, TKM, W2>;                             \
+    auto kern = gemm_bf16_tile_wdirect_kernel<BM, BN, WM, WN, E, TKM, W2, ADMA>;              \
     if (smem > 64 * 1024) {                                                                   \
       hipError_t e = hipFuncSetAttribute((const void*)kern,                                   \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
@@ -599,20 +699,34 @@ static int launch_tile(const void* A, const void* W, void* C, int M, int N, int 
 // variant, plain W: 0 = 128x128 (waves 64x64), 4 = 256x256 (waves 128x64, 8 waves);
 //          pre-tiled W (w_tiled; N % 16 == 0 and K % 64 == 0), taken straight from memory
 //          into the MFMA operands: 6 = 128x128 (waves 64x64), 16 = 128x128 with k-tiles of 128
-//          and the waves side by side (128x32: for few tiles; K % 128 == 0), 10 = 128x256 (waves 128x64: no
-//          two waves load the same part of W, two workgroups share a CU, and W is loaded
-//          two k-tiles ahead when their number is even)
+//          and the waves side by side (128x32: for few tiles; K % 128 == 0), 10 = 128x256
+//          (waves 128x64: no two waves load the same part of W, two workgroups share a CU,
+//          and W is loaded two k-tiles ahead when their number is even).  10 copies the
+//          tokens straight into LDS, and so does 6 from 512 tiles on: with two workgroups or
+//          more to a CU that was 2 to 10 % faster (2048 tokens), with fewer 10 to 34 % slower
+//          (512 tokens: nothing hides the copies' longer way).  7 and 11 are the tiles of 6
+//          and 10 with the tokens through registers, for comparison.
 extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, int N, int K,
                                  int epi, int variant, int w_tiled, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K % 8 != 0 || (epi == EPI_SWIGLU && N % 32 != 0)) return -3;
   if (w_tiled) {
     if (N % 16 != 0 || K % 64 != 0) return -3;
-    if (variant == 6) return launch_tile_wdirect<128, 128, 64, 64>(A, W, C, M, N, K, epi, stream);
+    if (variant == 6 && (long long)((M + 127) / 128) * ((N + 127) / 128) >= 512)
+      return launch_tile_wdirect<128, 128, 64, 64, TK, false, true>(A, W, C, M, N, K, epi, stream);
+    if (variant == 6 || variant == 7)
+      return launch_tile_wdirect<128, 128, 64, 64>(A, W, C, M, N, K, epi, stream);
     if (variant == 16)
       return launch_tile_wdirect<128, 128, 128, 32, 128>(A, W, C, M, N, K, epi, stream);
     if (variant == 10) {
       if (K % (2 * TK) == 0)     // W two k-tiles ahead: an even number of k-tiles
+        return launch_tile_wdirect<128, 256, 128, 64, TK, true, true>(A, W, C, M, N, K, epi,
+                                                                      stream);
+      return launch_tile_wdirect<128, 256, 128, 64, TK, false, true>(A, W, C, M, N, K, epi,
+                                                                     stream);
+    }
+    if (variant == 11) {       // as 10, the tokens through registers into LDS
+      if (K % (2 * TK) == 0)
         return launch_tile_wdirect<128, 256, 128, 64, TK, true>(A, W, C, M, N, K, epi, stream);
       return launch_tile_wdirect<128, 256, 128, 64>(A, W, C, M, N, K, epi, stream);
     }
