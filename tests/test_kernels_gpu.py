@@ -849,24 +849,30 @@ def test_cast_and_poison_pages():
         assert bad[:, [0, 4, 7]].all() and not bad[:, [1, 2, 3, 5, 6, 8]].any()
 
 
-@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("variant", [1, 2, 3])
 @pytest.mark.parametrize("nH,nKV,hd,ps,window", [
     (8, 2, 128, 16, 0), (10, 2, 128, 16, 0), (16, 2, 64, 32, 0), (3, 1, 128, 48, 0),
-    (2, 2, 64, 16, 0), (18, 2, 128, 16, 0), (8, 2, 128, 16, 150), (5, 1, 64, 16, 64)])
+    (2, 2, 64, 16, 0), (18, 2, 128, 16, 0), (8, 2, 128, 16, 150), (5, 1, 64, 16, 64),
+    (4, 2, 128, 16, 0), (6, 2, 64, 16, 90)])
 def test_both_prefill_kernels_on_portions_and_whole_prompts(nH, nKV, hd, ps, window, variant):
-    """Each of the two MFMA prefill kernels, chosen by hand, over groups of 1, 3, 4, 5, 8 and 9
-    query heads (9: two blocks of heads per kv head), whole prompts and portions whose keys
-    end at, before and after the edges of 64-key tiles, pages of 16, 32 and 48 rows in a
-    shuffled pool whose unwritten rows are NaN, with and without the engine's list of tiles."""
+    """Each MFMA prefill kernel, chosen by hand (1: every wave fetches its own keys and values;
+    2: staged in LDS, with two groups of waves on the even and the odd key tiles where four
+    heads or fewer share a kv head and the prompts are whole; 3: staged, one group), over
+    groups of 1, 2, 3, 4, 5, 8 and 9 query heads (9: two blocks of heads per kv head):
+    portions whose keys end at, before and after the edges of 64-key tiles, and whole prompts
+    with odd and even numbers of key tiles; pages of 16, 32 and 48 rows in a shuffled pool
+    whose unwritten rows are NaN, with and without the engine's list of tiles."""
     dtype = torch.bfloat16
-    ctx_lens = [64, 65, 127, 128, 129, 300, 1000, 40, 2]
-    q_lens = [64, 65, 127, 64, 2, 237, 130, 7, 2]
-    s = _paged_setup(dtype, nH, nKV, hd, ps, ctx_lens, q_lens, seed=41)
-    for hint in (False, True):
-        got, want = _run_attention(s, dtype, nH, nKV, hd, ps, window, q_lens, ctx_lens,
-                                   tiles_hint=hint, variant=variant)
-        assert not torch.isnan(got.float()).any(), "a row outside the context was read"
-        assert rel_err(got, want) <= 2 * tol(dtype)
+    for ctx_lens, q_lens in (([64, 65, 127, 128, 129, 300, 1000, 40, 2],
+                              [64, 65, 127, 64, 2, 237, 130, 7, 2]),
+                             ([64, 65, 128, 129, 192, 193, 300, 700, 2],
+                              [64, 65, 128, 129, 192, 193, 300, 700, 2])):
+        s = _paged_setup(dtype, nH, nKV, hd, ps, ctx_lens, q_lens, seed=41)
+        for hint in (False, True):
+            got, want = _run_attention(s, dtype, nH, nKV, hd, ps, window, q_lens, ctx_lens,
+                                       tiles_hint=hint, variant=variant)
+            assert not torch.isnan(got.float()).any(), "a row outside the context was read"
+            assert rel_err(got, want) <= 2 * tol(dtype)
 
 
 @pytest.mark.parametrize("nH,nKV,hd,window", [(10, 2, 128, 0), (8, 1, 64, 0), (4, 1, 128, 0),

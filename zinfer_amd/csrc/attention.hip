@@ -717,7 +717,12 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(
 // lane, the loads of a tile and their address arithmetic are shared by the heads of the group.
 // The stages are two arrays, not one indexed array: the compiler then knows that reads of one
 // stage do not wait for the loads into the other.
-template <int HD, bool POW2>
+// KS = 2 (up to four heads in the block): the workgroup's waves form two groups with stages of
+// their own that take the even and the odd key tiles of the same heads and combine their
+// partials through LDS at the end, in a fixed order.  The kernel's time follows the longest
+// chain of dependent key tiles (the last query tile under the causal bound), which gets half
+// as long; used where the grid fills the chip only once or twice (short prompts).
+template <int HD, bool POW2, int KS>
 __global__ __launch_bounds__(512) void attn_prefill_shared_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int* __restrict__ block_table,
@@ -730,8 +735,11 @@ __global__ __launch_bounds__(512) void attn_prefill_shared_kernel(
   constexpr int TILE_CHUNKS = 4 * GROUP_CHUNKS;  // of 64 rows: keys first, then values
   __shared__ u32x4_t stage0[2 * TILE_CHUNKS];
   __shared__ u32x4_t stage1[2 * TILE_CHUNKS];
-  auto page_of = [&](int key) { return POW2 ? key >> ps_shift : key / ps; };
-  auto row_of = [&](int key) { return POW2 ? key & (ps - 1) : key % ps; };
+  __shared__ u32x4_t stage2[KS == 2 ? 2 * TILE_CHUNKS : 1];      // the second group's
+  __shared__ u32x4_t stage3[KS == 2 ? 2 * TILE_CHUNKS : 1];
+  __shared__ float other_ml[KS == 2 ? 4 : 1][64][2];
+  auto page_of = [&](int key) __attribute__((always_inline)) { return POW2 ? key >> ps_shift : key / ps; };
+  auto row_of = [&](int key) __attribute__((always_inline)) { return POW2 ? key & (ps - 1) : key % ps; };
   const int kvh = blockIdx.x % nKV;
   const int hb = (blockIdx.x / nKV) % head_blocks;
   const int entry = blockIdx.x / (nKV * head_blocks);
@@ -758,47 +766,56 @@ __global__ __launch_bounds__(512) void attn_prefill_shared_kernel(
   const int k_lo = gridDim.y > 1 ? max(lo_min, (int)blockIdx.y * split_keys) : lo_min;
   const int k_hi = gridDim.y > 1 ? min(p_max, ((int)blockIdx.y + 1) * split_keys - 1) : p_max;
   if (k_lo > k_hi) return;      // uniform over the workgroup: before any barrier
-  const int g = hb * nwaves + wave;
+  // waves per key group (= heads of the block), this wave's group and its place in it
+  const int gw = nwaves / KS, kgrp = wave / gw, wv = wave % gw;
+  const int g = hb * gw + wv;
   const bool active = g < G;
   const int head = kvh * G + min(g, G - 1);
 
   // groups of 16 rows that hold live keys of this request: every load is clamped into them
   const int lo_grp = (lo_min / 16) * 16, hi_grp = (p_max / 16) * 16;
-  auto source_of = [&](int base) { return min(max(base, lo_grp), hi_grp); };
+  auto source_of = [&](int base) __attribute__((always_inline)) { return min(max(base, lo_grp), hi_grp); };
   // pool offsets in 16-byte pieces: a page holds nKV * ps * HD / 8 of them
   const int gpp = ps / 16;                       // groups of 16 rows in a page
   const uint32_t page_chunks = (uint32_t)nKV * ps * (HD / 8);
   const uint32_t head_chunks = (uint32_t)kvh * ps * (HD / 8);
   const u32x4_t* k_chunks = (const u32x4_t*)k_pool;
   const u32x4_t* v_chunks = (const u32x4_t*)v_pool;
-  auto issue = [&](int kb, u32x4_t* stage) {
-    // where the tile's four groups of 16 rows lie in the pools: four scalar look-ups in flight
-    // together, then the copies
-    int gi[4], pg[4];
-#pragma unroll
-    for (int grp = 0; grp < 4; ++grp) gi[grp] = source_of(kb + 16 * grp) / 16;
-#pragma unroll
-    for (int grp = 0; grp < 4; ++grp) pg[grp] = table[POW2 ? gi[grp] >> (ps_shift - 4) : gi[grp] / gpp];
+  // The pages of the four groups of 16 rows of the tile at kb: lane i (mod 4) looks up group
+  // i's.  A vector load, so that it is waited for with the tile's copies at the end of the
+  // tile, a whole tile after it was asked for (as scalar loads the look-ups were waited for
+  // at the next LDS read: some 600 cycles of every tile).
+  auto pages_of = [&](int kb) __attribute__((always_inline)) {
+    const int gi = source_of(kb + 16 * (lane & 3)) / 16;
+    return table[POW2 ? gi >> (ps_shift - 4) : gi / gpp];
+  };
+  // Copies the tile at kb into `stage`; its pages were looked up a tile earlier (pg_lanes),
+  // and the pages of this group's tile after it are looked up now.
+  int pg_lanes = 0;
+  auto issue = [&](int kb, u32x4_t* stage) __attribute__((always_inline)) {
     uint64_t at[4];
 #pragma unroll
-    for (int grp = 0; grp < 4; ++grp)
-      at[grp] = (uint64_t)(uint32_t)pg[grp] * page_chunks + head_chunks +
-                (uint32_t)(POW2 ? gi[grp] & (gpp - 1) : gi[grp] % gpp) * GROUP_CHUNKS;
-    for (int c0 = wave * 64; c0 < TILE_CHUNKS; c0 += 64 * nwaves) {
+    for (int grp = 0; grp < 4; ++grp) {
+      const int gi = source_of(kb + 16 * grp) / 16;
+      at[grp] = (uint64_t)(uint32_t)__builtin_amdgcn_readlane(pg_lanes, grp) * page_chunks +
+                head_chunks + (uint32_t)(POW2 ? gi & (gpp - 1) : gi % gpp) * GROUP_CHUNKS;
+    }
+    if (kb + 64 * KS <= k_hi) pg_lanes = pages_of(kb + 64 * KS);
+    for (int c0 = wv * 64; c0 < TILE_CHUNKS; c0 += 64 * gw) {
       const int grp = c0 / GROUP_CHUNKS;
-      const uint64_t base = grp == 0 ? at[0] : grp == 1 ? at[1] : grp == 2 ? at[2] : at[3];
-      const uint64_t from = base + (uint32_t)(c0 % GROUP_CHUNKS + lane);
+      const uint64_t base = (grp == 0 ? at[0] : grp == 1 ? at[1] : grp == 2 ? at[2] : at[3]) +
+                            (uint32_t)(c0 % GROUP_CHUNKS);
       __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)(k_chunks + from),
+          (const __attribute__((address_space(1))) void*)(k_chunks + base + lane),
           (__attribute__((address_space(3))) void*)(stage + c0), 16, 0, 0);
       __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)(v_chunks + from),
+          (const __attribute__((address_space(1))) void*)(v_chunks + base + lane),
           (__attribute__((address_space(3))) void*)(stage + TILE_CHUNKS + c0), 16, 0, 0);
     }
   };
   // the loads into LDS count as vector-memory operations: all of this wave's have landed,
   // then all waves meet
-  auto landed = [&]() {
+  auto landed = [&]() __attribute__((always_inline)) {
     __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0)
     __syncthreads();
   };
@@ -825,12 +842,9 @@ __global__ __launch_bounds__(512) void attn_prefill_shared_kernel(
 
   // one tile out of `stage`; the next one is requested into `next` once this tile's first
   // products are under way (every wave has left `next` behind at the barrier before)
-  auto tile = [&](int kb, const u32x4_t* stage, u32x4_t* next) {
-    if (!active) {
-      if (kb + 64 <= k_hi) issue(kb + 64, next);
-      return;
-    }
-    if (kb + 64 <= k_hi) issue(kb + 64, next);
+  auto tile = [&](int kb, const u32x4_t* stage, u32x4_t* next) __attribute__((always_inline)) {
+    if (kb + 64 * KS <= k_hi) issue(kb + 64 * KS, next);     // this group's next tile
+    if (!active) return;
     const u32x4_t* sk = stage + k_at;
     const u32x2_t* sv = (const u32x2_t*)(stage + TILE_CHUNKS) + v_at;
     f32x16_t st[2];
@@ -870,14 +884,14 @@ __global__ __launch_bounds__(512) void attn_prefill_shared_kernel(
       if (__builtin_expect(!__any(tmax > m_ref + 20.f), 1)) {
         m = m_ref;
         float psum = 0.f;
-        auto terms = [&](int h) {
+        auto terms = [&](int h) __attribute__((always_inline)) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             st[h][r] = exp2_raw(fmaf(st[h][r], scale_log2e, -m_ref));
             psum += st[h][r];
           }
         };
-        auto values = [&](int h) {
+        auto values = [&](int h) __attribute__((always_inline)) {
 #pragma unroll
           for (int u = 0; u < 2; ++u) {
             u32x4_t pk = u32x4_t{pack_bf16(st[h][8 * u + 0], st[h][8 * u + 1]),
@@ -962,7 +976,7 @@ __global__ __launch_bounds__(512) void attn_prefill_shared_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) o[dt][r] *= corr;
     }
-    auto packed = [&](int h, int u) {
+    auto packed = [&](int h, int u) __attribute__((always_inline)) {
       // slots e = 0..7 <-> st[h][8 u + e]: keys base + 4 hf + e (e < 4) and
       // base + 8 + 4 hf + (e - 4), base = kb + 32 h + 16 u
       u32x4_t pk = u32x4_t{pack_bf16(st[h][8 * u + 0], st[h][8 * u + 1]),
@@ -1016,15 +1030,50 @@ __global__ __launch_bounds__(512) void attn_prefill_shared_kernel(
     }
   };
 
+  // group r takes the tiles kb0 + 64 (KS i + r); every wave comes by every barrier (the
+  // loop's bounds are the first group's)
   const int kb0 = (k_lo / 64) * 64;
-  issue(kb0, stage0);
-  landed();
-  for (int kb = kb0; kb <= k_hi; kb += 128) {
-    tile(kb, stage0, stage1);
+  auto run = [&](u32x4_t* sa, u32x4_t* sb) __attribute__((always_inline)) {
+    const int off = 64 * kgrp;
+    if (kb0 + off <= k_hi) {
+      pg_lanes = pages_of(kb0 + off);
+      issue(kb0 + off, sa);
+    }
     landed();
-    if (kb + 64 > k_hi) break;
-    tile(kb + 64, stage1, stage0);
-    landed();
+    for (int kb = kb0; kb <= k_hi; kb += 128 * KS) {
+      if (kb + off <= k_hi) tile(kb + off, sa, sb);
+      landed();
+      if (kb + 64 * KS > k_hi) break;
+      if (kb + 64 * KS + off <= k_hi) tile(kb + 64 * KS + off, sb, sa);
+      landed();
+    }
+  };
+  if (KS == 1 || kgrp == 0) run(stage0, stage1);
+  else run(stage2, stage3);
+  if (KS == 2) {
+    // the second group's partials go through its own stages (64 floats of O^T a lane: half a
+    // stage a wave) to the wave of the first group with the same head
+    float* spot = (float*)((wv < 2 ? stage2 : stage3) + (wv % 2) * TILE_CHUNKS) + lane;
+    if (kgrp == 1) {
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) spot[(dt * 16 + r) * 64] = o[dt][r];
+      other_ml[wv][lane][0] = m;
+      other_ml[wv][lane][1] = l;
+    }
+    __syncthreads();
+    if (kgrp == 1) return;
+    const float m_b = other_ml[wv][lane][0], l_b = other_ml[wv][lane][1];
+    const float m_new = fmaxf(m, m_b);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float ca = exp2f(m - m_use), cb = exp2f(m_b - m_use);
+    l = l * ca + l_b * cb;
+    m = m_new;
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[dt][r] = o[dt][r] * ca + spot[(dt * 16 + r) * 64] * cb;
   }
   if (!active || !q_valid) return;
   if (gridDim.y > 1) {
@@ -1103,7 +1152,8 @@ __global__ __launch_bounds__(64) void attn_prefill_merge_kernel(
 // are split over workgroups and merged by a second kernel.
 // variant: 0 chooses; 1 the kernel whose waves fetch their own keys and values; 2 the kernel
 // that stages them in LDS for the heads of a group (head sizes 64 and 128, splits of a
-// multiple of 64 keys), -2 where it does not apply.
+// multiple of 64 keys), -2 where it does not apply; 3 the same without the two groups of
+// waves on the even and the odd key tiles.
 extern "C" int zf_attn_prefill_bf16(const void* q, const void* k_pool, const void* v_pool,
                                     const int* block_table, const int* q_start,
                                     const int* ctx_len, void* out, float scale, int window,
@@ -1115,7 +1165,7 @@ extern "C" int zf_attn_prefill_bf16(const void* q, const void* k_pool, const voi
                                     hipStream_t stream) {
   if (n_seqs <= 0 || max_q_len <= 0) return 0;
   if (page_size % 16 != 0 || nKV <= 0 || nH % nKV != 0) return -2;
-  if (variant < 0 || variant > 2) return -2;
+  if (variant < 0 || variant > 3) return -2;
   if (split_keys > 0 && (split_keys % 32 != 0 || max_splits < 1 || ws_o == nullptr ||
                          ws_ml == nullptr || seq_index == nullptr))
     return -2;
@@ -1131,20 +1181,33 @@ extern "C" int zf_attn_prefill_bf16(const void* q, const void* k_pool, const voi
   // at every length from 512 tokens to 16 K, 1.1 to 1.9 times); a lone head would be one wave
   // per workgroup and stays with the first kernel, whose waves split its key tiles
   const bool shared_ok = (hd == 64 || hd == 128) && split_keys % 64 == 0;
-  if (variant == 2 && !shared_ok) return -2;
-  if (variant == 2 || (variant == 0 && shared_ok && G >= 2)) {
-    const int waves = G < 8 ? G : 8, head_blocks = (G + waves - 1) / waves;
+  if ((variant == 2 || variant == 3) && !shared_ok) return -2;
+  if (variant == 2 || variant == 3 || (variant == 0 && shared_ok && G >= 2)) {
+    const int heads = G < 8 ? G : 8, head_blocks = (G + heads - 1) / heads;
     dim3 sgrid(entries * head_blocks * nKV, split_keys > 0 ? max_splits : 1);
-#define ZF_PRE_S(HD, POW2)                                                                      \
-  hipLaunchKernelGGL((attn_prefill_shared_kernel<HD, POW2>), sgrid, dim3(64 * waves), 0, stream, \
+    // two groups of waves on the even and the odd key tiles where the heads leave room for
+    // them and the longest chain of tiles sets the time: short contexts before the portions
+    // (allow_split) and a grid that fills the chip at most twice.  (8 K keys before a
+    // 2048-token portion: 14 % slower with them; a whole 2048-token prompt: 73 -> 63 us with 4
+    // heads per kv head, 66 -> 45 us with 2.)
+    const int ks = (variant != 3 && heads <= 4 && split_keys == 0 && allow_split && sgrid.x <= 1024) ? 2 : 1;
+    const dim3 sblock(64 * heads * ks);
+#define ZF_PRE_S(HD, POW2, KS)                                                                  \
+  hipLaunchKernelGGL((attn_prefill_shared_kernel<HD, POW2, KS>), sgrid, sblock, 0, stream,      \
                      (const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool,            \
                      block_table, q_start, ctx_len, (bf16_t*)out, scale_log2e, window, nH, nKV, \
                      page_size, max_pages, skip_single, q_tiles, head_blocks, ps_shift, ws_o,   \
                      ws_ml, split_keys, max_splits, tile_map)
-    if (hd == 64 && ps_shift >= 0) ZF_PRE_S(64, true);
-    else if (hd == 64) ZF_PRE_S(64, false);
-    else if (ps_shift >= 0) ZF_PRE_S(128, true);
-    else ZF_PRE_S(128, false);
+#define ZF_PRE_SK(HD, POW2)                                                                     \
+  do {                                                                                          \
+    if (ks == 2) ZF_PRE_S(HD, POW2, 2);                                                         \
+    else ZF_PRE_S(HD, POW2, 1);                                                                 \
+  } while (0)
+    if (hd == 64 && ps_shift >= 0) ZF_PRE_SK(64, true);
+    else if (hd == 64) ZF_PRE_SK(64, false);
+    else if (ps_shift >= 0) ZF_PRE_SK(128, true);
+    else ZF_PRE_SK(128, false);
+#undef ZF_PRE_SK
 #undef ZF_PRE_S
     if (split_keys > 0)
       hipLaunchKernelGGL(attn_prefill_merge_kernel, dim3(n_tokens, nH), dim3(64), 0, stream,
