@@ -435,7 +435,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
     auto step = [&](int kt, const u32x4_t* cur, u32x4_t* other, auto BUF) {
       constexpr int B = decltype(BUF)::value;
       meet();
-      dma_a(min(kt + 1, ktiles - 1) * TKM, other);
       const int wnxt = min(kt + (W2 ? 2 : 1), ktiles - 1);
       __builtin_amdgcn_sched_barrier(0);
       u32x4_t af[2][FM];
@@ -454,6 +453,15 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
                 *(const bf16x8_t*)&af[ks % 2][i], *(const bf16x8_t*)&wreg[B][ks][j], acc[i][j],
                 0, 0, 0);
+        if (ks == 0) {
+          // the next tile's copies, behind the first k-step's MFMAs: issuing a copy holds
+          // the wave for some 60 cycles, which now pass while those MFMAs run (gate/up at
+          // 2048 tokens: 361 -> 347 us); still older than this step's W loads, as the wait
+          // at the next step's start counts on
+          __builtin_amdgcn_sched_barrier(0);
+          dma_a(min(kt + 1, ktiles - 1) * TKM, other);
+          __builtin_amdgcn_sched_barrier(0);
+        }
         gload_w(BUF, wnxt, ks);
         __builtin_amdgcn_sched_barrier(0);
       }
