@@ -710,17 +710,18 @@ static int launch_tile(const void* A, const void* W, void* C, int M, int N, int 
 //          and the waves side by side (128x32: for few tiles; K % 128 == 0), 10 = 128x256
 //          (waves 128x64: no two waves load the same part of W, two workgroups share a CU,
 //          and W is loaded two k-tiles ahead when their number is even).  10 copies the
-//          tokens straight into LDS, and so does 6 from 512 tiles on: with two workgroups or
-//          more to a CU that was 2 to 10 % faster (2048 tokens), with fewer 10 to 34 % slower
-//          (512 tokens: nothing hides the copies' longer way).  7 and 11 are the tiles of 6
-//          and 10 with the tokens through registers, for comparison.
+//          tokens straight into LDS, and so does 6 from 384 tiles on: with two workgroups to
+//          most CUs that was 2 to 18 % faster (qkv at 1024 and 2048 tokens), with one 10 to
+//          34 % slower (512 tokens, or 256 tiles at 1024: nothing hides the copies' longer
+//          way).  7 and 11 are the tiles of 6 and 10 with the tokens through registers, for
+//          comparison.
 extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, int N, int K,
                                  int epi, int variant, int w_tiled, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K % 8 != 0 || (epi == EPI_SWIGLU && N % 32 != 0)) return -3;
   if (w_tiled) {
     if (N % 16 != 0 || K % 64 != 0) return -3;
-    if (variant == 6 && (long long)((M + 127) / 128) * ((N + 127) / 128) >= 512)
+    if (variant == 6 && (long long)((M + 127) / 128) * ((N + 127) / 128) >= 384)
       return launch_tile_wdirect<128, 128, 64, 64, TK, false, true>(A, W, C, M, N, K, epi, stream);
     if (variant == 6 || variant == 7)
       return launch_tile_wdirect<128, 128, 64, 64>(A, W, C, M, N, K, epi, stream);
