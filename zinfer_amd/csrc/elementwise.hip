@@ -227,7 +227,7 @@ __global__ void qk_norm_rope_kv_write_kernel(
 // takes 64 / LPH heads of one token, so that loads and stores are 8 or 16 bytes wide and
 // there are far fewer waves than (token, head) pairs.
 template <typename T, int LPH>
-__global__ __launch_bounds__(64) void qk_norm_rope_kv_write_vec_kernel(
+__global__ __launch_bounds__(256) void qk_norm_rope_kv_write_vec_kernel(
     T* __restrict__ qkv, const float* __restrict__ q_gain, const float* __restrict__ k_gain,
     float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int* __restrict__ positions, const int* __restrict__ slot_mapping,
@@ -235,8 +235,10 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_vec_kernel(
     int hd, int page_size, int tiled) {
   constexpr int HPW = 64 / LPH;
   const int t = blockIdx.x;
-  const int lane = threadIdx.x, li = lane % LPH;
-  const int head = blockIdx.y * HPW + lane / LPH;
+  const int lane = threadIdx.x % 64, li = lane % LPH;
+  // four waves to a workgroup (a quarter of the workgroups to hand out: 2048 tokens of 48
+  // heads took 25 us as 24576 workgroups of one wave)
+  const int head = (blockIdx.y * 4 + threadIdx.x / 64) * HPW + lane / LPH;
   const int half = hd / 2;
   const bool active = head < nH + 2 * nKV && 4 * li < half;
   const int row_width = (nH + 2 * nKV) * hd;
@@ -336,7 +338,7 @@ static void launch_qk_vec(T* qkv, const float* q_gain, const float* k_gain, floa
   const int lanes = hd / 8, heads = nH + 2 * nKV;
 #define ZF_QKV(LPH)                                                                            \
   hipLaunchKernelGGL((qk_norm_rope_kv_write_vec_kernel<T, LPH>),                               \
-                     dim3(Tn, (heads + 64 / LPH - 1) / (64 / LPH)), dim3(64), 0, stream, qkv,  \
+                     dim3(Tn, (heads + 256 / LPH - 1) / (256 / LPH)), dim3(256), 0, stream, qkv, \
                      q_gain, k_gain, eps, cos_t, sin_t, positions, slot_mapping, k_pool,       \
                      v_pool, q_out, nH, nKV, hd, page_size, tiled)
   if (lanes <= 2) ZF_QKV(2);
