@@ -212,23 +212,58 @@ def test_gemm_many_large_tiles(kind, K, M, N, variant):
     ops = _ops()
     assert ops._tile_variant(M, N, True, kind == "accumulate", K) == variant
     assert variant == 10 or ((M + 127) // 128) * ((N + 127) // 128) >= 384
-    a = _rand((M, K), torch.bfloat16, 35)
-    w = _rand((N, K), torch.bfloat16, 36, 0.05)
+    _check_tiled(ops, kind, M, N, K, variant)
+
+
+def _check_tiled(ops, kind, M, N, K, variant, seed=35):
+    """One tiled kernel on pre-tiled W against the plain product."""
+    a = _rand((M, K), torch.bfloat16, seed)
+    w = _rand((N, K), torch.bfloat16, seed + 1, 0.05)
     if kind == "swiglu":
         wi = ops.interleave_gate_up(w[:N // 2].to(DEV), w[N // 2:].to(DEV))
         want = torch.empty((M, N // 2), dtype=torch.bfloat16)
         ref.gemm_swiglu(a, wi.cpu(), want)
         got = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
-        ops.gemm_swiglu(a.to(DEV), ops.pretile_weight(wi), got, w_tiled=True)
+        ops.gemm_swiglu(a.to(DEV), ops.pretile_weight(wi), got, w_tiled=True, tile_variant=variant)
         assert rel_err(got, want) <= tol(torch.bfloat16)
         return
     acc = kind == "accumulate"
-    base = _rand((M, N), torch.float32, 37).to(torch.float32 if acc else torch.bfloat16)
+    base = _rand((M, N), torch.float32, seed + 2).to(torch.float32 if acc else torch.bfloat16)
     want = base.clone()
     ref.gemm(a, w, want, acc)
     got = base.clone().to(DEV)
-    ops.gemm(a.to(DEV), ops.pretile_weight(w.to(DEV)), got, acc, w_tiled=True)
+    ops.gemm(a.to(DEV), ops.pretile_weight(w.to(DEV)), got, acc, w_tiled=True, tile_variant=variant)
     assert rel_err(got, want) <= (2e-5 if acc else tol(torch.bfloat16))
+
+
+@pytest.mark.parametrize("kind", ["store", "accumulate", "swiglu"])
+@pytest.mark.parametrize("M,N,K,variant", [
+    (256, 256, 128, 20), (700, 640, 384, 20), (513, 448, 640, 20), (2100, 1600, 256, 20),
+    (256, 192, 128, 21), (1000, 960, 512, 21), (300, 576, 384, 21), (257, 832, 256, 21),
+    (256, 128, 128, 22), (999, 448, 256, 22), (513, 384, 640, 22), (300, 8192 + 64, 128, 22)])
+def test_gemm_256_token_tiles(kind, M, N, K, variant):
+    """The kernel with one 256-token tile per CU (256, 192 or 128 outputs wide): edges in M and
+    N that are no multiple of the tile, one to five rounds of its ring of four k-tiles, more
+    tiles than CUs, every epilogue."""
+    _check_tiled(_ops(), kind, M, N, K, variant, seed=41)
+
+
+def test_gemm_256_token_tiles_are_chosen_and_agree():
+    """Where the cost model picks the 256-token tiles the product goes through them, with the
+    same bits as through the 128-token tiles: the sums are added in the same order."""
+    ops = _ops()
+    for M, N, K in [(2048, 6144, 512), (1536, 6144, 256), (3072, 4096, 384)]:
+        variant = ops._tile256_variant(M, N, K)
+        assert variant in (20, 21, 22), (M, N, K, variant)
+        a = _rand((M, K), torch.bfloat16, 51).to(DEV)
+        wt = ops.pretile_weight(_rand((N, K), torch.bfloat16, 52, 0.05).to(DEV))
+        chosen = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+        forced = torch.empty_like(chosen)
+        small = torch.empty_like(chosen)
+        ops.gemm(a, wt, chosen, w_tiled=True)
+        ops.gemm(a, wt, forced, w_tiled=True, tile_variant=variant)
+        ops.gemm(a, wt, small, w_tiled=True, tile_variant=6)
+        assert torch.equal(chosen, forced) and torch.equal(chosen, small)
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64, 65, 200, 300])

@@ -304,6 +304,81 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_ker
     }
 }
 
+// Epilogue through LDS of the kernels whose waves hold 32-row x 32-column MFMA results: a
+// 32x32 result has a lane's 16 values in 16 different rows, so direct stores would be 2 or 4
+// bytes wide in runs of 64 bytes.  Each wave lays 32 rows of WN columns of its tile (the FN
+// column blocks from J0 on, at rows mw.., columns nw..) down in its own slab (32 rows of
+// WN + 4 floats) and reads them back along the rows, 16 bytes per lane.  All waves of the
+// workgroup call it together.
+template <int FM, int FN, int WN, int EPI, int J0 = 0, int FNALL = FN>
+__device__ __forceinline__ void store_through_slab(f32x16_t (&acc)[FM][FNALL], float* slab, int mw,
+                                                   int nw, int M, int N, void* Cv, int lane) {
+  static_assert(WN == 32 * FN && J0 + FN <= FNALL, "column blocks");
+  constexpr int SLAB_ROW = WN + 4;
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        slab[(8 * (r / 4) + 4 * (lane / 32) + r % 4) * SLAB_ROW + j * 32 + lane % 32] = acc[i][J0 + j][r];
+    __syncthreads();
+    if (EPI == EPI_SWIGLU) {
+      // 16 gate columns, then the 16 up columns that belong to them: 8 outputs per lane
+      constexpr int LPR = WN / 16;                  // lanes per row
+#pragma unroll
+      for (int it = 0; it < 32 * LPR / 64; ++it) {
+        const int row = it * (64 / LPR) + lane / LPR, q = lane % LPR;
+        const int m = mw + i * 32 + row;
+        const int c = (q / 2) * 32 + (q % 2) * 8;   // first gate column inside the wave's tile
+        const int n = nw + c;
+        if (m < M && n < N) {
+          const float* src = slab + row * SLAB_ROW + c;
+          const float4 g0 = *(const float4*)src, g1 = *(const float4*)(src + 4);
+          const float4 u0 = *(const float4*)(src + 16), u1 = *(const float4*)(src + 20);
+          const u32x4_t v = u32x4_t{
+              pack_bf16x2(swiglu_f(g0.x, u0.x), swiglu_f(g0.y, u0.y)),
+              pack_bf16x2(swiglu_f(g0.z, u0.z), swiglu_f(g0.w, u0.w)),
+              pack_bf16x2(swiglu_f(g1.x, u1.x), swiglu_f(g1.y, u1.y)),
+              pack_bf16x2(swiglu_f(g1.z, u1.z), swiglu_f(g1.w, u1.w))};
+          *(u32x4_t*)((bf16_t*)Cv + (size_t)m * (N / 2) + (n / 32) * 16 + (n % 32)) = v;
+        }
+      }
+    } else if (EPI == EPI_STORE_BF16) {
+      constexpr int LPR = WN / 8;
+#pragma unroll
+      for (int it = 0; it < 32 * LPR / 64; ++it) {
+        const int row = it * (64 / LPR) + lane / LPR, c = (lane % LPR) * 8;
+        const int m = mw + i * 32 + row, n = nw + c;
+        if (m < M && n < N) {
+          const float* src = slab + row * SLAB_ROW + c;
+          const float4 x0 = *(const float4*)src, x1 = *(const float4*)(src + 4);
+          const u32x4_t v = u32x4_t{pack_bf16x2(x0.x, x0.y), pack_bf16x2(x0.z, x0.w),
+                                    pack_bf16x2(x1.x, x1.y), pack_bf16x2(x1.z, x1.w)};
+          *(u32x4_t*)((bf16_t*)Cv + (size_t)m * N + n) = v;
+        }
+      }
+    } else {
+      constexpr int LPR = WN / 4;
+#pragma unroll
+      for (int it = 0; it < 32 * LPR / 64; ++it) {
+        const int row = it * (64 / LPR) + lane / LPR, c = (lane % LPR) * 4;
+        const int m = mw + i * 32 + row, n = nw + c;
+        if (m < M && n < N) {
+          float4 x = *(const float4*)(slab + row * SLAB_ROW + c);
+          float4* dst = (float4*)((float*)Cv + (size_t)m * N + n);
+          if (EPI == EPI_ACC_F32) {
+            const float4 old = *dst;
+            x = float4{old.x + x.x, old.y + x.y, old.z + x.z, old.w + x.w};
+          }
+          *dst = x;
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
 // ---------------------------------------------------------------- large M, pre-tiled W: W not staged
 // Tiles of BM tokens x BN outputs, k-tiles of TKM.  Only the tokens go through LDS; every wave
 // takes its W operands straight from the pre-tiled matrix (16-byte pieces that lie in runs of
@@ -562,75 +637,295 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
   }
   }
 
-  // Epilogue through LDS: a 32x32 MFMA result has a lane's 16 values in 16 different rows,
-  // so direct stores would be 2 or 4 bytes wide in runs of 64 bytes.  Each wave lays 32 rows
-  // of its tile down in its own slab (rows padded by 4 floats) and reads them back along the
-  // rows, 16 bytes per lane.  (The main loop's last barrier has freed the token stages.)
-  constexpr int SLAB_ROW = WN + 4;     // the launch sizes the LDS for stages and slabs
-  float* slab = (float*)lds_raw + (size_t)wave * 32 * SLAB_ROW;
-  const int mw = m0 + wm * WM, nw = n0 + wn * WN;
+  // (the main loop's last barrier has freed the token stages; the launch sizes the LDS for
+  // stages and slabs)
+  float* slab = (float*)lds_raw + (size_t)wave * 32 * (WN + 4);
+  store_through_slab<FM, FN, WN, EPI>(acc, slab, m0 + wm * WM, n0 + wn * WN, M, N, Cv, lane);
+}
+
+// ---------------------------------------------------------------- large M: 256-token tiles, one workgroup to a CU
+// Tiles of 256 tokens x BN outputs (128, 192 or 256), one workgroup of 4 waves (2 x 2) per
+// CU, each wave alone on its SIMD with a tile of 128 x BN / 2 (up to 256 accumulator
+// registers).  The kernel above moves (BM + BN) / (BM * BN) bytes per flop from L2 through a
+// CU's vector memory path, which at 128 x 256 tiles is as busy as the MFMAs; here it is half
+// to two thirds of that, and a wave's 16 MFMAs per k-step of 16 need 8 LDS reads of 16 bytes
+// a lane.  Both operands go from memory into LDS by direct-to-LDS loads, k-tiles of 32 in a
+// ring of 4 stages (separate arrays, so that the compiler knows which reads wait for which
+// copies): the tokens as rows of 64 bytes whose four 16-byte pieces are permuted (piece c
+// of row r at place c ^ ((r >> 2) & 3): the 16 rows a quarter wave reads fall into 16
+// different groups of banks), W as it lies in the pre-tiled matrix (16 outputs x 8 k are 256
+// consecutive bytes).  A step's operands of the first k-step of 16 are read at the end of
+// the step before; in the middle of a step the wave waits for the next tile's copies (those
+// of the two tiles behind it stay in flight), meets the others (which have then read all of
+// this step's tile), and the copies of the tile four ahead begin, into the stage just read.
+// A wave issues one instruction at a time, so what is not an MFMA follows single MFMAs,
+// evenly spread.  The sums are added in the same order as in the kernels above: the results
+// are the same bits.  (Keeping W out of LDS, every wave with its own operands in four
+// register sets and the waves side by side, runs at the same speed.)
+
+// which of a k-step's cnt loads follows MFMA m of nm (-1: none)
+constexpr int copy_after(int m, int nm, int cnt) {
+  for (int d = 0; d < cnt; ++d)
+    if (m == (d + 1) * nm / cnt - 1) return d;
+  return -1;
+}
+// how many of the nr operand reads have been issued before MFMA m: one behind every MFMA
+// without a load, and those that would be left over at the end behind the first as well
+constexpr int reads_before(int m, int nm, int cnt, int nr) {
+  int free_slots = 0;
+  for (int k = 0; k < nm; ++k) free_slots += copy_after(k, nm, cnt) < 0;
+  const int extra = nr > free_slots ? nr - free_slots : 0;
+  int done = 0;
+  for (int k = 0; k < m && done < nr; ++k)
+    if (copy_after(k, nm, cnt) < 0) done += 1 + (k == 0 ? extra : 0);
+  return done < nr ? done : nr;
+}
+
+template <int BN, int EPI>
+__global__ __launch_bounds__(256) void gemm_bf16_tile256_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
+    int N, int K, int tiles_m, int tiles_n) {
+  constexpr int BM = 256, NT = 256, WM = 128, WN = BN / 2, FM = WM / 32, FN = WN / 32;
+  static_assert(BN == 128 || BN == 192 || BN == 256, "tile width");
+  constexpr int A_PLACES = BM * 4, W_PLACES = BN * 4;    // 16-byte pieces of a k-tile of 32
+  constexpr int A_CHUNKS = A_PLACES / NT, W_CHUNKS = W_PLACES / NT;     // copies per thread
+  constexpr int CHUNKS = A_CHUNKS + W_CHUNKS;
+  constexpr int PART1 = (CHUNKS + 1) / 2;   // a tile's copies are issued in two parts
+  __shared__ u32x4_t stage0[A_PLACES + W_PLACES];
+  __shared__ u32x4_t stage1[A_PLACES + W_PLACES];
+  __shared__ u32x4_t stage2[A_PLACES + W_PLACES];
+  __shared__ u32x4_t stage3[A_PLACES + W_PLACES];
+  auto stage_of = [&](auto IDX) __attribute__((always_inline)) -> u32x4_t* {
+    constexpr int I = decltype(IDX)::value;
+    if constexpr (I == 0) return stage0;
+    else if constexpr (I == 1) return stage1;
+    else if constexpr (I == 2) return stage2;
+    else return stage3;
+  };
+
+  const int nblocks = tiles_m * tiles_n;
+  int b = blockIdx.x;
+  {
+    const int base = nblocks / 8, rem = nblocks % 8;
+    const int xcd = b % 8, idx = b / 8;
+    b = xcd * base + min(xcd, rem) + idx;
+  }
+  const int GROUP = 8;
+  const int in_group = GROUP * tiles_n;
+  const int first_m = (b / in_group) * GROUP;
+  const int gsize = min(tiles_m - first_m, GROUP);
+  const int tm = first_m + (b % in_group) % gsize;
+  const int tn = (b % in_group) / gsize;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int wm = wave / 2, wn = wave % 2;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);        // the LDS address is a scalar
+
+  f32x16_t acc[FM][FN];
 #pragma unroll
-  for (int i = 0; i < FM; ++i) {
+  for (int i = 0; i < FM; ++i)
 #pragma unroll
     for (int j = 0; j < FN; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        slab[(8 * (r / 4) + 4 * (lane / 32) + r % 4) * SLAB_ROW + j * 32 + lane % 32] = acc[i][j][r];
-    __syncthreads();
-    if (EPI == EPI_SWIGLU) {
-      // 16 gate columns, then the 16 up columns that belong to them: 8 outputs per lane
-      constexpr int LPR = WN / 16;                  // lanes per row
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // Sources, as a base all lanes share plus a 32-bit offset per lane.  Tokens: place p =
+  // tid + 256 c is row p / 4 = tid / 4 + 64 c, slot p % 4, and takes piece slot ^ ((row >> 2)
+  // & 3) of the row's 64 bytes (rows beyond M: the last row).  W copied into LDS: place q =
+  // tid + 256 c of the stage's W part is group q / 64 = wave + 4 c of the tile's 16-row
+  // groups, and inside it [8-k half h][k-step of 16][output]: lane = 32 h + 16 ks + n; in
+  // the pre-tiled matrix a group's 64 k lie as [h][4 k-steps][16 outputs] pieces of 8.
+  // W into registers: the operand of column block j, k-step ks: column n = n0 + wn WN + 32 j
+  // + lane % 32, half lane / 32.  Groups beyond N are clamped (never stored).
+  const char* a_tile = (const char*)(A + (size_t)m0 * K);
+  uint32_t asrc[A_CHUNKS];
 #pragma unroll
-      for (int it = 0; it < 32 * LPR / 64; ++it) {
-        const int row = it * (64 / LPR) + lane / LPR, q = lane % LPR;
-        const int m = mw + i * 32 + row;
-        const int c = (q / 2) * 32 + (q % 2) * 8;   // first gate column inside the wave's tile
-        const int n = nw + c;
-        if (m < M && n < N) {
-          const float* src = slab + row * SLAB_ROW + c;
-          const float4 g0 = *(const float4*)src, g1 = *(const float4*)(src + 4);
-          const float4 u0 = *(const float4*)(src + 16), u1 = *(const float4*)(src + 20);
-          const u32x4_t v = u32x4_t{
-              pack_bf16x2(swiglu_f(g0.x, u0.x), swiglu_f(g0.y, u0.y)),
-              pack_bf16x2(swiglu_f(g0.z, u0.z), swiglu_f(g0.w, u0.w)),
-              pack_bf16x2(swiglu_f(g1.x, u1.x), swiglu_f(g1.y, u1.y)),
-              pack_bf16x2(swiglu_f(g1.z, u1.z), swiglu_f(g1.w, u1.w))};
-          *(u32x4_t*)((bf16_t*)Cv + (size_t)m * (N / 2) + (n / 32) * 16 + (n % 32)) = v;
-        }
-      }
-    } else if (EPI == EPI_STORE_BF16) {
-      constexpr int LPR = WN / 8;
-#pragma unroll
-      for (int it = 0; it < 32 * LPR / 64; ++it) {
-        const int row = it * (64 / LPR) + lane / LPR, c = (lane % LPR) * 8;
-        const int m = mw + i * 32 + row, n = nw + c;
-        if (m < M && n < N) {
-          const float* src = slab + row * SLAB_ROW + c;
-          const float4 x0 = *(const float4*)src, x1 = *(const float4*)(src + 4);
-          const u32x4_t v = u32x4_t{pack_bf16x2(x0.x, x0.y), pack_bf16x2(x0.z, x0.w),
-                                    pack_bf16x2(x1.x, x1.y), pack_bf16x2(x1.z, x1.w)};
-          *(u32x4_t*)((bf16_t*)Cv + (size_t)m * N + n) = v;
-        }
-      }
-    } else {
-      constexpr int LPR = WN / 4;
-#pragma unroll
-      for (int it = 0; it < 32 * LPR / 64; ++it) {
-        const int row = it * (64 / LPR) + lane / LPR, c = (lane % LPR) * 4;
-        const int m = mw + i * 32 + row, n = nw + c;
-        if (m < M && n < N) {
-          float4 x = *(const float4*)(slab + row * SLAB_ROW + c);
-          float4* dst = (float4*)((float*)Cv + (size_t)m * N + n);
-          if (EPI == EPI_ACC_F32) {
-            const float4 old = *dst;
-            x = float4{old.x + x.x, old.y + x.y, old.z + x.z, old.w + x.w};
-          }
-          *dst = x;
-        }
-      }
-    }
-    __syncthreads();
+  for (int c = 0; c < A_CHUNKS; ++c) {
+    const int row = tid / 4 + 64 * c, piece = (tid % 4) ^ ((tid / 16) & 3);
+    asrc[c] = ((uint32_t)(min(m0 + row, M - 1) - m0) * (uint32_t)K + piece * 8) * 2;
   }
+  const int kt64 = K / 64;
+  const int grp0 = min(n0 / 16, N / 16 - 1);
+  const char* w_tile = (const char*)(W + (size_t)grp0 * kt64 * 1024);
+  uint32_t wsrc[W_CHUNKS];
+#pragma unroll
+  for (int c = 0; c < W_CHUNKS; ++c) {
+    const int grp = min(n0 / 16 + wave + 4 * c, N / 16 - 1) - grp0;
+    wsrc[c] = ((uint32_t)grp * (uint32_t)kt64 * 1024 +
+               ((lane / 32) * 64 + ((lane / 16) % 2) * 16 + lane % 16) * 8) * 2;
+  }
+  // Where k-tile t (of 32) starts in the tokens' rows and in a group's pre-tiled 64 k, as
+  // offsets all lanes share; tiles behind the last one are the last one again.  (t is a
+  // multiple of 4 plus a constant, so which half of the 64 k it is is known when compiling.)
+  const int ktiles = K / 32, klast = ktiles - 1;
+  const uint32_t last_a = (uint32_t)klast * 64, last_w = (uint32_t)(klast / 2) * 2048 + 512;
+  struct TileSrc { const char* a; const char* w; };
+  auto tile_src = [&](int base4, auto OFF) __attribute__((always_inline)) -> TileSrc {
+    constexpr int off = decltype(OFF)::value;
+    const uint32_t oa = min((uint32_t)base4 * 64 + off * 64, last_a);
+    const uint32_t ow = min((uint32_t)base4 * 1024 + (off / 2) * 2048 + (off % 2) * 512, last_w);
+    return TileSrc{a_tile + oa, w_tile + ow};
+  };
+  // copy number q (0 .. CHUNKS - 1) of a k-tile into stage SET
+  auto copy_one = [&](TileSrc src, auto SET, auto Q) __attribute__((always_inline)) {
+    constexpr int q = decltype(Q)::value;
+    u32x4_t* stage = stage_of(SET);
+    if constexpr (q < A_CHUNKS)
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(src.a + asrc[q]),
+          (__attribute__((address_space(3))) void*)(stage + (wave_u * 64 + q * NT)), 16, 0, 0);
+    else
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(src.w + wsrc[q - A_CHUNKS]),
+          (__attribute__((address_space(3))) void*)(stage + (A_PLACES + wave_u * 64 +
+                                                             (q - A_CHUNKS) * NT)), 16, 0, 0);
+  };
+  // MFMA operands of k-step ks (0, 1) of a stage: tokens of row block i at a_at[ks] + 128 i,
+  // outputs of column block j at w_at[ks] + 128 j
+  int a_at[2], w_at[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    a_at[ks] = (wm * WM + lane % 32) * 4 + ((2 * ks + lane / 32) ^ (((lane % 32) >> 2) & 3));
+    w_at[ks] = A_PLACES + (wn * (WN / 16) + (lane % 32) / 16) * 64 + (lane / 32) * 32 + ks * 16 +
+               lane % 16;
+  }
+  constexpr int NR = FM + FN;       // operand reads from LDS per k-step
+  u32x4_t af[2][FM], wf[2][FN];
+  // operand read number c of a k-step: the FM token blocks, then the FN output blocks
+  auto read_one = [&](const u32x4_t* stage, auto KS, auto C) __attribute__((always_inline)) {
+    constexpr int ks = decltype(KS)::value, c = decltype(C)::value;
+    if constexpr (c < FM) af[ks][c] = stage[a_at[ks] + c * 128];
+    else wf[ks][c - FM] = stage[w_at[ks] + (c - FM) * 128];
+  };
+  auto reads_from = [&](auto& self, const u32x4_t* stage, auto KS, auto C0, auto CNT)
+                        __attribute__((always_inline)) -> void {
+    constexpr int c0 = decltype(C0)::value, n = decltype(CNT)::value;
+    if constexpr (n > 0) {
+      read_one(stage, KS, C0);
+      self(self, stage, KS, std::integral_constant<int, c0 + 1>{}, std::integral_constant<int, n - 1>{});
+    }
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
+  // loads q0 .. q0 + n - 1 of a tile
+  auto copies_from = [&](auto& self, TileSrc src, auto SET, auto Q0, auto CNT)
+                         __attribute__((always_inline)) -> void {
+    constexpr int q0 = decltype(Q0)::value, n = decltype(CNT)::value;
+    if constexpr (n > 0) {
+      copy_one(src, SET, Q0);
+      self(self, src, SET, std::integral_constant<int, q0 + 1>{}, std::integral_constant<int, n - 1>{});
+    }
+  };
+  auto copies = [&](TileSrc src, auto SET, auto Q0, auto CNT) __attribute__((always_inline)) {
+    copies_from(copies_from, src, SET, Q0, CNT);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // the loads still in flight behind a tile's own when a step waits for it: two whole tiles
+  constexpr int AHEAD = 2 * CHUNKS;
+  // (and every LDS read done: the barrier frees this step's stage for the next copies, and
+  // the second k-step's operands, read a few MFMAs ago, are only used behind it)
+  constexpr int WAIT = 0x0070 | (AHEAD & 15) | ((AHEAD >> 4) << 14);     // vmcnt(AHEAD) lgkmcnt(0)
+  // A k-step's FM * FN MFMAs on register set / stage CUR; behind them the other k-step's
+  // operand reads (from read_from) and cnt loads of a later tile (from q0 on, into INTO).
+  auto half_step = [&](auto KS, TileSrc src, auto INTO, auto Q0, auto CNT,
+                       const u32x4_t* read_from, auto READ_KS) __attribute__((always_inline)) {
+    constexpr int ks = decltype(KS)::value, q0 = decltype(Q0)::value, cnt = decltype(CNT)::value;
+    constexpr int NM = FM * FN;
+    auto one = [&](auto MI) __attribute__((always_inline)) {
+      constexpr int m = decltype(MI)::value, i = m / FN, j = m % FN;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+          *(const bf16x8_t*)&af[ks][i], *(const bf16x8_t*)&wf[ks][j], acc[i][j], 0, 0, 0);
+      // Load d follows MFMA (d + 1) * NM / cnt - 1: evenly spread.  The reads follow the
+      // first MFMAs that have no load (what does not fit: behind the first as well), so that
+      // they have landed when the k-step ends.
+      constexpr int d_here = copy_after(m, NM, cnt);
+      constexpr int r0 = reads_before(m, NM, cnt, NR), r1 = reads_before(m + 1, NM, cnt, NR);
+      reads_from(reads_from, read_from, READ_KS, std::integral_constant<int, r0>{},
+                 std::integral_constant<int, r1 - r0>{});
+      if constexpr (d_here >= 0)
+        copy_one(src, INTO, std::integral_constant<int, q0 + (d_here >= 0 ? d_here : 0)>{});
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    auto run = [&](auto& self, auto MI) __attribute__((always_inline)) -> void {
+      constexpr int m = decltype(MI)::value;
+      if constexpr (m < NM) {
+        one(MI);
+        self(self, std::integral_constant<int, m + 1>{});
+      }
+    };
+    run(run, std::integral_constant<int, 0>{});
+  };
+  // prologue: tiles 0, 1, 2 and the first part of tile 3; tile 0 has landed, its first operands
+  copies(tile_src(0, I0{}), I0{}, I0{}, std::integral_constant<int, CHUNKS>{});
+  copies(tile_src(0, I1{}), I1{}, I0{}, std::integral_constant<int, CHUNKS>{});
+  copies(tile_src(0, I2{}), I2{}, I0{}, std::integral_constant<int, CHUNKS>{});
+  copies(tile_src(0, I3{}), I3{}, I0{}, std::integral_constant<int, PART1>{});
+  {
+    constexpr int A0 = 2 * CHUNKS + PART1;
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (A0 & 15) | ((A0 >> 4) << 14));
+  }
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  reads_from(reads_from, stage0, I0{}, I0{}, std::integral_constant<int, NR>{});
+  // Step base4 + I on stage I.  First half: the first k-step's MFMAs, the second one's
+  // operands read, the second part of tile + 3's loads issued (into the stage before this
+  // one); then the wait for tile + 1 and the barrier; second half: the second k-step's
+  // MFMAs, the next step's first operands read, the first part of tile + 4's loads issued
+  // into this step's own stage, which every wave has read by now.
+  auto step = [&](int base4, auto IDX) __attribute__((always_inline)) {
+    constexpr int I = decltype(IDX)::value;
+    using NXT = std::integral_constant<int, (I + 1) % 4>;
+    using PRV = std::integral_constant<int, (I + 3) % 4>;
+    half_step(I0{}, tile_src(base4, std::integral_constant<int, I + 3>{}), PRV{},
+              std::integral_constant<int, PART1>{}, std::integral_constant<int, CHUNKS - PART1>{},
+              stage_of(IDX), I1{});
+    __builtin_amdgcn_s_waitcnt(WAIT);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    half_step(I1{}, tile_src(base4, std::integral_constant<int, I + 4>{}), IDX, I0{},
+              std::integral_constant<int, PART1>{}, stage_of(NXT{}), I0{});
+  };
+  int kt = 0;         // (K % 128 == 0: the launch sees to it.  No test before the loop, behind
+  do {                //  which loads could be moved)
+    step(kt, I0{});
+    step(kt, I1{});
+    step(kt, I2{});
+    step(kt, I3{});
+    kt += 4;
+  } while (kt < ktiles);
+  // nothing may still be on its way into LDS when the stages become the epilogue's slabs (a
+  // wave's own stage) or the workgroup ends
+  __builtin_amdgcn_s_waitcnt(0x0f70);       // vmcnt(0)
+  __syncthreads();
+  float* slab = (float*)(wave == 0 ? stage0 : wave == 1 ? stage1 : wave == 2 ? stage2 : stage3);
+  static_assert(32 * (WN + 4) * sizeof(float) <= (A_PLACES + W_PLACES) * 16 || FN == 3, "slab");
+  const int mw = m0 + wm * WM, nw = n0 + wn * WN;
+  if constexpr (FN == 3) {
+    store_through_slab<FM, 2, 64, EPI, 0, FN>(acc, slab, mw, nw, M, N, Cv, lane);
+    store_through_slab<FM, 1, 32, EPI, 2, FN>(acc, slab, mw, nw + 64, M, N, Cv, lane);
+  } else {
+    store_through_slab<FM, FN, WN, EPI>(acc, slab, mw, nw, M, N, Cv, lane);
+  }
+}
+
+template <int BN>
+static int launch_tile256(const void* A, const void* W, void* C, int M, int N, int K, int epi,
+                          hipStream_t stream) {
+  if (N % 16 != 0 || K % 128 != 0) return -3;
+  const int tiles_m = (M + 255) / 256, tiles_n = (N + BN - 1) / BN;
+  const dim3 grid(tiles_m * tiles_n), block(256);
+#define ZF_T256(E)                                                                             \
+  hipLaunchKernelGGL((gemm_bf16_tile256_kernel<BN, E>), grid, block, 0, stream,                \
+                     (const bf16_t*)A, (const bf16_t*)W, C, M, N, K, tiles_m, tiles_n)
+  if (epi == EPI_STORE_BF16) ZF_T256(EPI_STORE_BF16);
+  else if (epi == EPI_STORE_F32) ZF_T256(EPI_STORE_F32);
+  else if (epi == EPI_SWIGLU) ZF_T256(EPI_SWIGLU);
+  else ZF_T256(EPI_ACC_F32);
+#undef ZF_T256
+  return (int)hipGetLastError();
 }
 
 // adds the float32 partials [ksplit, M, N] in split order and applies the epilogue (defined
@@ -734,6 +1029,9 @@ extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, i
       return launch_tile_wdirect<128, 256, 128, 64, TK, false, true>(A, W, C, M, N, K, epi,
                                                                      stream);
     }
+    if (variant == 20) return launch_tile256<256>(A, W, C, M, N, K, epi, stream);
+    if (variant == 21) return launch_tile256<192>(A, W, C, M, N, K, epi, stream);
+    if (variant == 22) return launch_tile256<128>(A, W, C, M, N, K, epi, stream);
     if (variant == 11) {       // as 10, the tokens through registers into LDS
       if (K % (2 * TK) == 0)
         return launch_tile_wdirect<128, 256, 128, 64, TK, true>(A, W, C, M, N, K, epi, stream);

@@ -416,6 +416,57 @@ def _tile_ksplit(M: int, N: int, K: int) -> int:
     return best
 
 
+# Rates per CU (flop/s) of the tiled kernels on pre-tiled weights, from gate/up of the 8B shape
+# at 16384 tokens: the 256-token tiles of 256, 192 and 128 outputs (one workgroup to a CU),
+# and the 128-token tiles two to a CU ("pair") or one ("alone").
+_TILE256_RATE = {20: 5.18e12, 21: 4.52e12, 22: 3.73e12}
+_TILE256_WIDTH = {20: 256, 21: 192, 22: 128}
+_TILE128_RATE = {10: (4.79e12, 3.86e12), 16: (3.9e12, 2.9e12), 6: (3.6e12, 2.7e12)}
+
+
+def _tile256_time(variant: int, M: int, N: int, K: int) -> float:
+    bn = _TILE256_WIDTH[variant]
+    tiles = ((M + 255) // 256) * ((N + bn - 1) // bn)
+    rounds = (tiles + 255) // 256
+    t = rounds * 2.0 * 256 * bn * K / _TILE256_RATE[variant]
+    # on a narrow output the 256-token tiles fall behind this estimate once every CU takes
+    # more than one (o_proj and down at 8192 tokens and more: by 6 to 20 %)
+    return t * (1.08 if (rounds > 1 and N <= 5120) else 1.0) + 4e-6
+
+
+def _tile128_time(M: int, N: int, K: int, variant: int, ksplit: int) -> float:
+    bn = 256 if variant == 10 else 128
+    tiles = ((M + 127) // 128) * ((N + bn - 1) // bn) * ksplit
+    per = 2.0 * 128 * bn * (K / ksplit)
+    pair, alone = _TILE128_RATE[variant if ksplit == 1 else 6]
+    rem = tiles % 512
+    t = (tiles // 512) * 2 * per / pair + (0.0 if rem == 0 else per / alone if rem <= 256 else 2 * per / pair)
+    if ksplit > 1:      # the partials, written and read again, and the second launch
+        t += 4e-6 + M * N * 4.0 * ksplit * 2 / 4e12
+    return t + 4e-6
+
+
+def _tile256_variant(M: int, N: int, K: int, accumulate: bool = False):
+    """The 256-token tile kernel (20: 256 outputs a tile, 21: 192, 22: 128) if it is expected
+    to beat what ``_tile_variant`` and ``_tile_ksplit`` choose by 5 % or more, else None.  One
+    workgroup per CU and tile: what counts is how evenly the tiles fill 256 CUs (2048 tokens
+    into 6144 outputs are 256 tiles of 256 x 192, where 128 x 128 tiles fill 512 places one
+    and a half times: 110 -> 80 us) and, where they fill them many times over, the larger
+    tile's lesser traffic from L2 (gate/up at 8192 tokens: 1341 -> 1259 us).  Times are
+    estimated from rates measured on MI355X; against a sweep of the Qwen3-8B, 14B and 32B
+    widths at 512 to 16384 tokens the choice is within 1 % of the best on the whole and
+    never more than 14 % off.  A residual sum that is split along K keeps its split (the
+    kernel that adds the partials also norms)."""
+    if M <= 256 or K % 128 != 0 or N % 16 != 0:
+        return None
+    ks = _tile_ksplit(M, N, K)
+    if ks > 1 and accumulate:
+        return None
+    now = _tile128_time(M, N, K, _tile_variant(M, N, True, accumulate, K), ks)
+    best = min((20, 21, 22), key=lambda v: _tile256_time(v, M, N, K))
+    return best if _tile256_time(best, M, N, K) < 0.95 * now else None
+
+
 def can_pretile(w: torch.Tensor) -> bool:
     return w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[0] % 64 == 0 \
         and w.shape[1] % 64 == 0
@@ -435,9 +486,10 @@ def pretile_weight(w: torch.Tensor) -> torch.Tensor:
 
 
 def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
-         w_tiled: bool = False) -> None:
+         w_tiled: bool = False, tile_variant: Optional[int] = None) -> None:
     """out = a w^T (w is [N, K]); with ``accumulate`` out += a w^T, in 32-bit.  ``w_tiled``:
-    ``w`` went through ``pretile_weight``.
+    ``w`` went through ``pretile_weight``.  ``tile_variant`` (tests and measurements): this
+    tiled kernel, whatever the number of rows.
 
     bfloat16 operands with K a multiple of 8 go to the MFMA kernels (weight streaming for up
     to 16 rows of ``a``, and up to 64 where the kernel for 17 to 128 rows does not cover the
@@ -458,7 +510,10 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         epi = _EPI_ACC_F32 if accumulate else \
             (_EPI_STORE_BF16 if out.dtype == torch.bfloat16 else _EPI_STORE_F32)
         plan = _small_plan(M, N, K, w_tiled) if M > 16 else None
-        if plan is not None and plan[0] == "mid":
+        if tile_variant is not None:
+            _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, epi, tile_variant,
+                                         1 if w_tiled else 0, _stream()), "gemm (tiled)")
+        elif plan is not None and plan[0] == "mid":
             mid = plan[1]
             ws = _workspace("gemm_splitk", mid * M * N, torch.float32, a.device) if mid > 1 else None
             _check(lib.zf_gemm_bf16_mid(_ptr(a), _ptr(w), _ptr(out), _ptr(ws), M, N, K, epi, mid,
@@ -470,6 +525,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
                                            rg, ks, 1 if w_tiled else 0, _stream()),
                    "gemm (weight streaming)")
         else:
+            big = _tile256_variant(M, N, K, accumulate) if w_tiled else None
+            if big is not None:
+                _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, epi, big, 1,
+                                             _stream()), "gemm (256-token tiles)")
+                return
             ksplit = _tile_ksplit(M, N, K) if w_tiled else 1
             if ksplit > 1:
                 ws = _workspace("gemm_splitk", ksplit * M * N, torch.float32, a.device)
@@ -640,7 +700,8 @@ def can_fuse_swiglu(w: torch.Tensor) -> bool:
     return w.is_cuda and w.dtype == torch.bfloat16 and w.shape[0] % 64 == 0 and w.shape[1] % 8 == 0
 
 
-def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bool = False) -> None:
+def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bool = False,
+                tile_variant: Optional[int] = None) -> None:
     """out[M, I] = silu(a Wg^T) * (a Wu^T) as bfloat16, with ``w`` [2 I, K] from
     ``interleave_gate_up`` (then possibly ``pretile_weight``): the activation is applied to
     the 32-bit sums in the product's epilogue, nothing of width 2 I is written."""
@@ -655,7 +716,11 @@ def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bo
         return
     lib = build.load("gemm")
     plan = _small_plan(M, N, K, w_tiled, swiglu=True) if M > 16 else None
-    if plan is not None and plan[0] == "mid":
+    if tile_variant is not None:
+        _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, _EPI_SWIGLU,
+                                     tile_variant, 1 if w_tiled else 0, _stream()),
+               "gemm_swiglu (tiled)")
+    elif plan is not None and plan[0] == "mid":
         _check(lib.zf_gemm_bf16_mid(_ptr(a), _ptr(w), _ptr(out), _ptr(None), M, N, K, _EPI_SWIGLU,
                                     1, _stream()), "gemm_swiglu (17 to 128 tokens)")
     elif M <= SKINNY_MAX_M:
@@ -664,7 +729,9 @@ def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bo
                                        _EPI_SWIGLU, rg, 1, 1 if w_tiled else 0, _stream()),
                "gemm_swiglu (weight streaming)")
     else:
+        big = _tile256_variant(M, N, K) if w_tiled else None
         _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, _EPI_SWIGLU,
+                                     big if big is not None else
                                      _tile_variant(M, N, w_tiled, False, K), 1 if w_tiled else 0,
                                      _stream()),
                "gemm_swiglu (tiled)")
