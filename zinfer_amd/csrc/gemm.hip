@@ -685,6 +685,8 @@ template <int BN, int EPI>
 __global__ __launch_bounds__(256) void gemm_bf16_tile256_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
     int N, int K, int tiles_m, int tiles_n) {
+  // (the host pass, which only needs the launch stub, does not know the buffer descriptor type)
+#if defined(__HIP_DEVICE_COMPILE__)
   constexpr int BM = 256, NT = 256, WM = 128, WN = BN / 2, FM = WM / 32, FN = WN / 32;
   static_assert(BN == 128 || BN == 192 || BN == 256, "tile width");
   constexpr int A_PLACES = BM * 4, W_PLACES = BN * 4;    // 16-byte pieces of a k-tile of 32
@@ -760,26 +762,34 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256_kernel(
   // multiple of 4 plus a constant, so which half of the 64 k it is is known when compiling.)
   const int ktiles = K / 32, klast = ktiles - 1;
   const uint32_t last_a = (uint32_t)klast * 64, last_w = (uint32_t)(klast / 2) * 2048 + 512;
-  struct TileSrc { const char* a; const char* w; };
+  struct TileSrc { uint32_t a; uint32_t w; };
   auto tile_src = [&](int base4, auto OFF) __attribute__((always_inline)) -> TileSrc {
     constexpr int off = decltype(OFF)::value;
     const uint32_t oa = min((uint32_t)base4 * 64 + off * 64, last_a);
     const uint32_t ow = min((uint32_t)base4 * 1024 + (off / 2) * 2048 + (off % 2) * 512, last_w);
-    return TileSrc{a_tile + oa, w_tile + ow};
+    return TileSrc{oa, ow};
   };
+  // The copies address memory through buffer descriptors (the tile's first token row, the
+  // tile's first group of W; no bound that the offsets could reach): base, an offset per
+  // lane and one all lanes share, so that a copy costs no address arithmetic and issues
+  // faster than one with a 64-bit address per lane.
+  const __amdgpu_buffer_rsrc_t a_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)a_tile, 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t w_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)w_tile, 0, 0x7fffffff, 0x00020000);
   // copy number q (0 .. CHUNKS - 1) of a k-tile into stage SET
   auto copy_one = [&](TileSrc src, auto SET, auto Q) __attribute__((always_inline)) {
     constexpr int q = decltype(Q)::value;
     u32x4_t* stage = stage_of(SET);
     if constexpr (q < A_CHUNKS)
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)(src.a + asrc[q]),
-          (__attribute__((address_space(3))) void*)(stage + (wave_u * 64 + q * NT)), 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          a_rsrc, (__attribute__((address_space(3))) void*)(stage + (wave_u * 64 + q * NT)), 16,
+          asrc[q], src.a, 0, 0);
     else
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)(src.w + wsrc[q - A_CHUNKS]),
-          (__attribute__((address_space(3))) void*)(stage + (A_PLACES + wave_u * 64 +
-                                                             (q - A_CHUNKS) * NT)), 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          w_rsrc, (__attribute__((address_space(3))) void*)(stage + (A_PLACES + wave_u * 64 +
+                                                                    (q - A_CHUNKS) * NT)), 16,
+          wsrc[q - A_CHUNKS], src.w, 0, 0);
   };
   // MFMA operands of k-step ks (0, 1) of a stage: tokens of row block i at a_at[ks] + 128 i,
   // outputs of column block j at w_at[ks] + 128 j
@@ -909,6 +919,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256_kernel(
   } else {
     store_through_slab<FM, FN, WN, EPI>(acc, slab, mw, nw, M, N, Cv, lane);
   }
+#endif
 }
 
 template <int BN>
