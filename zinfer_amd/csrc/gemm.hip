@@ -399,6 +399,8 @@ template <int BM, int BN, int WM, int WN, int EPI, int TKM = TK, bool W2 = false
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdirect_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
     int N, int K, int tiles_m, int tiles_n) {
+  // (the host pass, which only needs the launch stub, does not know the buffer descriptor type)
+#if defined(__HIP_DEVICE_COMPILE__)
   constexpr int NWN = BN / WN, NT = (BM / WM) * NWN * 64;
   constexpr int FM = WM / 32, FN = WN / 32;
   constexpr int LROW = TKM + 8, KCH = TKM / 8;      // LDS row in elements; 16-byte chunks per row
@@ -438,20 +440,26 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
   // W operand of MFMA (j, ks): column n = n0 + wn * WN + 32 j + lane % 32, k = 16 ks +
   // 8 (lane / 32) .. + 8 of the k-tile: piece 64 (lane / 32) + 16 ks + n % 16 of the 16-row
   // group n / 16.  Groups beyond N are clamped (their columns are never stored).
-  const bf16_t* wbase[FN];
+  // (loaded through a buffer descriptor on the tile's first group: a 32-bit offset per lane
+  // and one all lanes share instead of a 64-bit address per lane, which issues faster and
+  // needs no address arithmetic)
+  const int grp0 = min(n0 / 16, N / 16 - 1);
+  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(W + (size_t)grp0 * (K / 64) * 1024), 0, 0x7fffffff, 0x00020000);
+  uint32_t wbase[FN];
 #pragma unroll
   for (int j = 0; j < FN; ++j) {
     const int n = n0 + wn * WN + j * 32 + lane % 32;
-    const int grp = min(n / 16, N / 16 - 1);
-    wbase[j] = W + (size_t)grp * (K / 64) * 1024 + ((lane / 32) * 64 + n % 16) * 8;
+    const int grp = min(n / 16, N / 16 - 1) - grp0;
+    wbase[j] = ((uint32_t)grp * (uint32_t)(K / 64) * 1024 + ((lane / 32) * 64 + n % 16) * 8) * 2;
   }
   u32x4_t wreg[W2 ? 2 : 1][TKM / 16][FN];
   auto gload_w = [&](auto BUF, int kt, int ks) {
     constexpr int B = decltype(BUF)::value;
+    const uint32_t at = ((uint32_t)kt * (TKM / 64) + ks / 4) * 2048 + (ks % 4) * 256;
 #pragma unroll
     for (int j = 0; j < FN; ++j)
-      wreg[B][ks][j] = *(const u32x4_t*)(wbase[j] + ((size_t)kt * (TKM / 64) + ks / 4) * 1024 +
-                                      (ks % 4) * 128);
+      wreg[B][ks][j] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wbase[j], at, 0);
   };
   // gridDim.y workgroups share a tile's k-tiles (split-K for products with few tiles); each
   // then leaves a float32 partial [gridDim.y, M, N] in Cv for skinny_reduce_kernel
@@ -474,14 +482,15 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
       const int p = tid + c * NT, row = p / 8, piece = (p % 8) ^ ((row >> 1) & 7);
       asrc[c] = (uint32_t)(min(m0 + row, M - 1) - m0) * (uint32_t)K + piece * 8;
     }
-    const bf16_t* a_tile = A + (size_t)m0 * K;
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(A + (size_t)m0 * K), 0, 0x7fffffff, 0x00020000);
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);      // the LDS address is a scalar
     auto dma_a = [&](int k0, u32x4_t* stage) {
 #pragma unroll
       for (int c = 0; c < A_CHUNKS; ++c)
-        __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(a_tile + k0 + asrc[c]),
-            (__attribute__((address_space(3))) void*)(stage + (wave_u * 64 + c * NT)), 16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            a_rsrc, (__attribute__((address_space(3))) void*)(stage + (wave_u * 64 + c * NT)), 16,
+            asrc[c] * 2, (uint32_t)k0 * 2, 0, 0);
     };
     // the operand of MFMA row block i, k-step ks: row 32 i + lane % 32, piece 2 ks + lane / 32
     int a_at[TKM / 16];
@@ -641,6 +650,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
   // stages and slabs)
   float* slab = (float*)lds_raw + (size_t)wave * 32 * (WN + 4);
   store_through_slab<FM, FN, WN, EPI>(acc, slab, m0 + wm * WM, n0 + wn * WN, M, N, Cv, lane);
+#endif
 }
 
 // ---------------------------------------------------------------- large M: 256-token tiles, one workgroup to a CU

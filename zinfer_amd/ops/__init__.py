@@ -421,7 +421,7 @@ def _tile_ksplit(M: int, N: int, K: int) -> int:
 # and the 128-token tiles two to a CU ("pair") or one ("alone").
 _TILE256_RATE = {20: 5.18e12, 21: 4.52e12, 22: 3.73e12}
 _TILE256_WIDTH = {20: 256, 21: 192, 22: 128}
-_TILE128_RATE = {10: (4.79e12, 3.86e12), 16: (3.9e12, 2.9e12), 6: (3.6e12, 2.7e12)}
+_TILE128_RATE = {10: (5.13e12, 3.85e12), 16: (3.8e12, 2.9e12), 6: (3.77e12, 2.7e12)}
 
 
 def _tile256_time(variant: int, M: int, N: int, K: int) -> float:
@@ -451,12 +451,12 @@ def _tile256_variant(M: int, N: int, K: int, accumulate: bool = False):
     to beat what ``_tile_variant`` and ``_tile_ksplit`` choose by 5 % or more, else None.  One
     workgroup per CU and tile: what counts is how evenly the tiles fill 256 CUs (2048 tokens
     into 6144 outputs are 256 tiles of 256 x 192, where 128 x 128 tiles fill 512 places one
-    and a half times: 110 -> 80 us) and, where they fill them many times over, the larger
-    tile's lesser traffic from L2 (gate/up at 8192 tokens: 1341 -> 1259 us).  Times are
-    estimated from rates measured on MI355X; against a sweep of the Qwen3-8B, 14B and 32B
-    widths at 512 to 16384 tokens the choice is within 1 % of the best on the whole and
-    never more than 14 % off.  A residual sum that is split along K keeps its split (the
-    kernel that adds the partials also norms)."""
+    and a half times: 101 -> 83 us; 14B down at 3072 tokens: 603 -> 441).  Where both kinds
+    fill the chip many times over they run equally fast (gate/up at 8192 tokens: 1250 us).
+    Times are estimated from rates measured on MI355X; against a sweep of the Qwen3-8B, 14B
+    and 32B widths at 512 to 16384 tokens the choice is within 1 % of the best on the whole.
+    A residual sum that is split along K keeps its split (the kernel that adds the partials
+    also norms)."""
     if M <= 256 or K % 128 != 0 or N % 16 != 0:
         return None
     ks = _tile_ksplit(M, N, K)
