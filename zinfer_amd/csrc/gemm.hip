@@ -508,46 +508,54 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
       for (int ks = 0; ks < TKM / 16; ++ks) gload_w(Buf1{}, min(kt0 + 1, ktiles - 1), ks);
       __builtin_amdgcn_sched_barrier(0);
     }
-    // Before a step: its tokens' copies have landed (they are older than the (TKM / 16) * FN
-    // = 8 W loads issued since, which may stay in flight), then all waves meet: every wave
-    // has also read its last operands out of the other stage.
-    static_assert((TKM / 16) * FN == 8, "the wait counts a step's W loads");
+    // Before a step: its tokens' copies have landed (the last of them is older than the 6 W
+    // loads of the step before that were issued behind it, which may stay in flight), then
+    // all waves meet: every wave has also read its last operands out of the other stage.
+    static_assert(FN == 2 && TKM == 64 && A_CHUNKS == 4, "the wait counts the loads behind the last copy");
     auto meet = [&]() {
-      __builtin_amdgcn_s_waitcnt(0x0f78);     // vmcnt(8)
+      __builtin_amdgcn_s_waitcnt(0x0f76);     // vmcnt(6)
       __builtin_amdgcn_s_barrier();
     };
+    // A k-step's MFMAs run output block by output block, so that a W register is free after
+    // the first FM of them.  What else a wave issues follows single MFMAs: the next k-step's
+    // FM operand reads behind the first FM MFMAs, then (k-steps 0 and 1) two of the next
+    // tile's four copies, then the two W loads that refill this k-step's registers, the
+    // second behind the last MFMA.  (All copies in one place hold the wave, and with it its
+    // MFMAs, while the CU's one path to memory takes them one by one.)
     auto step = [&](int kt, const u32x4_t* cur, u32x4_t* other, auto BUF) {
       constexpr int B = decltype(BUF)::value;
       meet();
       const int wnxt = min(kt + (W2 ? 2 : 1), ktiles - 1);
+      const uint32_t next_k0 = (uint32_t)min(kt + 1, ktiles - 1) * TKM * 2;
       __builtin_amdgcn_sched_barrier(0);
       u32x4_t af[2][FM];
 #pragma unroll
       for (int i = 0; i < FM; ++i) af[0][i] = cur[a_at[0] + i * 256];
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int ks = 0; ks < TKM / 16; ++ks) {
-        if (ks + 1 < TKM / 16) {
+      for (int ks = 0; ks < 4; ++ks) {
+        const uint32_t w_at = ((uint32_t)wnxt * (TKM / 64) + ks / 4) * 2048 + (ks % 4) * 256;
 #pragma unroll
-          for (int i = 0; i < FM; ++i) af[(ks + 1) % 2][i] = cur[a_at[ks + 1] + i * 256];
-        }
+        for (int m = 0; m < 2 * FM; ++m) {
+          const int j = m / FM, i = m % FM;
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              *(const bf16x8_t*)&af[ks % 2][i], *(const bf16x8_t*)&wreg[B][ks][j], acc[i][j],
+              0, 0, 0);
+          if (m < FM && ks < 3) af[(ks + 1) % 2][m] = cur[a_at[ks + 1] + m * 256];
+          // copies 2 ks and 2 ks + 1 of the four: behind the first two MFMAs of the second block
+          if (ks < 2 && (m == FM || (FM > 2 && m == FM + 1))) {
+            const int c0 = 2 * ks + (FM == 2 ? 0 : m - FM), c1 = FM == 2 ? c0 + 2 : c0 + 1;
 #pragma unroll
-        for (int i = 0; i < FM; ++i)
-#pragma unroll
-          for (int j = 0; j < FN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                *(const bf16x8_t*)&af[ks % 2][i], *(const bf16x8_t*)&wreg[B][ks][j], acc[i][j],
-                0, 0, 0);
-        if (ks == 0) {
-          // the next tile's copies, behind the first k-step's MFMAs: issuing a copy holds
-          // the wave for some 60 cycles, which now pass while those MFMAs run (gate/up at
-          // 2048 tokens: 361 -> 347 us); still older than this step's W loads, as the wait
-          // at the next step's start counts on
+            for (int c = c0; c < c1; ++c)
+              __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                  a_rsrc, (__attribute__((address_space(3))) void*)(other + (wave_u * 64 + c * NT)),
+                  16, asrc[c] * 2, next_k0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);      // (older than the W loads that follow)
+          }
+          if (m == 2 * FM - 2) wreg[B][ks][0] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wbase[0], w_at, 0);
+          if (m == 2 * FM - 1) wreg[B][ks][1] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wbase[1], w_at, 0);
           __builtin_amdgcn_sched_barrier(0);
-          dma_a(min(kt + 1, ktiles - 1) * TKM, other);
-          __builtin_amdgcn_sched_barrier(0);
         }
-        gload_w(BUF, wnxt, ks);
-        __builtin_amdgcn_sched_barrier(0);
       }
     };
     if (W2) {       // an even number of k-tiles (the launch sees to it)
