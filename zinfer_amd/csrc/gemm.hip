@@ -576,14 +576,19 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
     __builtin_amdgcn_s_waitcnt(0x0f70);       // vmcnt(0)
   } else {
   u32x4_t areg[A_CHUNKS];
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(A + (size_t)m0 * K), 0, 0x7fffffff, 0x00020000);
+  uint32_t a_from[A_CHUNKS];
+#pragma unroll
+  for (int c = 0; c < A_CHUNKS; ++c) {
+    const int chunk = tid + c * NT;
+    const int row = chunk / KCH, kc = (chunk % KCH) * 8;
+    a_from[c] = ((uint32_t)(min(m0 + row, M - 1) - m0) * (uint32_t)K + kc) * 2;
+  }
   auto gload_a = [&](int k0) {
 #pragma unroll
-    for (int c = 0; c < A_CHUNKS; ++c) {
-      const int chunk = tid + c * NT;
-      const int row = chunk / KCH, kc = (chunk % KCH) * 8;
-      const int m = min(m0 + row, M - 1);
-      areg[c] = *(const u32x4_t*)(A + (size_t)m * K + k0 + kc);
-    }
+    for (int c = 0; c < A_CHUNKS; ++c)
+      areg[c] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_from[c], (uint32_t)k0 * 2, 0);
   };
   auto lstore = [&](int stage) {
     bf16_t* a_s = lds + stage * BM * LROW;
