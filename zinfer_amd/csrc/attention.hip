@@ -731,6 +731,8 @@ __global__ __launch_bounds__(512) void attn_prefill_shared_kernel(
     int q_tiles, int head_blocks, int ps_shift, float* __restrict__ ws_o,
     float* __restrict__ ws_ml, int split_keys, int max_splits,
     const int* __restrict__ tile_map) {
+  // (the host pass, which only needs the launch stub, does not know the buffer descriptor type)
+#if defined(__HIP_DEVICE_COMPILE__)
   constexpr int GROUP_CHUNKS = 2 * HD;          // 16-byte pieces of 16 rows of one kv head
   constexpr int TILE_CHUNKS = 4 * GROUP_CHUNKS;  // of 64 rows: keys first, then values
   __shared__ u32x4_t stage0[2 * TILE_CHUNKS];
@@ -805,12 +807,17 @@ __global__ __launch_bounds__(512) void attn_prefill_shared_kernel(
       const int grp = c0 / GROUP_CHUNKS;
       const uint64_t base = (grp == 0 ? at[0] : grp == 1 ? at[1] : grp == 2 ? at[2] : at[3]) +
                             (uint32_t)(c0 % GROUP_CHUNKS);
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)(k_chunks + base + lane),
-          (__attribute__((address_space(3))) void*)(stage + c0), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)(v_chunks + base + lane),
-          (__attribute__((address_space(3))) void*)(stage + TILE_CHUNKS + c0), 16, 0, 0);
+      // (through buffer descriptors on the 1 KB to copy: the lanes add a 32-bit offset, no
+      // 64-bit address per lane; the pools may be larger than a 32-bit offset reaches)
+      const __amdgpu_buffer_rsrc_t k_rsrc =
+          __builtin_amdgcn_make_buffer_rsrc((void*)(k_chunks + base), 0, 1024, 0x00020000);
+      const __amdgpu_buffer_rsrc_t v_rsrc =
+          __builtin_amdgcn_make_buffer_rsrc((void*)(v_chunks + base), 0, 1024, 0x00020000);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          k_rsrc, (__attribute__((address_space(3))) void*)(stage + c0), 16, lane * 16, 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          v_rsrc, (__attribute__((address_space(3))) void*)(stage + TILE_CHUNKS + c0), 16,
+          lane * 16, 0, 0, 0);
     }
   };
   // the loads into LDS count as vector-memory operations: all of this wave's have landed,
@@ -1103,6 +1110,7 @@ __global__ __launch_bounds__(512) void attn_prefill_shared_kernel(
                           pack_bf16(o[dt][r4 * 4 + 2] * inv, o[dt][r4 * 4 + 3] * inv)};
       *(u32x2_t*)(orow + d) = w;
     }
+#endif
 }
 
 // Combines the key splits of one (token, head) of a prompt portion in split order and writes
