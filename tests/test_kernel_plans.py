@@ -54,6 +54,20 @@ def test_tiled_products(N, K):
     assert ops._tile_variant(512, 24576, True, False, 4096) == 10
 
 
+def test_64_token_tiles_for_a_few_hundred_tokens_on_a_narrow_output():
+    """Measured on MI355X: qkv of the 8B and 14B shapes up to 512 / 544 tokens (at most 512
+    tiles of 64 x 128); not gate/up, not down (long K), not a residual sum, not 128 tokens
+    and fewer (the kernels for those), not 768 and more."""
+    assert ops._tile64_covers(512, 6144, 4096, False) and ops._tile64_covers(160, 6144, 4096, False)
+    assert ops._tile64_covers(544, 7168, 5120, False)
+    assert not ops._tile64_covers(768, 6144, 4096, False)
+    assert not ops._tile64_covers(512, 24576, 4096, False)
+    assert not ops._tile64_covers(512, 4096, 12288, False)
+    assert not ops._tile64_covers(512, 4096, 4096, True)
+    assert not ops._tile64_covers(128, 6144, 4096, False)
+    assert not ops._tile64_covers(512, 6144, 4096 + 64, False)
+
+
 def test_256_token_tiles_are_chosen_where_they_fill_the_chip_evenly():
     """Measured on MI355X (Qwen3-8B widths): 2048 tokens into 6144 outputs are 256 tiles of
     256 x 192 (101 -> 83 us), 3072 into 4096 are 192 of 256 x 256 (110 -> 106; with 12288

@@ -248,6 +248,27 @@ def test_gemm_256_token_tiles(kind, M, N, K, variant):
     _check_tiled(_ops(), kind, M, N, K, variant, seed=41)
 
 
+@pytest.mark.parametrize("M,N,K", [(130, 768, 256), (300, 1088, 384), (520, 1024, 128), (640, 896, 640)])
+def test_gemm_64_token_tiles_above_128_tokens(M, N, K):
+    """A few hundred tokens on a narrow output go through tiles of 64 tokens x 128 outputs,
+    unsplit: edges in M and N, one to five k-tiles of 128, against the plain product and, bit
+    for bit, the 128-token tiles."""
+    ops = _ops()
+    assert ops._tile64_covers(M, N, K, False) and not ops._tile64_covers(M, N, K, True)
+    a = _rand((M, K), torch.bfloat16, 61)
+    w = _rand((N, K), torch.bfloat16, 62, 0.05)
+    wt = ops.pretile_weight(w.to(DEV))
+    for dtype in (torch.bfloat16, torch.float32):
+        want = torch.empty((M, N), dtype=dtype)
+        ref.gemm(a, w, want, False)
+        got = torch.full((M, N), float("nan"), dtype=dtype, device=DEV)
+        ops.gemm(a.to(DEV), wt, got, w_tiled=True)
+        assert rel_err(got, want) <= (2e-5 if dtype == torch.float32 else tol(torch.bfloat16))
+        other = torch.empty_like(got)
+        ops.gemm(a.to(DEV), wt, other, w_tiled=True, tile_variant=6)
+        assert torch.equal(got, other)
+
+
 def test_gemm_256_token_tiles_are_chosen_and_agree():
     """Where the cost model picks the 256-token tiles the product goes through them, with the
     same bits as through the 128-token tiles: the sums are added in the same order."""
