@@ -6,6 +6,7 @@ error.  Kernels take every size a configuration allows or refuse it with a clear
 from __future__ import annotations
 
 import ctypes
+import functools
 from typing import Optional
 
 import torch
@@ -424,6 +425,7 @@ _TILE256_WIDTH = {20: 256, 21: 192, 22: 128}
 _TILE128_RATE = {10: (5.13e12, 3.85e12), 16: (3.8e12, 2.9e12), 6: (3.77e12, 2.7e12)}
 
 
+@functools.lru_cache(maxsize=None)
 def _tile64_covers(M: int, N: int, K: int, accumulate: bool) -> bool:
     """A few hundred tokens on a narrow output, no residual sum: tiles of 64 tokens x 128
     outputs, unsplit, where there are at most 512 of them (two to a CU): the 128-token tiles
@@ -438,6 +440,7 @@ def _tile64_covers(M: int, N: int, K: int, accumulate: bool) -> bool:
 
 
 def _tile256_time(variant: int, M: int, N: int, K: int) -> float:
+    """Estimated seconds of the 256-token tile kernel: rounds of up to 256 tiles, one to a CU."""
     bn = _TILE256_WIDTH[variant]
     tiles = ((M + 255) // 256) * ((N + bn - 1) // bn)
     rounds = (tiles + 255) // 256
@@ -448,6 +451,8 @@ def _tile256_time(variant: int, M: int, N: int, K: int) -> float:
 
 
 def _tile128_time(M: int, N: int, K: int, variant: int, ksplit: int) -> float:
+    """Estimated seconds of the 128-token tile kernels: rounds of up to 512 tiles, two to a CU
+    (a last round of up to 256 tiles runs one to a CU, each faster than two)."""
     bn = 256 if variant == 10 else 128
     tiles = ((M + 127) // 128) * ((N + bn - 1) // bn) * ksplit
     per = 2.0 * 128 * bn * (K / ksplit)
@@ -459,6 +464,7 @@ def _tile128_time(M: int, N: int, K: int, variant: int, ksplit: int) -> float:
     return t + 4e-6
 
 
+@functools.lru_cache(maxsize=None)
 def _tile256_variant(M: int, N: int, K: int, accumulate: bool = False):
     """The 256-token tile kernel (20: 256 outputs a tile, 21: 192, 22: 128) if it is expected
     to beat what ``_tile_variant`` and ``_tile_ksplit`` choose by 5 % or more, else None.  One
