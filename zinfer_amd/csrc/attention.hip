@@ -326,83 +326,79 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   }
 }
 
-// Combines the splits of one (sequence, head) in split order and writes bfloat16.  One wave:
-// every lane first takes one split's (max, sum) of a chunk of 64 splits, so that the weights
-// exp2(m - max) are formed side by side; then the lanes, each owning hd / 64 output elements,
-// add the partial outputs with eight loads in flight.
-__global__ __launch_bounds__(64) void attn_decode_merge_kernel(
+// Combines the splits of one (sequence, head) and writes bfloat16.  One workgroup of 4 waves.
+// A split's partial output is hd floats in a row: hd / 4 lanes take it as one 16-byte load
+// each, so a wave load covers 256 / hd splits and the workgroup's 4 waves 1024 / hd splits
+// ("slots"); slot j takes the splits first + j, first + j + slots, ... with 8 loads in
+// flight: 128 splits of a 32 K context are two trips to memory (one wave of 8 loads over
+// all of them took sixteen: 26 us, more than the attention kernel before it).  The first
+// loads do not wait for the weights: they are asked for together with the (max, sum) pairs.
+// Sums are added slot by slot and the slots in a fixed order, which the context length
+// alone decides.
+template <int HD>
+__global__ __launch_bounds__(256) void attn_decode_merge_kernel(
     const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
     const int* __restrict__ q_start, const int* __restrict__ ctx_len, bf16_t* __restrict__ out,
-    int window, int nH, int hd, int max_splits) {
-  const int s = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    int window, int nH, int max_splits) {
+  constexpr int LPS = HD / 4;            // lanes per split
+  constexpr int SLOTS = 256 / LPS;       // splits the workgroup takes at a time
+  constexpr int U = 8;                   // loads in flight per lane
+  __shared__ float red[4];
+  __shared__ __attribute__((aligned(16))) float part[SLOTS][HD];
+  __shared__ float part_den[SLOTS];
+  const int s = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
   if (q_start[s + 1] - q_start[s] != 1) return;
   const int ctx = ctx_len[s], pos = ctx - 1;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int first = lo / DEC_SPLIT, last = pos / DEC_SPLIT;
   const size_t base = ((size_t)s * nH + head) * max_splits;
-  // the first eight splits' partial outputs are asked for together with the (max, sum)
-  // pairs, before the weights are known: one trip to memory less for contexts of up to
-  // 2048 keys, where this kernel is nothing but such trips
-  float v0[8][8];
+  const int slot = tid / LPS, piece = tid % LPS;
+  const f32x4_t* src = (const f32x4_t*)(ws_o + base * HD) + piece;     // + split * LPS
+  // the first U splits of this slot, before the weights are known
+  f32x4_t v[U];
+  float2 ml[U];
 #pragma unroll
-  for (int u = 0; u < 8; ++u) {
-    const float* src = ws_o + (base + min(first + u, last)) * hd;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int d = lane + 64 * i;
-      v0[u][i] = (d < hd) ? src[d] : 0.f;
-    }
+  for (int u = 0; u < U; ++u) {
+    const int sp = min(first + slot + u * SLOTS, last);
+    v[u] = src[(size_t)sp * LPS];
+    ml[u] = *(const float2*)(ws_ml + (base + sp) * 2);
   }
   float mx = -INFINITY;
-  for (int sp = first + lane; sp <= last; sp += 64) mx = fmaxf(mx, ws_ml[(base + sp) * 2]);
+  for (int sp = first + tid; sp <= last; sp += 256) mx = fmaxf(mx, ws_ml[(base + sp) * 2]);
   mx = wave_max(mx);
-  float acc[8];
+  if (tid % 64 == 0) red[tid / 64] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float den = 0.f;
+  for (int sp0 = first + slot; sp0 <= last; sp0 += U * SLOTS) {
+    if (sp0 != first + slot) {
 #pragma unroll
-  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-  float denom = 0.f;
-  for (int chunk = first; chunk <= last; chunk += 64) {
-    const int mine = chunk + lane;
-    float w_l = 0.f, l_l = 0.f;
-    if (mine <= last) {
-      const float2 ml = *(const float2*)(ws_ml + (base + mine) * 2);
-      w_l = exp2f(ml.x - mx);
-      l_l = ml.y;
+      for (int u = 0; u < U; ++u) {
+        const int sp = min(sp0 + u * SLOTS, last);
+        v[u] = src[(size_t)sp * LPS];
+        ml[u] = *(const float2*)(ws_ml + (base + sp) * 2);
+      }
     }
-    denom += wave_sum(w_l * l_l);
-    const int n = min(64, last - chunk + 1);
-    for (int i0 = 0; i0 < n; i0 += 8) {
-      float v[8][8];
-      if (chunk == first && i0 == 0) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
+    for (int u = 0; u < U; ++u) {
+      const float w = (sp0 + u * SLOTS <= last) ? exp2f(ml[u].x - mx) : 0.f;
+      den = fmaf(w, ml[u].y, den);
 #pragma unroll
-          for (int i = 0; i < 8; ++i) v[u][i] = v0[u][i];
-      } else {
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int sp = min(chunk + i0 + u, last);
-          const float* src = ws_o + (base + sp) * hd;
-#pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            const int d = lane + 64 * i;
-            v[u][i] = (d < hd) ? src[d] : 0.f;
-          }
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const float w = (i0 + u < n) ? __shfl(w_l, i0 + u, 64) : 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] = fmaf(w, v[u][i], acc[i]);
-      }
+      for (int e = 0; e < 4; ++e) acc[e] = fmaf(w, v[u][e], acc[e]);
     }
   }
-  const float inv = 1.0f / denom;
-  bf16_t* orow = out + ((size_t)q_start[s] * nH + head) * hd;
+  *(f32x4_t*)&part[slot][4 * piece] = acc;
+  if (piece == 0) part_den[slot] = den;
+  __syncthreads();
+  if (tid < HD) {
+    float o = 0.f, denom = 0.f;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int d = lane + 64 * i;
-    if (d < hd) orow[d] = float_to_bf16(acc[i] * inv);
+    for (int j = 0; j < SLOTS; ++j) {
+      o += part[j][tid];
+      denom += part_den[j];
+    }
+    out[((size_t)q_start[s] * nH + head) * HD + tid] = float_to_bf16(o / denom);
   }
 }
 
@@ -429,8 +425,14 @@ extern "C" int zf_attn_decode_bf16(const void* q, const void* k_pool, const void
   else if (hd == 256) ZF_DEC(256);
   else return -2;
 #undef ZF_DEC
-  hipLaunchKernelGGL(attn_decode_merge_kernel, dim3(n_seqs, nH), dim3(64), 0, stream, ws_o, ws_ml,
-                     q_start, ctx_len, (bf16_t*)out, window, nH, hd, max_splits);
+#define ZF_DEC_MERGE(HD)                                                                        \
+  hipLaunchKernelGGL(attn_decode_merge_kernel<HD>, dim3(n_seqs, nH), dim3(256), 0, stream, ws_o, \
+                     ws_ml, q_start, ctx_len, (bf16_t*)out, window, nH, max_splits)
+  if (hd == 32) ZF_DEC_MERGE(32);
+  else if (hd == 64) ZF_DEC_MERGE(64);
+  else if (hd == 128) ZF_DEC_MERGE(128);
+  else ZF_DEC_MERGE(256);
+#undef ZF_DEC_MERGE
   ZF_CHECK_LAUNCH();
 }
 
