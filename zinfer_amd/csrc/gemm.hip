@@ -1458,9 +1458,30 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_skinny_kernel(
   }
 }
 
-template <int EPI>
+// VEC: four outputs a thread with 16-byte loads (M * N a multiple of 4, so that every
+// partial starts on a 16-byte boundary); else one output a thread.
+template <int EPI, bool VEC>
 __global__ void skinny_reduce_kernel(const float* __restrict__ ws, void* __restrict__ Cv,
                                      size_t mn, int ksplit) {
+  if (VEC) {
+    const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i >= mn) return;
+    float4 s = float4{0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < ksplit; ++k) {
+      const float4 p = *(const float4*)(ws + (size_t)k * mn + i);
+      s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
+    }
+    if (EPI == EPI_STORE_BF16) {
+      *(u32x2_t*)((bf16_t*)Cv + i) = u32x2_t{pack_bf16x2(s.x, s.y), pack_bf16x2(s.z, s.w)};
+    } else if (EPI == EPI_STORE_F32) {
+      *(float4*)((float*)Cv + i) = s;
+    } else {
+      float4* dst = (float4*)((float*)Cv + i);
+      const float4 old = *dst;
+      *dst = float4{old.x + s.x, old.y + s.y, old.z + s.z, old.w + s.w};
+    }
+    return;
+  }
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= mn) return;
   float s = 0.f;
@@ -1476,18 +1497,22 @@ __global__ void skinny_reduce_kernel(const float* __restrict__ ws, void* __restr
 static int launch_reduce(const void* ws, void* C, int M, int N, int ksplit, int epi,
                          hipStream_t stream) {
   const size_t mn = (size_t)M * N;
-  const unsigned blocks = (unsigned)((mn + 255) / 256);
-  if (epi == EPI_STORE_BF16)
-    hipLaunchKernelGGL(skinny_reduce_kernel<EPI_STORE_BF16>, dim3(blocks), dim3(256), 0, stream,
-                       (const float*)ws, C, mn, ksplit);
-  else if (epi == EPI_STORE_F32)
-    hipLaunchKernelGGL(skinny_reduce_kernel<EPI_STORE_F32>, dim3(blocks), dim3(256), 0, stream,
-                       (const float*)ws, C, mn, ksplit);
-  else if (epi == EPI_ACC_F32)
-    hipLaunchKernelGGL(skinny_reduce_kernel<EPI_ACC_F32>, dim3(blocks), dim3(256), 0, stream,
-                       (const float*)ws, C, mn, ksplit);
-  else
-    return -3;
+  const bool vec = mn % 4 == 0;
+  const unsigned blocks = (unsigned)(((vec ? mn / 4 : mn) + 255) / 256);
+#define ZF_REDUCE(E)                                                                           \
+  do {                                                                                         \
+    if (vec)                                                                                   \
+      hipLaunchKernelGGL((skinny_reduce_kernel<E, true>), dim3(blocks), dim3(256), 0, stream,  \
+                         (const float*)ws, C, mn, ksplit);                                     \
+    else                                                                                       \
+      hipLaunchKernelGGL((skinny_reduce_kernel<E, false>), dim3(blocks), dim3(256), 0, stream, \
+                         (const float*)ws, C, mn, ksplit);                                     \
+  } while (0)
+  if (epi == EPI_STORE_BF16) ZF_REDUCE(EPI_STORE_BF16);
+  else if (epi == EPI_STORE_F32) ZF_REDUCE(EPI_STORE_F32);
+  else if (epi == EPI_ACC_F32) ZF_REDUCE(EPI_ACC_F32);
+  else return -3;
+#undef ZF_REDUCE
   return (int)hipGetLastError();
 }
 
