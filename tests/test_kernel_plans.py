@@ -55,17 +55,23 @@ def test_tiled_products(N, K):
 
 
 def test_64_token_tiles_for_a_few_hundred_tokens_on_a_narrow_output():
-    """Measured on MI355X: qkv of the 8B and 14B shapes up to 512 / 544 tokens (at most 512
-    tiles of 64 x 128); not gate/up, not down (long K), not a residual sum, not 128 tokens
-    and fewer (the kernels for those), not 768 and more."""
-    assert ops._tile64_covers(512, 6144, 4096, False) and ops._tile64_covers(160, 6144, 4096, False)
-    assert ops._tile64_covers(544, 7168, 5120, False)
+    """Measured on MI355X with weights from HBM: where one round of the chip holds the 64 x 128
+    tiles (qkv of the 8B shape up to 320 tokens), or where the 128-token tiles would need a
+    second round (qkv of the 14B shape at 513 to 576 tokens); not against a single round of
+    128-token tiles, not gate/up, not down (long K), not a residual sum, not 128 tokens and
+    fewer (the kernels for those), not 768 and more."""
+    assert ops._tile64_covers(272, 6144, 4096, False) and ops._tile64_covers(160, 6144, 4096, False)
+    assert ops._tile64_covers(384, 6144, 4096, False)          # 288 tiles
+    assert ops._tile64_covers(544, 7168, 5120, False)          # 128-token tiles: 280
+    assert ops._tile64_covers(384, 5120, 8192, False)
+    assert not ops._tile64_covers(512, 6144, 4096, False)      # 384 against 192 in one round
+    assert not ops._tile64_covers(384, 7168, 5120, False)
     assert not ops._tile64_covers(768, 6144, 4096, False)
     assert not ops._tile64_covers(512, 24576, 4096, False)
     assert not ops._tile64_covers(512, 4096, 12288, False)
     assert not ops._tile64_covers(512, 4096, 4096, True)
     assert not ops._tile64_covers(128, 6144, 4096, False)
-    assert not ops._tile64_covers(512, 6144, 4096 + 64, False)
+    assert not ops._tile64_covers(272, 6144, 4096 + 64, False)
 
 
 def test_256_token_tiles_are_chosen_where_they_fill_the_chip_evenly():

@@ -142,6 +142,39 @@ __device__ __forceinline__ size_t tiled_offset(int n, int k, int K) {
          ((kk / 16) * 16 + n % 16) * 8 + kk % 8;
 }
 
+// XCD-aware tile order.  Consecutive workgroups go to different XCDs (8 of them, each with its
+// own L2), so workgroup b takes place (b % 8) * per_xcd + b / 8 of the tile order: one XCD
+// then walks neighbouring tiles.  The order runs through groups of at most GROUP tile rows,
+// down the rows of a group first, so that the tiles an XCD walks share W tiles in its L2.  The
+// rows are dealt evenly over the groups (9 rows in groups of 8: 5 + 4, not 8 + 1): a group of
+// one row would send an XCD through every W tile on its own.
+template <int GROUP>
+__device__ __forceinline__ void tile_of_workgroup(int b, int tiles_m, int tiles_n, int& tm,
+                                                  int& tn) {
+  const int nblocks = tiles_m * tiles_n;
+  {
+    const int base = nblocks / 8, rem = nblocks % 8;
+    const int xcd = b % 8, idx = b / 8;
+    b = xcd * base + min(xcd, rem) + idx;   // XCD x owns base (+1 if x < rem) tiles in a row
+  }
+  const int ngroups = (tiles_m + GROUP - 1) / GROUP;
+  const int rows = tiles_m / ngroups, longer = tiles_m % ngroups;   // the first groups: rows + 1
+  const int in_longer = (rows + 1) * tiles_n;
+  int first_m, gsize, at;
+  if (b < longer * in_longer) {
+    gsize = rows + 1;
+    first_m = (b / in_longer) * gsize;
+    at = b % in_longer;
+  } else {
+    const int bb = b - longer * in_longer, in_group = rows * tiles_n;
+    gsize = rows;
+    first_m = longer * (rows + 1) + (bb / in_group) * rows;
+    at = bb % in_group;
+  }
+  tm = first_m + at % gsize;
+  tn = at / gsize;
+}
+
 template <int BM, int BN, int WM, int WN, int EPI, bool WT>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
@@ -157,23 +190,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_ker
   // stage s: A at s*(BM+BN)*LDS_ROW, W after it
   constexpr int STAGE = (BM + BN) * LDS_ROW;
 
-  // XCD-aware tile order: consecutive workgroups go to different XCDs (8 of them, each with
-  // its own L2), so workgroup b works on tile (b % 8) * per_xcd + b / 8: one XCD then walks
-  // neighbouring tiles, grouped 8 tiles of M deep so that they share W tiles in its L2.
-  const int nblocks = tiles_m * tiles_n;
-  int b = blockIdx.x;
-  {
-    const int base = nblocks / 8, rem = nblocks % 8;
-    const int xcd = b % 8, idx = b / 8;
-    b = xcd * base + min(xcd, rem) + idx;   // XCD x owns base (+1 if x < rem) tiles in a row
-  }
-  const int GROUP = 8;
-  const int in_group = GROUP * tiles_n;
-  const int g = b / in_group;
-  const int first_m = g * GROUP;
-  const int gsize = min(tiles_m - first_m, GROUP);
-  const int tm = first_m + (b % in_group) % gsize;
-  const int tn = (b % in_group) / gsize;
+  int tm, tn;
+  tile_of_workgroup<(BM >= 128 ? 8 : 1024 / BM)>(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
   const int tid = threadIdx.x;
@@ -409,20 +427,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   bf16_t* lds = (bf16_t*)lds_raw;       // two stages of BM rows of LROW elements
 
-  const int nblocks = tiles_m * tiles_n;
-  int b = blockIdx.x;
-  {
-    const int base = nblocks / 8, rem = nblocks % 8;
-    const int xcd = b % 8, idx = b / 8;
-    b = xcd * base + min(xcd, rem) + idx;
-  }
-  const int GROUP = 8;
-  const int in_group = GROUP * tiles_n;
-  const int g = b / in_group;
-  const int first_m = g * GROUP;
-  const int gsize = min(tiles_m - first_m, GROUP);
-  const int tm = first_m + (b % in_group) % gsize;
-  const int tn = (b % in_group) / gsize;
+  int tm, tn;
+  tile_of_workgroup<(BM >= 128 ? 8 : 1024 / BM)>(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
   const int tid = threadIdx.x;
@@ -728,19 +734,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256_kernel(
     else return stage3;
   };
 
-  const int nblocks = tiles_m * tiles_n;
-  int b = blockIdx.x;
-  {
-    const int base = nblocks / 8, rem = nblocks % 8;
-    const int xcd = b % 8, idx = b / 8;
-    b = xcd * base + min(xcd, rem) + idx;
-  }
-  const int GROUP = 8;
-  const int in_group = GROUP * tiles_n;
-  const int first_m = (b / in_group) * GROUP;
-  const int gsize = min(tiles_m - first_m, GROUP);
-  const int tm = first_m + (b % in_group) % gsize;
-  const int tn = (b % in_group) / gsize;
+  int tm, tn;
+  tile_of_workgroup<(BM >= 128 ? 8 : 1024 / BM)>(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;

@@ -378,8 +378,9 @@ def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = Fals
                   K: int = 0) -> int:
     """Which tiled kernel: with pre-tiled weights the kernels that take W straight from
     memory (10: 128 x 256 tiles, two workgroups to a CU, when they fill the chip; else 128 x
-    128 tiles, 16: with the waves side by side and k-tiles of 128 for a long K, 6: with
-    2 x 2 waves); otherwise the kernels that stage both operands through LDS (4: 256 x 256
+    128 tiles, 16: with the waves side by side and k-tiles of 128, for a long K or when one
+    round of the chip holds the tiles (weights from HBM, 512 tokens: qkv of the 8B shape 43 ->
+    38 us), 6: with 2 x 2 waves); otherwise the kernels that stage both operands through LDS (4: 256 x 256
     when they still fill the chip, else 0: 128 x 128).  Measured on MI355X at the Qwen3-8B and
     Qwen3-14B sizes."""
     if w_tiled:
@@ -390,7 +391,8 @@ def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = Fals
         # tiles along the tokens (512 tokens into 24576 outputs) the large tiles still win
         if tiles >= 160 and not (256 < tiles < 512 and tiles_m > 4):
             return 10
-        return 16 if K >= 8192 and K % 128 == 0 else 6
+        one_round = tiles_m * ((N + 127) // 128) <= 256
+        return 16 if K > 0 and K % 128 == 0 and (K >= 8192 or one_round) else 6
     tiles = ((M + 255) // 256) * ((N + 255) // 256)
     return 4 if tiles >= 160 else 0
 
@@ -428,15 +430,20 @@ _TILE128_RATE = {10: (5.13e12, 3.85e12), 16: (3.8e12, 2.9e12), 6: (3.77e12, 2.7e
 @functools.lru_cache(maxsize=None)
 def _tile64_covers(M: int, N: int, K: int, accumulate: bool) -> bool:
     """A few hundred tokens on a narrow output, no residual sum: tiles of 64 tokens x 128
-    outputs, unsplit, where there are at most 512 of them (two to a CU): the 128-token tiles
-    would be too few to fill the chip and need a split along K with its second kernel.
-    Measured on MI355X: qkv of the 8B shape at 160 to 512 tokens 1.12 to 1.5 times faster
-    (512 tokens: 41 -> 35 us), of the 14B shape at 544 tokens 76 -> 65 us; at 640 tokens
-    and more, on gate/up and on down (K long) the larger tiles win.  A residual sum keeps
-    its split, whose second kernel is also the norm."""
+    outputs, unsplit.  A CU finishes one such tile in about two thirds of the time of a
+    128 x 128 tile, and a second round doubles that, so they are taken where one round holds
+    them (up to 288: the last few share CUs), or where the 128-token tiles would need a
+    second round themselves while these stay within two.  Measured on MI355X with weights
+    that come from HBM (more copies in turn than the last-level cache holds): qkv of the
+    8B shape at 272 tokens 36 -> 26 us, o_proj-like 5120 x 8192 at 384 tokens 72 -> 51 us,
+    qkv of the 14B shape at 528 to 576 tokens 70 -> 58 us; with 300 to 512 tiles against one
+    round of the larger ones they lose (14B qkv at 384 tokens 47 -> 57 us).  A residual sum
+    keeps its split along K, whose second kernel is also the norm."""
     if accumulate or not (128 < M <= 640 and K % 128 == 0 and N % 16 == 0 and K <= 8192):
         return False
-    return ((M + 63) // 64) * ((N + 127) // 128) <= 512
+    cols = (N + 127) // 128
+    tiles64, tiles128 = ((M + 63) // 64) * cols, ((M + 127) // 128) * cols
+    return tiles64 <= 288 or (tiles128 > 256 and tiles64 <= 512)
 
 
 def _tile256_time(variant: int, M: int, N: int, K: int) -> float:
