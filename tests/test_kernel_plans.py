@@ -51,6 +51,9 @@ def test_tiled_products(N, K):
                             (256, 4096, 4096): 4, (256, 6144, 4096): 2, (1024, 5120, 17408): 3,
                             (1024, 4096, 12288): 1}.items():
         assert ops._tile_ksplit(M, n, k) == want, (M, n, k)
+    # a stored product whose tiles need a second round anyway stays whole; a residual sum splits
+    assert ops._tile_ksplit(768, 6144, 4096, False) == 1 and ops._tile_ksplit(768, 6144, 4096) > 1
+    assert ops._tile_ksplit(384, 6144, 4096, False) == 3
     assert ops._tile_variant(512, 24576, True, False, 4096) == 10
 
 

@@ -397,17 +397,20 @@ def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = Fals
     return 4 if tiles >= 160 else 0
 
 
-def _tile_ksplit(M: int, N: int, K: int) -> int:
+def _tile_ksplit(M: int, N: int, K: int, accumulate: bool = True) -> int:
     """Workgroups per 128 x 128 tile along K: products of a few hundred tokens on a narrow
     output have too few tiles for 256 CUs, or a number that fills them unevenly (160 tiles:
     96 CUs idle; 320: a second round for a quarter of them).  Two workgroups fit a CU, so the
     split is chosen to fill 256 or a multiple of 512 places as evenly as it can, each
     workgroup keeping at least 8 k-tiles of 64.  Every split costs partials of M * N floats,
     written and read again (against the product's own time that is about 400 / K a split),
-    and the first one a second launch.  Measured on MI355X at the Qwen3-8B and Qwen3-14B
-    sizes, 256 to 1024 tokens."""
+    and the first one a second launch.  A product that is stored, not added to the residual,
+    stays whole once its tiles need a second round anyway (257 and more: 768 tokens of the 8B
+    shape's qkv 66 -> 59 us); the residual sum gains from the split up to 383 tiles, since the
+    kernel that adds the partials is the norm's as well.  Measured on MI355X at the Qwen3-8B,
+    14B and 32B sizes, 256 to 1024 tokens, the weights from HBM."""
     tiles = ((M + 127) // 128) * ((N + 127) // 128)
-    if tiles >= 384:
+    if tiles >= 384 or (tiles > 256 and not accumulate):
         return 1
     best, best_cost = 1, None
     for ks in range(1, min(8, K // 64 // 8) + 1):
@@ -485,7 +488,7 @@ def _tile256_variant(M: int, N: int, K: int, accumulate: bool = False):
     also norms)."""
     if M <= 256 or K % 128 != 0 or N % 16 != 0:
         return None
-    ks = _tile_ksplit(M, N, K)
+    ks = _tile_ksplit(M, N, K, accumulate)
     if ks > 1 and accumulate:
         return None
     now = _tile128_time(M, N, K, _tile_variant(M, N, True, accumulate, K), ks)
@@ -559,7 +562,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
                 _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, epi, big, 1,
                                              _stream()), "gemm (256-token tiles)")
                 return
-            ksplit = _tile_ksplit(M, N, K) if w_tiled else 1
+            ksplit = _tile_ksplit(M, N, K, accumulate) if w_tiled else 1
             if ksplit > 1:
                 ws = _workspace("gemm_splitk", ksplit * M * N, torch.float32, a.device)
                 _check(lib.zf_gemm_bf16_tile_splitk(_ptr(a), _ptr(w), _ptr(out), _ptr(ws), M, N,
