@@ -623,6 +623,78 @@ def test_qk_norm_rope_kv_write(dtype, nH, nKV, hd, page_size, use_norm, use_rope
     assert rel_err(got_inplace, want_inplace) <= tol(dtype)
 
 
+@pytest.mark.parametrize("nH,nKV,hd,page_size,window,use_norm,use_rope", [
+    (32, 8, 128, 16, 0, True, True), (8, 2, 32, 16, 0, True, True), (6, 6, 64, 32, 0, True, False),
+    (16, 1, 64, 16, 37, False, True), (9, 3, 256, 16, 0, True, True), (10, 2, 128, 48, 300, True, True),
+    (36, 4, 32, 16, 0, False, False), (32, 2, 128, 16, 0, True, True), (9, 1, 256, 32, 0, True, True)])
+def test_decode_attention_fused_equals_the_two_kernels(nH, nKV, hd, page_size, window, use_norm,
+                                                       use_rope):
+    """The decode attention that norms and rotates q and k and stores the token's key and
+    value itself, against qk_norm_rope_kv_write followed by paged_attention: the same bits in
+    the output and in both pools.  Contexts end at, before and after a split's (256) and a
+    page's edge; the slot of the token's own position holds NaN beforehand, as a page that is
+    used again may; 16 query heads to a kv head and head size 256 take two rounds of the
+    workgroup's lanes; the rotation's positions are not the cache's (they come from their own
+    array)."""
+    from zinfer_amd.parts.position import rotary_tables
+    dtype, ops = torch.bfloat16, _ops()
+    ctx_lens = [1, 15, 16, 17, 255, 256, 257, 600, 1025, 512, 513]
+    n = len(ctx_lens)
+    s = _paged_setup(dtype, nH, nKV, hd, page_size, ctx_lens, [1] * n, seed=21)
+    num_pages = s["k_pool"].shape[0]
+    k_pool = s["k_pool"].view(num_pages, nKV, page_size, hd).clone()
+    v_pool = s["v_pool"].view(num_pages, nKV, hd, page_size).clone()
+    slots = []
+    for i, c in enumerate(ctx_lens):
+        pg, r = int(s["block_table"][i, (c - 1) // page_size]), (c - 1) % page_size
+        k_pool[pg, :, r] = float("nan")
+        v_pool[pg, :, :, r] = float("nan")
+        slots.append(pg * page_size + r)
+    k_tiled = ref.tile_k_pool(k_pool.view(num_pages, -1).to(DEV), nKV, page_size, hd)
+    v_tiled = ref.tile_v_pool(v_pool.view(num_pages, -1).to(DEV), nKV, page_size, hd)
+    qkv = _rand((n, (nH + 2 * nKV) * hd), dtype, 22).to(DEV)
+    qg = (1 + 0.1 * _rand((hd,), torch.float32, 23)).to(DEV) if use_norm else None
+    kg = (1 + 0.1 * _rand((hd,), torch.float32, 24)).to(DEV) if use_norm else None
+    cos, sin = (t.to(DEV) for t in rotary_tables(hd, 10000.0, 1100)) if use_rope else (None, None)
+    positions = torch.tensor([c - 1 + 5 for c in ctx_lens], dtype=torch.int32, device=DEV)
+    slot_mapping = torch.tensor(slots, dtype=torch.int32, device=DEV)
+    d = {k: s[k].to(DEV) for k in ("block_table", "q_start", "ctx_len", "seq_index")}
+    scale, eps = 1.0 / math.sqrt(hd), 1e-6
+
+    kp_a, vp_a = k_tiled.clone(), v_tiled.clone()
+    q = torch.empty((n, nH * hd), dtype=dtype, device=DEV)
+    ops.qk_norm_rope_kv_write(qkv.clone(), qg, kg, eps, cos, sin, positions, slot_mapping, kp_a,
+                              vp_a, q, nH, nKV, hd, page_size)
+    want = torch.full((n, nH * hd), float("nan"), dtype=dtype, device=DEV)
+    ops.paged_attention(q, kp_a, vp_a, d["block_table"], d["q_start"], d["ctx_len"],
+                        d["seq_index"], want, scale, window, nH, nKV, hd, page_size, 1,
+                        max(ctx_lens), n_single=n)
+
+    kp_b, vp_b = k_tiled.clone(), v_tiled.clone()
+    before = qkv.clone()
+    got = torch.full((n, nH * hd), float("nan"), dtype=dtype, device=DEV)
+    ops.decode_attention_fused(qkv, qg, kg, eps, cos, sin, positions, slot_mapping, kp_b, vp_b,
+                               d["block_table"], d["q_start"], d["ctx_len"], got, scale, window,
+                               nH, nKV, hd, page_size, max(ctx_lens))
+    torch.cuda.synchronize()
+    assert not torch.isnan(want.float()).any() and not torch.isnan(got.float()).any()
+    bits = lambda t: t.view(torch.int16)
+    assert torch.equal(bits(got), bits(want))
+    assert torch.equal(bits(kp_b), bits(kp_a)) and torch.equal(bits(vp_b), bits(vp_a))
+    assert torch.equal(bits(qkv), bits(before)), "the product's rows are only read"
+    # and what both write is what the plain implementation writes
+    kc, vc = k_pool.view(num_pages, -1).clone(), v_pool.view(num_pages, -1).clone()
+    ref.qk_norm_rope_kv_write(before.cpu(), None if qg is None else qg.cpu(),
+                              None if kg is None else kg.cpu(), eps,
+                              None if cos is None else cos.cpu(), None if sin is None else sin.cpu(),
+                              positions.cpu(), slot_mapping.cpu(), kc, vc,
+                              torch.empty((n, nH * hd), dtype=dtype), nH, nKV, hd, page_size)
+    kc = ref.tile_k_pool(kc, nKV, page_size, hd)
+    live = ~torch.isnan(kc.float())
+    assert torch.equal(live, ~torch.isnan(kp_b.float().cpu()))
+    assert rel_err(torch.where(live, kp_b.cpu().float(), 0.0), torch.where(live, kc.float(), 0.0)) <= tol(dtype)
+
+
 def test_rope_reference_vector():
     """[1, 2, 3, 4] at position 1, theta 1e4: h0 = cos1 - 3 sin1, h1 = 2 cos(.01) - 4 sin(.01),
     h2 = 3 cos1 + sin1, h3 = 4 cos(.01) + 2 sin(.01) (src/kernel/attention/rope.zig:174-190)."""

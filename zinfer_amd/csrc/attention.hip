@@ -188,6 +188,141 @@ __device__ __forceinline__ size_t tiled_v_offset(int grp, int r16, int d, int hd
 #define DEC_SPLIT 256
 #define DEC_WAVE_KEYS 64
 
+// The scores of a wave's 64 keys against the G query columns, their soft-max terms and the
+// product with the values.  kf, vf and qf are the MFMA operands as the loads leave them; m, l
+// and o the wave's maximum, sum and un-normalised output.  One order of operations for every
+// kernel that decodes.
+//
+// PATCH: key kb + pn (0 <= pn < 64; pn < 0: none) is not what kf and vf hold for it but the
+// row k_new / v_new in LDS (the token's own key and value, which the cache did not hold yet
+// when the loads were asked for).  Its scores come from MFMAs of their own over a tile that
+// holds the row in its place, and land in the lanes and registers that hold that key's scores
+// anyway: an MFMA's output element depends on its own row and column alone, so the scores, and
+// with them everything after, are the bits that operands read from the cache would give.
+template <int HD, bool PATCH = false>
+__device__ __forceinline__ void decode_attend(const u32x4_t (&kf)[4][HD / 32],
+                                              const u32x2_t (&vf)[4][HD / 16],
+                                              const bf16x8_t (&qf)[HD / 32], int kb, int k_begin,
+                                              int k_end, int qd, float scale_log2e, float& m,
+                                              float& l, f32x4_t (&o)[HD / 16], int pn = -1,
+                                              const bf16_t* k_new = nullptr,
+                                              const bf16_t* v_new = nullptr) {
+  f32x4_t st[4];
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    st[h] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int stp = 0; stp < HD / 32; ++stp)
+      st[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&kf[h][stp], qf[stp],
+                                                      st[h], 0, 0, 0);
+  }
+  const int hn = pn / 16, jn = pn % 16, lane16 = threadIdx.x % 16;
+  if constexpr (PATCH) {
+    if (pn >= 0) {
+      // lane (j, qd) holds of a 16-key tile the row j, elements 32 stp + 8 qd .. + 7
+      f32x4_t sn = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int stp = 0; stp < HD / 32; ++stp) {
+        u32x4_t kx = *(const u32x4_t*)(k_new + stp * 32 + 8 * qd);
+        if (lane16 != jn) kx = u32x4_t{0, 0, 0, 0};
+        sn = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&kx, qf[stp], sn, 0, 0, 0);
+      }
+      // its scores: element jn % 4 of the lanes with qd = jn / 4, in group hn
+#pragma unroll
+      for (int h = 0; h < 4; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (h == hn && r == jn % 4 && qd == jn / 4) st[h][r] = sn[r];
+    }
+  }
+  // st[h][r]: key kb + 16 h + 4 qd + r, query column j
+  float sc[16];
+#pragma unroll
+  for (int h = 0; h < 4; ++h)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int key = kb + 16 * h + 4 * qd + r;
+      const float v = (key >= k_begin && key < k_end) ? st[h][r] * scale_log2e : -INFINITY;
+      sc[h * 4 + r] = v;
+      m = fmaxf(m, v);
+    }
+  m = fmaxf(m, __shfl_xor(m, 16, 64));
+  m = fmaxf(m, __shfl_xor(m, 32, 64));
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    sc[e] = exp2_raw(sc[e] - m);
+    l += sc[e];
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+#pragma unroll
+  for (int hh = 0; hh < 2; ++hh) {     // two MFMAs of 32 keys: groups 2 hh and 2 hh + 1
+    u32x4_t pk = u32x4_t{pack_bf16(sc[8 * hh + 0], sc[8 * hh + 1]),
+                         pack_bf16(sc[8 * hh + 2], sc[8 * hh + 3]),
+                         pack_bf16(sc[8 * hh + 4], sc[8 * hh + 5]),
+                         pack_bf16(sc[8 * hh + 6], sc[8 * hh + 7])};
+    const bf16x8_t pf = *(bf16x8_t*)&pk;
+    const int b0 = kb + 32 * hh + 4 * qd, b1 = b0 + 16;
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt) {
+      // stale or poisoned rows outside [k_begin, k_end) are zeroed: 0 * NaN would spoil the sum
+      u32x2_t v0 = keep_range4(vf[2 * hh][dt], k_begin - b0, k_end - b0);
+      u32x2_t v1 = keep_range4(vf[2 * hh + 1][dt], k_begin - b1, k_end - b1);
+      if constexpr (PATCH) {
+        // the lanes with qd = jn / 4 hold the values of keys 4 qd .. 4 qd + 3 at head
+        // element 16 dt + j, 16 bits each
+        if (pn >= 0 && hn / 2 == hh && qd == jn / 4) {
+          const uint32_t vn = v_new[16 * dt + lane16];
+          u32x2_t& v = hn % 2 ? v1 : v0;
+          const int w = (jn % 4) / 2, sh = 16 * (jn % 2);
+          v[w] = (v[w] & ~(0xffffu << sh)) | (vn << sh);
+        }
+      }
+      u32x4_t vv = u32x4_t{v0[0], v0[1], v1[0], v1[1]};
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8_t*)&vv, pf, o[dt], 0, 0, 0);
+    }
+  }
+}
+
+// The four waves' partials combined through LDS in wave order; the workgroup writes one
+// un-normalised partial (max, sum, O[G, hd]) per query head for its split.
+template <int HD>
+__device__ __forceinline__ void decode_write_partial(float (&s_o)[4][16][HD], float (&s_m)[4][16],
+                                                     float (&s_l)[4][16], int wave, int j, int qd,
+                                                     float m, float l,
+                                                     const f32x4_t (&o)[HD / 16], int G,
+                                                     size_t first_slot, int max_splits,
+                                                     float* __restrict__ ws_o,
+                                                     float* __restrict__ ws_ml) {
+  // this wave's partial for query column j: rows d = 16 dt + 4 qd + r
+#pragma unroll
+  for (int dt = 0; dt < HD / 16; ++dt) *(f32x4_t*)&s_o[wave][j][dt * 16 + 4 * qd] = o[dt];
+  if (qd == 0) {
+    s_m[wave][j] = m;
+    s_l[wave][j] = l;
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < G * HD; idx += 256) {
+    const int col = idx / HD, d = idx % HD;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) mx = fmaxf(mx, s_m[w][col]);
+    float acc = 0.f, den = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = exp2f(s_m[w][col] - mx);     // a wave without keys has max -inf: weight 0
+      acc += f * s_o[w][col][d];
+      den += f * s_l[w][col];
+    }
+    const size_t slot = first_slot + (size_t)col * max_splits;   // of (sequence, head, split)
+    ws_o[slot * HD + d] = acc;
+    if (d == 0) {
+      ws_ml[slot * 2] = mx;
+      ws_ml[slot * 2 + 1] = den;
+    }
+  }
+}
+
 template <int HD>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool,
@@ -250,80 +385,205 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 #pragma unroll
       for (int dt = 0; dt < HD / 16; ++dt)
         vf[h][dt] = __builtin_nontemporal_load((const u32x2_t*)(vg[h] + dt * 256));
-    f32x4_t st[4];
+    decode_attend<HD>(kf, vf, qf, kb, k_begin, k_end, qd, scale_log2e, m, l, o);
+  }
+  decode_write_partial<HD>(s_o, s_m, s_l, wave, j, qd, m, l, o, G,
+                           ((size_t)s * nH + kvh * G) * max_splits + sp, max_splits, ws_o, ws_ml);
+}
+
+// What the fused decode kernel needs to do the work of the kernel before it as well (the
+// per-head norm of q and k, their rotation, the new key and value into the cache).
+struct DecodeFused {
+  const float* q_gain;      // null: no norm
+  const float* k_gain;
+  float eps;
+  const float* cos_t;       // [positions, hd / 2], null: no rotation
+  const float* sin_t;
+  const int* positions;     // [n_seqs]
+  const int* slot_mapping;  // [n_seqs]: page * page_size + row of the token's own key and value
+};
+
+// A decode step's attention from the q/k/v product's rows [n_seqs, (nH + 2 nKV) * hd], which
+// it only reads: every sequence has one token, token s is sequence s's.  Grid, splits and the
+// arithmetic of the attention are attn_decode_kernel's.  Before it, a workgroup norms and
+// rotates its kv head's G query rows itself (into LDS, rounded to bfloat16 as the separate
+// kernel leaves them in memory; every split's workgroup repeats these few hundred flops), and
+// the workgroup whose split holds the token's own position does the same for the new key and
+// stores it and the new value in the cache.
+//
+// Order.  A lane's loads return in the order it asked for them, so whatever the norm and
+// rotation need from memory is asked for first and the keys right behind it: the arithmetic
+// then runs while the keys' loads are in flight and waits for none of them.  The values are
+// asked for behind the arithmetic (with both in flight beside what the norm holds, three
+// waves would no longer fit a SIMD's registers); they are needed last.  The wave that holds
+// the token's own position cannot read it from the cache (the stores come later than its
+// loads of the keys): it takes the new key and value from LDS into the operand registers of
+// the lanes that hold that position, once its loads have landed.
+//
+// The page of a 16-key group is the same for a whole wave, so the look-ups and the blocks'
+// addresses are scalar and a load's address is one of them plus a lane's offset: the loads
+// hold no address registers, which leaves room for what the norm holds meanwhile.
+template <int HD>
+__global__ __launch_bounds__(256, HD <= 128 ? 3 : 1) void attn_decode_fused_kernel(
+    const bf16_t* __restrict__ qkv, bf16_t* __restrict__ k_pool, bf16_t* __restrict__ v_pool,
+    const int* __restrict__ block_table, const int* __restrict__ ctx_len,
+    float* __restrict__ ws_o, float* __restrict__ ws_ml, float scale_log2e, int window, int nH,
+    int nKV, int ps, int max_pages, int max_splits, DecodeFused fu) {
+  __shared__ __attribute__((aligned(16))) float s_o[4][16][HD];
+  __shared__ float s_m[4][16], s_l[4][16];
+  // rows 0 .. G - 1: the query heads; row 16: the new key; row 17: the new value
+  __shared__ __attribute__((aligned(16))) bf16_t s_q[18][HD + 8];
+  const int kvh = blockIdx.x, sp = blockIdx.y, s = blockIdx.z;
+  const int ctx = ctx_len[s], pos = ctx - 1;
+  const int slot = fu.slot_mapping[s];
+  const int rope_pos = fu.cos_t ? fu.positions[s] : 0;
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  if (max(lo, sp * DEC_SPLIT) >= min(ctx, (sp + 1) * DEC_SPLIT)) return;   // whole workgroup
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+  const int lane = threadIdx.x % 64, j = lane % 16, qd = lane / 16;
+  const int kb = sp * DEC_SPLIT + wave * DEC_WAVE_KEYS;
+  const int k_begin = max(lo, kb), k_end = min(ctx, kb + DEC_WAVE_KEYS);
+  const bool has_keys = k_begin < k_end;
+  const int G = nH / nKV;
+  const int* table = block_table + (size_t)s * max_pages;
+
+  // LPH lanes to a head, 8 elements each; the workgroup takes HEADS heads at a time.  Item
+  // i < G is query head kvh * G + i, item G the new key (where the split holds the token's
+  // own position).
+  constexpr int LPH = HD / 8, HEADS = 256 / LPH;
+  constexpr int V_EARLY = HD == 128 ? 2 : 4;      // groups whose values are asked for with the keys
+  const int li = threadIdx.x % LPH;
+  const bool own = pos / DEC_SPLIT == sp;
+  const int items = own ? G + 1 : G;
+  const int row_width = (nH + 2 * nKV) * HD;
+  const bf16_t* row = qkv + (size_t)s * row_width;
+  struct Item {
+    u32x2_t raw0, raw1;
+    HeadCoef cf;
+    bool active, is_q;
+  };
+  auto fetch = [&](int item) {
+    Item it;
+    it.active = item < items;
+    it.is_q = item < G;
+    const int head = !it.active ? 0 : it.is_q ? kvh * G + item : nH + kvh;
+    it.raw0 = *(const u32x2_t*)(row + (size_t)head * HD + 4 * li);
+    it.raw1 = *(const u32x2_t*)(row + (size_t)head * HD + HD / 2 + 4 * li);
+    load_head_coef(it.cf, li, HD, it.is_q ? fu.q_gain : fu.k_gain, fu.cos_t, fu.sin_t, rope_pos);
+    return it;
+  };
+  const Item first = fetch(threadIdx.x / LPH);
+  u32x4_t v_new = u32x4_t{0, 0, 0, 0};
+  if (own && threadIdx.x < HD / 8)      // the new value: 8 elements a lane
+    v_new = *(const u32x4_t*)(row + (size_t)(nH + nKV + kvh) * HD + 8 * threadIdx.x);
+
+  u32x4_t kf[4][HD / 32];
+  u32x2_t vf[4][HD / 16];
+  size_t blk[4] = {0, 0, 0, 0};
+  if (has_keys) {
+    // the four 16-key groups of this wave; a group outside [k_begin, k_end) may have no page
+    // at all: it reads the group of a key that certainly exists and is masked
+    // (the four look-ups are scalar loads: asked for together, waited for once)
+    int key_of[4], page_of[4];
 #pragma unroll
     for (int h = 0; h < 4; ++h) {
-      st[h] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int stp = 0; stp < HD / 32; ++stp)
-        st[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&kf[h][stp], qf[stp],
-                                                        st[h], 0, 0, 0);
+      const int base = kb + 16 * h;
+      const bool any = base < k_end && base + 16 > k_begin;
+      key_of[h] = any ? base : (k_begin / 16) * 16;
     }
-    // st[h][r]: key kb + 16 h + 4 qd + r, query column j
-    float sc[16];
+#pragma unroll
+    for (int h = 0; h < 4; ++h) page_of[h] = table[key_of[h] / ps];
+#pragma unroll
+    for (int h = 0; h < 4; ++h)
+      blk[h] = (((size_t)page_of[h] * nKV + kvh) * ps + (key_of[h] % ps)) * HD;
 #pragma unroll
     for (int h = 0; h < 4; ++h)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int key = kb + 16 * h + 4 * qd + r;
-        const float v = (key >= k_begin && key < k_end) ? st[h][r] * scale_log2e : -INFINITY;
-        sc[h * 4 + r] = v;
-        m = fmaxf(m, v);
-      }
-    m = fmaxf(m, __shfl_xor(m, 16, 64));
-    m = fmaxf(m, __shfl_xor(m, 32, 64));
+      for (int stp = 0; stp < HD / 32; ++stp)
+        kf[h][stp] = __builtin_nontemporal_load(
+            (const u32x4_t*)(k_pool + blk[h] + stp * 512) + lane);
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      sc[e] = exp2_raw(sc[e] - m);
-      l += sc[e];
+    for (int h = 0; h < V_EARLY; ++h)
+#pragma unroll
+      for (int dt = 0; dt < HD / 16; ++dt)
+        vf[h][dt] = __builtin_nontemporal_load(
+            (const u32x2_t*)(v_pool + blk[h] + dt * 256) + lane);
+  }
+  // (nothing below may move above the loads, and none of them below it)
+  __builtin_amdgcn_sched_barrier(0);
+
+  const int page = slot / ps, r = slot % ps;
+  // the block of the token's 16-row group in the pools
+  const size_t grp_at = (((size_t)page * nKV + kvh) * ps + (r / 16) * 16) * HD;
+  auto finish = [&](int item, const Item& it) {
+    float x0[4], x1[4];
+    const u32x2_t a = it.active ? it.raw0 : u32x2_t{0, 0}, b = it.active ? it.raw1 : u32x2_t{0, 0};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      x0[e] = bf16_to_float((bf16_t)(a[e / 2] >> (16 * (e % 2))));
+      x1[e] = bf16_to_float((bf16_t)(b[e / 2] >> (16 * (e % 2))));
     }
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
+    head_norm_rotate<LPH>(x0, x1, HD, it.active, fu.eps, it.cf);
+    if (!it.active) return;
+    const u32x2_t y0 = u32x2_t{pack_bf16x2(x0[0], x0[1]), pack_bf16x2(x0[2], x0[3])};
+    const u32x2_t y1 = u32x2_t{pack_bf16x2(x1[0], x1[1]), pack_bf16x2(x1[2], x1[3])};
+    bf16_t* dst = s_q[it.is_q ? item : 16];
+    *(u32x2_t*)(dst + 4 * li) = y0;
+    *(u32x2_t*)(dst + HD / 2 + 4 * li) = y1;
+    if (!it.is_q) {    // element d of row r at [d / 32][16 ((d % 32) / 8) + r % 16][d % 8]
+      bf16_t* grp = k_pool + grp_at;
+      const int d0 = 4 * li, d1 = HD / 2 + 4 * li;
+      *(u32x2_t*)(grp + (d0 / 32) * 512 + (((d0 % 32) / 8) * 16 + r % 16) * 8 + d0 % 8) = y0;
+      *(u32x2_t*)(grp + (d1 / 32) * 512 + (((d1 % 32) / 8) * 16 + r % 16) * 8 + d1 % 8) = y1;
+    }
+  };
+  finish(threadIdx.x / LPH, first);
+  // (more than HEADS items: 16 query heads to a kv head, or head size 256 with more than 7;
+  // these loads queue behind the keys and values)
+  for (int it0 = HEADS; it0 < items; it0 += HEADS) {
+    const Item it = fetch(it0 + threadIdx.x / LPH);
+    finish(it0 + threadIdx.x / LPH, it);
+  }
+  if (own && threadIdx.x < HD / 8) {
+    *(u32x4_t*)(s_q[17] + 8 * threadIdx.x) = v_new;
+    // element d of row r at [d / 16][16 (r % 16 / 4) + d % 16][r % 4]
+    bf16_t* grp = v_pool + grp_at + ((r % 16) / 4) * 64 + r % 4;
 #pragma unroll
-    for (int hh = 0; hh < 2; ++hh) {     // two MFMAs of 32 keys: groups 2 hh and 2 hh + 1
-      u32x4_t pk = u32x4_t{pack_bf16(sc[8 * hh + 0], sc[8 * hh + 1]),
-                           pack_bf16(sc[8 * hh + 2], sc[8 * hh + 3]),
-                           pack_bf16(sc[8 * hh + 4], sc[8 * hh + 5]),
-                           pack_bf16(sc[8 * hh + 6], sc[8 * hh + 7])};
-      const bf16x8_t pf = *(bf16x8_t*)&pk;
-      const int b0 = kb + 32 * hh + 4 * qd, b1 = b0 + 16;
-#pragma unroll
-      for (int dt = 0; dt < HD / 16; ++dt) {
-        // stale or poisoned rows outside [k_begin, k_end) are zeroed: 0 * NaN would spoil the sum
-        const u32x2_t v0 = keep_range4(vf[2 * hh][dt], k_begin - b0, k_end - b0);
-        const u32x2_t v1 = keep_range4(vf[2 * hh + 1][dt], k_begin - b1, k_end - b1);
-        u32x4_t vv = u32x4_t{v0[0], v0[1], v1[0], v1[1]};
-        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8_t*)&vv, pf, o[dt], 0, 0, 0);
-      }
+    for (int i = 0; i < 8; ++i) {
+      const int d = 8 * threadIdx.x + i;
+      grp[(d / 16) * 256 + (d % 16) * 4] = (bf16_t)(v_new[i / 2] >> (16 * (i % 2)));
     }
   }
-  // this wave's partial for query column j: rows d = 16 dt + 4 qd + r
+  __builtin_amdgcn_sched_barrier(0);
+  if (has_keys) {
 #pragma unroll
-  for (int dt = 0; dt < HD / 16; ++dt) *(f32x4_t*)&s_o[wave][j][dt * 16 + 4 * qd] = o[dt];
-  if (qd == 0) {
-    s_m[wave][j] = m;
-    s_l[wave][j] = l;
+    for (int h = V_EARLY; h < 4; ++h)
+#pragma unroll
+      for (int dt = 0; dt < HD / 16; ++dt)
+        vf[h][dt] = __builtin_nontemporal_load(
+            (const u32x2_t*)(v_pool + blk[h] + dt * 256) + lane);
   }
+  __builtin_amdgcn_sched_barrier(0);
   __syncthreads();
-  for (int idx = threadIdx.x; idx < G * HD; idx += 256) {
-    const int col = idx / HD, d = idx % HD;
-    float mx = -INFINITY;
+
+  float m = -INFINITY, l = 0.f;
+  f32x4_t o[HD / 16];
 #pragma unroll
-    for (int w = 0; w < 4; ++w) mx = fmaxf(mx, s_m[w][col]);
-    float acc = 0.f, den = 0.f;
+  for (int dt = 0; dt < HD / 16; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  if (has_keys) {
+    bf16x8_t qf[HD / 32];
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const float f = exp2f(s_m[w][col] - mx);     // a wave without keys has max -inf: weight 0
-      acc += f * s_o[w][col][d];
-      den += f * s_l[w][col];
+    for (int st = 0; st < HD / 32; ++st) {
+      u32x4_t v = *(const u32x4_t*)(s_q[min(j, G - 1)] + st * 32 + 8 * qd);
+      if (j >= G) v = u32x4_t{0, 0, 0, 0};
+      qf[st] = *(bf16x8_t*)&v;
     }
-    const size_t slot = ((size_t)s * nH + kvh * G + col) * max_splits + sp;
-    ws_o[slot * HD + d] = acc;
-    if (d == 0) {
-      ws_ml[slot * 2] = mx;
-      ws_ml[slot * 2 + 1] = den;
-    }
+    const int pn = (pos >= kb && pos < kb + DEC_WAVE_KEYS) ? pos - kb : -1;
+    decode_attend<HD, true>(kf, vf, qf, kb, k_begin, k_end, qd, scale_log2e, m, l, o, pn,
+                            s_q[16], s_q[17]);
   }
+  decode_write_partial<HD>(s_o, s_m, s_l, wave, j, qd, m, l, o, G,
+                           ((size_t)s * nH + kvh * G) * max_splits + sp, max_splits, ws_o, ws_ml);
 }
 
 // Combines the splits of one (sequence, head) and writes bfloat16.  One workgroup of 4 waves.
@@ -404,6 +664,20 @@ __global__ __launch_bounds__(256) void attn_decode_merge_kernel(
 
 // ws_o: n_seqs * nH * max_splits * hd floats, ws_ml: n_seqs * nH * max_splits * 2 floats,
 // max_splits >= ceil(longest context / 256); the pools are tiled.
+static int launch_decode_merge(const float* ws_o, const float* ws_ml, const int* q_start,
+                               const int* ctx_len, void* out, int window, int n_seqs, int nH,
+                               int hd, int max_splits, hipStream_t stream) {
+#define ZF_DEC_MERGE(HD)                                                                        \
+  hipLaunchKernelGGL(attn_decode_merge_kernel<HD>, dim3(n_seqs, nH), dim3(256), 0, stream, ws_o, \
+                     ws_ml, q_start, ctx_len, (bf16_t*)out, window, nH, max_splits)
+  if (hd == 32) ZF_DEC_MERGE(32);
+  else if (hd == 64) ZF_DEC_MERGE(64);
+  else if (hd == 128) ZF_DEC_MERGE(128);
+  else ZF_DEC_MERGE(256);
+#undef ZF_DEC_MERGE
+  ZF_CHECK_LAUNCH();
+}
+
 extern "C" int zf_attn_decode_bf16(const void* q, const void* k_pool, const void* v_pool,
                                    const int* block_table, const int* q_start,
                                    const int* ctx_len, void* out, float* ws_o, float* ws_ml,
@@ -425,15 +699,47 @@ extern "C" int zf_attn_decode_bf16(const void* q, const void* k_pool, const void
   else if (hd == 256) ZF_DEC(256);
   else return -2;
 #undef ZF_DEC
-#define ZF_DEC_MERGE(HD)                                                                        \
-  hipLaunchKernelGGL(attn_decode_merge_kernel<HD>, dim3(n_seqs, nH), dim3(256), 0, stream, ws_o, \
-                     ws_ml, q_start, ctx_len, (bf16_t*)out, window, nH, max_splits)
-  if (hd == 32) ZF_DEC_MERGE(32);
-  else if (hd == 64) ZF_DEC_MERGE(64);
-  else if (hd == 128) ZF_DEC_MERGE(128);
-  else ZF_DEC_MERGE(256);
-#undef ZF_DEC_MERGE
-  ZF_CHECK_LAUNCH();
+  return launch_decode_merge(ws_o, ws_ml, q_start, ctx_len, out, window, n_seqs, nH, hd,
+                             max_splits, stream);
+}
+
+// A decode step's attention from the q/k/v product's own rows: every sequence has one token,
+// token s is sequence s's (q_start is 0, 1, ..., n_seqs).  qkv [n_seqs, (nH + 2 nKV) * hd]
+// bfloat16 is read, not changed; the per-head RMSNorm of q and k (gains float32 [hd], or
+// both null), their rotation (tables float32 [*, hd / 2] read at positions[s], or both null)
+// and the write of the token's key and value into the tiled pools at slot_mapping[s] (the
+// slot of position ctx_len[s] - 1) happen inside the attention kernel, with the arithmetic
+// of zf_qk_norm_rope_kv_write.
+extern "C" int zf_attn_decode_fused_bf16(const void* qkv, const float* q_gain,
+                                         const float* k_gain, float eps, const float* cos_t,
+                                         const float* sin_t, const int* positions,
+                                         const int* slot_mapping, void* k_pool, void* v_pool,
+                                         const int* block_table, const int* q_start,
+                                         const int* ctx_len, void* out, float* ws_o,
+                                         float* ws_ml, float scale, int window, int n_seqs,
+                                         int nH, int nKV, int hd, int page_size, int max_pages,
+                                         int max_splits, hipStream_t stream) {
+  if (n_seqs <= 0) return 0;
+  if (page_size % 16 != 0 || nKV <= 0 || nH % nKV != 0 || nH / nKV > 16) return -2;
+  if ((q_gain == nullptr) != (k_gain == nullptr) || (cos_t == nullptr) != (sin_t == nullptr) ||
+      slot_mapping == nullptr || (cos_t != nullptr && positions == nullptr))
+    return -2;
+  const DecodeFused fu{q_gain, k_gain, eps, cos_t, sin_t, positions, slot_mapping};
+  const float scale_log2e = scale * 1.4426950408889634f;
+  dim3 grid(nKV, max_splits, n_seqs);
+#define ZF_DEC(HD)                                                                              \
+  hipLaunchKernelGGL(attn_decode_fused_kernel<HD>, grid, dim3(256), 0, stream,                  \
+                     (const bf16_t*)qkv, (bf16_t*)k_pool, (bf16_t*)v_pool, block_table,         \
+                     ctx_len, ws_o, ws_ml, scale_log2e, window, nH, nKV, page_size, max_pages,  \
+                     max_splits, fu)
+  if (hd == 32) ZF_DEC(32);
+  else if (hd == 64) ZF_DEC(64);
+  else if (hd == 128) ZF_DEC(128);
+  else if (hd == 256) ZF_DEC(256);
+  else return -2;
+#undef ZF_DEC
+  return launch_decode_merge(ws_o, ws_ml, q_start, ctx_len, out, window, n_seqs, nH, hd,
+                             max_splits, stream);
 }
 
 // ---------------------------------------------------------------- prefill: portions of prompts

@@ -274,34 +274,11 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_vec_kernel(
   }
   // query and key heads (lanes of value heads have left: the shuffles below stay inside
   // groups of LPH lanes, which are all of one head)
-  const float* gain = is_q ? q_gain : k_gain;
-  if (gain) {
-    float ss = 0.f;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) ss += x0[e] * x0[e] + x1[e] * x1[e];
-#pragma unroll
-    for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
-    const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
-    if (active) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        x0[e] = x0[e] * inv * gain[4 * li + e];
-        x1[e] = x1[e] * inv * gain[half + 4 * li + e];
-      }
-    }
-  }
+  HeadCoef cf;
+  load_head_coef(cf, active ? li : 0, hd, is_q ? q_gain : k_gain, cos_t, sin_t,
+                 cos_t ? positions[t] : 0);
+  head_norm_rotate<LPH>(x0, x1, hd, active, eps, cf);
   if (!active) return;
-  if (cos_t) {
-    const int pos = positions[t];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float c = cos_t[(size_t)pos * half + 4 * li + e], sn = sin_t[(size_t)pos * half + 4 * li + e];
-      const float r0 = x0[e] * c - x1[e] * sn;
-      const float r1 = x1[e] * c + x0[e] * sn;
-      x0[e] = r0;
-      x1[e] = r1;
-    }
-  }
   T* dst0;
   T* dst1;
   if (is_q) {

@@ -39,6 +39,63 @@ template <> __device__ __forceinline__ void store_from_float<bf16_t>(bf16_t* p, 
   *p = float_to_bf16(v);
 }
 
+// RMSNorm over a head and rotation of its pairs (i, i + hd / 2) for the 8 elements a lane
+// holds: x0 = elements 4 li .. 4 li + 3 of the head, x1 = those hd / 2 further on; LPH lanes
+// side by side hold the head (src/kernel/norm/basic.zig:5-22 and src/kernel/rope/basic.zig:5-30
+// of the reference: x / sqrt(mean(x^2) + eps) * gain, then (x0 c - x1 s, x1 c + x0 s) with the
+// angle of (position, pair)).  Every lane of the LPH calls it (the sum goes over all of them);
+// a lane that is not `active` holds zeros and keeps them.  The gains and the angles' cosines
+// and sines of the lane's elements are loaded apart (a null table: none), so that a kernel
+// can ask for them early.  One function for the kernel that writes the cache and for the
+// decode attention that does the same work itself, so that both round alike.
+struct HeadCoef {
+  float g0[4], g1[4], c[4], sn[4];
+  bool has_gain, has_rotation;
+};
+__device__ __forceinline__ void load_head_coef(HeadCoef& cf, int li, int hd,
+                                               const float* __restrict__ gain,
+                                               const float* __restrict__ cos_t,
+                                               const float* __restrict__ sin_t, int pos) {
+  const int half = hd / 2;
+  cf.has_gain = gain != nullptr;
+  cf.has_rotation = cos_t != nullptr;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    cf.g0[e] = cf.has_gain ? gain[4 * li + e] : 1.f;
+    cf.g1[e] = cf.has_gain ? gain[half + 4 * li + e] : 1.f;
+    cf.c[e] = cf.has_rotation ? cos_t[(size_t)pos * half + 4 * li + e] : 1.f;
+    cf.sn[e] = cf.has_rotation ? sin_t[(size_t)pos * half + 4 * li + e] : 0.f;
+  }
+}
+template <int LPH>
+__device__ __forceinline__ void head_norm_rotate(float (&x0)[4], float (&x1)[4], int hd,
+                                                 bool active, float eps, const HeadCoef& cf) {
+  if (cf.has_gain) {
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ss += x0[e] * x0[e] + x1[e] * x1[e];
+#pragma unroll
+    for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
+    if (active) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        x0[e] = x0[e] * inv * cf.g0[e];
+        x1[e] = x1[e] * inv * cf.g1[e];
+      }
+    }
+  }
+  if (active && cf.has_rotation) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float r0 = x0[e] * cf.c[e] - x1[e] * cf.sn[e];
+      const float r1 = x1[e] * cf.c[e] + x0[e] * cf.sn[e];
+      x0[e] = r0;
+      x1[e] = r1;
+    }
+  }
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int off = ZF_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, ZF_WAVE);

@@ -783,6 +783,63 @@ def mfma_attention_covers(dtype, n_heads, n_kv_heads, head_dim, page_size) -> bo
         and n_heads // n_kv_heads <= 16
 
 
+# Up to this many sequences a decode step's attention does the work of qk_norm_rope_kv_write
+# itself.  Measured on MI355X (Qwen3-8B shape, context 2100, per layer, against the two kernels
+# one after the other): 11.2 -> 8.2 us at batch 1, 15.0 -> 13.1 at 4, 19.1 -> 18.2 at 8,
+# 30.2 -> 29.3 at 16, 51.0 -> 50.0 at 32, but 94.6 -> 95.7 at 64, where the chip is busy
+# streaming keys and values and a workgroup's longer start costs more than a launch.
+FUSED_DECODE_MAX_SEQS = 32
+
+
+def decode_attention_fused(qkv, q_gain, k_gain, eps, cos, sin, positions, slot_mapping, k_pool,
+                           v_pool, block_table, q_start, ctx_len, out, scale, window, n_heads,
+                           n_kv_heads, head_dim, page_size, max_ctx_len) -> None:
+    """A decode step's attention straight from the q/k/v product: every sequence has exactly
+    one token (token s is sequence s's), ``qkv`` [n_seqs, (nH + 2 nKV) hd] is read and not
+    changed.  What ``qk_norm_rope_kv_write`` and ``paged_attention`` do one after the other
+    (per-head RMSNorm of q and k, rotation at ``positions``, the token's key and value into the
+    pools at ``slot_mapping``, attention over the cache) in one kernel less, with the same
+    arithmetic and so the same bits.  Only for shapes ``mfma_attention_covers``."""
+    _need_gpu(qkv, q_gain, k_gain, cos, sin, positions, slot_mapping, k_pool, v_pool, block_table,
+              q_start, ctx_len, out)
+    n_seqs = ctx_len.shape[0]
+    width = (n_heads + 2 * n_kv_heads) * head_dim
+    if not mfma_attention_covers(qkv.dtype, n_heads, n_kv_heads, head_dim, page_size):
+        raise KernelUnavailable("decode_attention_fused: bfloat16, head_dim 32/64/128/256, pages "
+                                "of a multiple of 16 rows and at most 16 query heads per kv head")
+    if qkv.shape != (n_seqs, width) or out.shape != (n_seqs, n_heads * head_dim) \
+            or out.dtype != qkv.dtype or k_pool.dtype != qkv.dtype or v_pool.dtype != qkv.dtype:
+        raise KernelUnavailable("decode_attention_fused: qkv must be [n_seqs, (nH + 2 nKV) * hd] "
+                                "and out [n_seqs, nH * hd], of the pools' dtype")
+    if (q_gain is None) != (k_gain is None) or (cos is None) != (sin is None):
+        raise KernelUnavailable("decode_attention_fused: gains and tables come in pairs")
+    for g in (q_gain, k_gain):
+        if g is not None and (g.dtype != torch.float32 or g.shape != (head_dim,)):
+            raise KernelUnavailable("decode_attention_fused: a gain must be float32 [head_dim]")
+    if cos is not None and (cos.dtype != torch.float32 or cos.shape[1] != head_dim // 2
+                            or cos.shape != sin.shape):
+        raise KernelUnavailable("decode_attention_fused: tables must be float32 [*, head_dim/2]")
+    for t, name in ((block_table, "block_table"), (q_start, "q_start"), (ctx_len, "ctx_len"),
+                    (positions, "positions"), (slot_mapping, "slot_mapping")):
+        _i32(t, name)
+    if q_start.shape[0] != n_seqs + 1 or block_table.shape[0] != n_seqs \
+            or positions.shape[0] != n_seqs or slot_mapping.shape[0] != n_seqs:
+        raise KernelUnavailable("decode_attention_fused: per-sequence arrays disagree in length")
+    if max_ctx_len > block_table.shape[1] * page_size:
+        raise KernelUnavailable("decode_attention_fused: block table shorter than the context")
+    max_splits = (max_ctx_len + DECODE_SPLIT_KEYS - 1) // DECODE_SPLIT_KEYS
+    ws_o = _workspace("attn_o", n_seqs * n_heads * max_splits * head_dim, torch.float32,
+                      qkv.device)
+    ws_ml = _workspace("attn_ml", n_seqs * n_heads * max_splits * 2, torch.float32, qkv.device)
+    lib = build.load("attention")
+    _check(lib.zf_attn_decode_fused_bf16(
+        _ptr(qkv), _ptr(q_gain), _ptr(k_gain), ctypes.c_float(eps), _ptr(cos), _ptr(sin),
+        _ptr(positions), _ptr(slot_mapping), _ptr(k_pool), _ptr(v_pool), _ptr(block_table),
+        _ptr(q_start), _ptr(ctx_len), _ptr(out), _ptr(ws_o), _ptr(ws_ml), ctypes.c_float(scale),
+        int(window), n_seqs, n_heads, n_kv_heads, head_dim, page_size, block_table.shape[1],
+        max_splits, _stream()), "decode_attention_fused")
+
+
 def _prefill_key_split(n_query_tiles: int, n_kv_heads: int, max_ctx_len: int):
     """(keys per split, splits) if a prompt portion's attention should also split its keys over
     workgroups: few query tiles behind a long context (a 512-token portion at context 4096: 128

@@ -7,8 +7,8 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Callable, Dict
 
-from . import (advance_decode, apply_penalties, argmax, argmax_no_alloc, cast, embed, gather_rows,
-               gemm, gemm_emit, gemm_given, gemm_sum_norm, gemm_swiglu, norm_gemm, paged_attention,
+from . import (advance_decode, apply_penalties, argmax, argmax_no_alloc, cast,
+               decode_attention_fused, embed, gather_rows, gemm, gemm_emit, gemm_given, gemm_sum_norm, gemm_swiglu, norm_gemm, paged_attention,
                poison_pages, qk_norm_rope_kv_write, randinit, rmsnorm, sample_topk, scale_cap, swiglu)
 
 
@@ -42,6 +42,9 @@ KERNELS: Dict[str, KernelEntry] = {
     "gemm_sum_norm": KernelEntry(gemm_sum_norm, "gemm", "tests/kernel_refs.py:rmsnorm"),
     "paged_attention": KernelEntry(paged_attention, "attention",
                                    "tests/kernel_refs.py:paged_attention"),
+    "decode_attention_fused": KernelEntry(
+        decode_attention_fused, "attention",
+        "tests/test_kernels_gpu.py:test_decode_attention_fused_equals_the_two_kernels"),
     "apply_penalties": KernelEntry(apply_penalties, "sampling",
                                    "zinfer_amd/sampling/sampler.py:adjust_logits"),
     "sample_topk": KernelEntry(sample_topk, "sampling",

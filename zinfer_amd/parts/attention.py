@@ -78,11 +78,27 @@ class GqaAttention(Mixer):
         act = self.ctx.act_dtype
         qkv = step.scratch("qkv", (T, self.q_width + 2 * self.kv_width), act)
         self.qkv.forward(h, qkv)
-        q = step.scratch("q", (T, self.q_width), act)
         tables = self.position.rotation_tables()
         kv = step.kv_tables(cache.group)
         eps = float(s.qk_norm_eps) if s.qk_norm_eps is not None else 0.0
-        if tables is not None or not self.position.custom_apply:
+        attn = step.scratch("attn", (T, self.q_width), act)
+        window = 0 if s.window is None else int(s.window)
+        plain_position = tables is not None or not self.position.custom_apply
+        if plain_position and step.max_q_len == 1 and cache.writes \
+                and step.n_seqs <= ops.FUSED_DECODE_MAX_SEQS and ops.mfma_attention_covers(
+                    act, s.n_heads, s.n_kv_heads, s.head_dim, cache.page_size):
+            # a decode step: the attention kernel norms and rotates q and k and stores the
+            # token's key and value itself (one kernel less, the same bits)
+            cos, sin = tables if tables is not None else (None, None)
+            ops.decode_attention_fused(
+                qkv, self.q_gain, self.k_gain, eps, cos, sin, step.positions, kv.slot_mapping,
+                cache.k_pool, cache.v_pool, kv.block_table, step.q_start, step.ctx_len, attn,
+                float(self.scale), window, s.n_heads, s.n_kv_heads, s.head_dim, cache.page_size,
+                step.max_ctx_len)
+            self.o.forward(attn, residual, accumulate=True, step=step)
+            return
+        q = step.scratch("q", (T, self.q_width), act)
+        if plain_position:
             cos, sin = tables if tables is not None else (None, None)
             ops.qk_norm_rope_kv_write(
                 qkv, self.q_gain, self.k_gain, eps, cos, sin, step.positions,
@@ -100,10 +116,8 @@ class GqaAttention(Mixer):
                                       kv.slot_mapping if cache.writes else None,
                                       cache.k_pool, cache.v_pool, q,
                                       s.n_heads, s.n_kv_heads, s.head_dim, cache.page_size)
-        attn = step.scratch("attn", (T, self.q_width), act)
         ops.paged_attention(q, cache.k_pool, cache.v_pool, kv.block_table, step.q_start,
-                            step.ctx_len, step.seq_index, attn, float(self.scale),
-                            0 if s.window is None else int(s.window),
+                            step.ctx_len, step.seq_index, attn, float(self.scale), window,
                             s.n_heads, s.n_kv_heads, s.head_dim, cache.page_size,
                             step.max_q_len, step.max_ctx_len, n_single=step.n_single,
                             n_query_tiles=step.n_query_tiles, q_tile_map=step.q_tile_map,
