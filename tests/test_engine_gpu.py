@@ -335,6 +335,40 @@ def test_graph_replays_with_forty_requests(tmp_path_factory):
         assert err <= LOGITS_TOL_BF16, (r, err)
 
 
+@pytest.mark.parametrize("name", ["D", "E"])
+def test_decode_attention_fused_or_not_gives_the_same_logits(name, tmp_path_factory, monkeypatch):
+    """A decode step whose attention kernel norms and rotates q and k and writes the cache
+    itself (steps of few sequences) against the same step with those as a kernel of their
+    own (as in larger and in mixed steps): the same bits in the logits, step after step over
+    page edges, and the same tokens afterwards from a step that reads all that was written."""
+    from zinfer_amd import ops
+    from zinfer_amd.engine import Engine, StepEntry
+    from zinfer_amd.models.build import load_model
+    path = tiny.model_dir_of(name, str(tmp_path_factory.getbasetemp()), torch.bfloat16)
+    V = tiny.CONFIGS[name]["vocab_size"]
+    reqs = {f"f{i}": tiny.random_tokens(n, V, 900 + i) for i, n in enumerate((31, 16, 47, 5, 64))}
+    engines = []
+    for _ in range(2):
+        _, model = load_model(path, "bfloat16", DEV)
+        engines.append(Engine(model, page_size=16, num_pages=40, max_requests=8, use_graphs=False))
+    fused, apart = engines
+    assert ops.FUSED_DECODE_MAX_SEQS >= len(reqs)
+    lg = None
+    for eng in engines:
+        lg = eng.step([StepEntry(r, t, [len(t) - 1]) for r, t in reqs.items()])
+    cur = fused.argmax(lg)
+    for k in range(20):
+        entries = [StepEntry(r, [t], [0]) for r, t in zip(reqs, cur)]
+        la = fused.step(entries)
+        monkeypatch.setattr(ops, "FUSED_DECODE_MAX_SEQS", 0)
+        lb = apart.step(entries)
+        monkeypatch.undo()
+        assert torch.equal(la, lb), f"decode step {k}"
+        cur = fused.argmax(la)
+    for eng in engines:
+        eng.cache.check()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decode_steps_in_a_row_equal_single_steps(dtype, tmp_path_factory):
     """Several decode steps without the host between them (the device moves tokens,
