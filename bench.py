@@ -120,6 +120,14 @@ def run_prefill(llm, cfg, T: int, seed: int) -> float:
     return min(times[1:])
 
 
+def decode_lead(batch: int, prompt_len: int, step_tokens: int) -> int:
+    """How many tokens the first request of ``batch`` may have decoded by the time the last
+    one's prompt is through: a step's token budget is shared between one prompt's portion and
+    the decode tokens of the requests already running."""
+    room = max(1, step_tokens - batch)
+    return batch * ((prompt_len + room - 1) // room)
+
+
 def run_decode(llm, cfg, batch: int, prompt_len: int, steps: int, warmup: int, seed: int):
     """Prefills ``batch`` requests through the scheduler, runs ``warmup`` untimed decode
     steps, then times exactly ``steps`` steps.  Returns (seconds, mean context length)."""
@@ -131,7 +139,7 @@ def run_decode(llm, cfg, batch: int, prompt_len: int, steps: int, warmup: int, s
     sched.chunk_size = sched.max_step_tokens
     # requests admitted early decode while later prompts are still being run, so they may be
     # many tokens ahead; none may finish before the timed steps are over
-    ahead = batch * ((prompt_len + sched.chunk_size - 1) // sched.chunk_size)
+    ahead = decode_lead(batch, prompt_len, sched.chunk_size)
     params = SamplingParams(temperature=0.0, max_new_tokens=warmup + steps + ahead + 8,
                             ignore_eos=True)
     for _ in range(batch):
@@ -377,12 +385,14 @@ def main_decode(args) -> int:
     if args.layers is not None:
         raw["num_hidden_layers"] = args.layers
     max_batch = args.batch if args.no_points else max(args.batch, 64)
-    ctx_cap = args.prompt_len + args.warmup + args.steps + max_batch + 64
+    step_tokens = max(2048, args.prompt_len)
+    ctx_cap = args.prompt_len + args.warmup + args.steps + 64 \
+        + decode_lead(max_batch, args.prompt_len, min(step_tokens, 8192))
     longest_prefill = args.prefill_tokens if args.no_points else max(args.prefill_tokens, 8192)
     tokens = max(max_batch * ctx_cap, longest_prefill + 64)
     t_build = time.perf_counter()
     llm = build_llm(raw, args.dtype, args.seed, tokens, max_batch,
-                    max_step_tokens=max(2048, args.prompt_len), multi_step=args.multi_step)
+                    max_step_tokens=step_tokens, multi_step=args.multi_step)
     cfg = llm.config
     build_s = time.perf_counter() - t_build
     elem = 2 if args.dtype == "bfloat16" else 4
