@@ -638,7 +638,47 @@ def test_decode_attention_fused_equals_the_two_kernels(nH, nKV, hd, page_size, w
     array)."""
     from zinfer_amd.parts.position import rotary_tables
     dtype, ops = torch.bfloat16, _ops()
-    ctx_lens = [1, 15, 16, 17, 255, 256, 257, 600, 1025, 512, 513]
+    _fused_against_two_kernels(ops, nH, nKV, hd, page_size, window, use_norm, use_rope,
+                               [1, 15, 16, 17, 255, 256, 257, 600, 1025, 512, 513])
+    # no context beyond one split: the attention kernels write the output themselves
+    _fused_against_two_kernels(ops, nH, nKV, hd, page_size, window, use_norm, use_rope,
+                               [1, 2, 16, 17, 100, 255, 256])
+
+
+@pytest.mark.parametrize("nH,nKV,hd,page_size,window", [(32, 8, 128, 16, 0), (6, 2, 64, 32, 20),
+                                                        (16, 1, 32, 16, 0), (6, 3, 256, 16, 0)])
+def test_decode_attention_one_split_writes_what_the_merge_would(nH, nKV, hd, page_size, window):
+    """No context beyond 256 keys: the decode attention writes its output itself and the merge
+    kernel is not launched.  The same batch with a context bound of two splits (as a wider
+    block table gives it) goes through the merge kernel: the same bits."""
+    dtype, ops = torch.bfloat16, _ops()
+    ctx_lens = [1, 2, 16, 17, 100, 255, 256]
+    n = len(ctx_lens)
+    s = _paged_setup(dtype, nH, nKV, hd, page_size, ctx_lens, [1] * n, seed=31)
+    d = {k: v.to(DEV) for k, v in s.items() if isinstance(v, torch.Tensor)}
+    d["k_pool"] = ref.tile_k_pool(d["k_pool"], nKV, page_size, hd)
+    d["v_pool"] = ref.tile_v_pool(d["v_pool"], nKV, page_size, hd)
+    wide = torch.full((n, 512 // page_size + 1), -1, dtype=torch.int32, device=DEV)
+    wide[:, :d["block_table"].shape[1]] = d["block_table"]
+    outs = []
+    for table, bound in ((d["block_table"], 256), (wide, 512)):
+        out = torch.full((n, nH * hd), float("nan"), dtype=dtype, device=DEV)
+        ops.paged_attention(d["q"], d["k_pool"], d["v_pool"], table, d["q_start"], d["ctx_len"],
+                            d["seq_index"], out, 1.0 / math.sqrt(hd), window, nH, nKV, hd,
+                            page_size, 1, bound, n_single=n)
+        outs.append(out)
+    assert not torch.isnan(outs[0].float()).any()
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+    want = torch.empty((n, nH * hd), dtype=dtype)
+    ref.paged_attention(s["q"], s["k_pool"], s["v_pool"], s["block_table"], s["q_start"],
+                        s["ctx_len"], s["seq_index"], want, 1.0 / math.sqrt(hd), window, nH, nKV,
+                        hd, page_size, 1, 256)
+    assert rel_err(outs[0], want) <= 2 * tol(dtype)
+
+
+def _fused_against_two_kernels(ops, nH, nKV, hd, page_size, window, use_norm, use_rope, ctx_lens):
+    from zinfer_amd.parts.position import rotary_tables
+    dtype = torch.bfloat16
     n = len(ctx_lens)
     s = _paged_setup(dtype, nH, nKV, hd, page_size, ctx_lens, [1] * n, seed=21)
     num_pages = s["k_pool"].shape[0]

@@ -285,7 +285,10 @@ __device__ __forceinline__ void decode_attend(const u32x4_t (&kf)[4][HD / 32],
 }
 
 // The four waves' partials combined through LDS in wave order; the workgroup writes one
-// un-normalised partial (max, sum, O[G, hd]) per query head for its split.
+// un-normalised partial (max, sum, O[G, hd]) per query head for its split.  With one split
+// (no context beyond 256 keys) it writes the output itself, out_row[col * HD + d] =
+// bfloat16(O / sum): what the merge kernel would make of a single partial, bit for bit, and
+// that kernel is not launched.
 template <int HD>
 __device__ __forceinline__ void decode_write_partial(float (&s_o)[4][16][HD], float (&s_m)[4][16],
                                                      float (&s_l)[4][16], int wave, int j, int qd,
@@ -293,7 +296,8 @@ __device__ __forceinline__ void decode_write_partial(float (&s_o)[4][16][HD], fl
                                                      const f32x4_t (&o)[HD / 16], int G,
                                                      size_t first_slot, int max_splits,
                                                      float* __restrict__ ws_o,
-                                                     float* __restrict__ ws_ml) {
+                                                     float* __restrict__ ws_ml,
+                                                     bf16_t* __restrict__ out_row) {
   // this wave's partial for query column j: rows d = 16 dt + 4 qd + r
 #pragma unroll
   for (int dt = 0; dt < HD / 16; ++dt) *(f32x4_t*)&s_o[wave][j][dt * 16 + 4 * qd] = o[dt];
@@ -314,6 +318,10 @@ __device__ __forceinline__ void decode_write_partial(float (&s_o)[4][16][HD], fl
       acc += f * s_o[w][col][d];
       den += f * s_l[w][col];
     }
+    if (max_splits == 1) {
+      out_row[idx] = float_to_bf16(acc / den);
+      continue;
+    }
     const size_t slot = first_slot + (size_t)col * max_splits;   // of (sequence, head, split)
     ws_o[slot * HD + d] = acc;
     if (d == 0) {
@@ -328,8 +336,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int* __restrict__ block_table,
     const int* __restrict__ q_start, const int* __restrict__ ctx_len, float* __restrict__ ws_o,
-    float* __restrict__ ws_ml, float scale_log2e, int window, int nH, int nKV, int ps,
-    int max_pages, int max_splits) {
+    float* __restrict__ ws_ml, bf16_t* __restrict__ out, float scale_log2e, int window, int nH,
+    int nKV, int ps, int max_pages, int max_splits) {
   __shared__ __attribute__((aligned(16))) float s_o[4][16][HD];
   __shared__ float s_m[4][16], s_l[4][16];
   const int kvh = blockIdx.x, sp = blockIdx.y, s = blockIdx.z;
@@ -388,7 +396,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     decode_attend<HD>(kf, vf, qf, kb, k_begin, k_end, qd, scale_log2e, m, l, o);
   }
   decode_write_partial<HD>(s_o, s_m, s_l, wave, j, qd, m, l, o, G,
-                           ((size_t)s * nH + kvh * G) * max_splits + sp, max_splits, ws_o, ws_ml);
+                           ((size_t)s * nH + kvh * G) * max_splits + sp, max_splits, ws_o, ws_ml,
+                           out + ((size_t)t * nH + kvh * G) * HD);
 }
 
 // What the fused decode kernel needs to do the work of the kernel before it as well (the
@@ -427,8 +436,9 @@ template <int HD>
 __global__ __launch_bounds__(256, HD <= 128 ? 3 : 1) void attn_decode_fused_kernel(
     const bf16_t* __restrict__ qkv, bf16_t* __restrict__ k_pool, bf16_t* __restrict__ v_pool,
     const int* __restrict__ block_table, const int* __restrict__ ctx_len,
-    float* __restrict__ ws_o, float* __restrict__ ws_ml, float scale_log2e, int window, int nH,
-    int nKV, int ps, int max_pages, int max_splits, DecodeFused fu) {
+    float* __restrict__ ws_o, float* __restrict__ ws_ml, bf16_t* __restrict__ out,
+    float scale_log2e, int window, int nH, int nKV, int ps, int max_pages, int max_splits,
+    DecodeFused fu) {
   __shared__ __attribute__((aligned(16))) float s_o[4][16][HD];
   __shared__ float s_m[4][16], s_l[4][16];
   // rows 0 .. G - 1: the query heads; row 16: the new key; row 17: the new value
@@ -583,7 +593,8 @@ __global__ __launch_bounds__(256, HD <= 128 ? 3 : 1) void attn_decode_fused_kern
                             s_q[16], s_q[17]);
   }
   decode_write_partial<HD>(s_o, s_m, s_l, wave, j, qd, m, l, o, G,
-                           ((size_t)s * nH + kvh * G) * max_splits + sp, max_splits, ws_o, ws_ml);
+                           ((size_t)s * nH + kvh * G) * max_splits + sp, max_splits, ws_o, ws_ml,
+                           out + ((size_t)s * nH + kvh * G) * HD);
 }
 
 // Combines the splits of one (sequence, head) and writes bfloat16.  One workgroup of 4 waves.
@@ -667,6 +678,7 @@ __global__ __launch_bounds__(256) void attn_decode_merge_kernel(
 static int launch_decode_merge(const float* ws_o, const float* ws_ml, const int* q_start,
                                const int* ctx_len, void* out, int window, int n_seqs, int nH,
                                int hd, int max_splits, hipStream_t stream) {
+  if (max_splits == 1) return (int)hipGetLastError();     // the attention kernel wrote the output
 #define ZF_DEC_MERGE(HD)                                                                        \
   hipLaunchKernelGGL(attn_decode_merge_kernel<HD>, dim3(n_seqs, nH), dim3(256), 0, stream, ws_o, \
                      ws_ml, q_start, ctx_len, (bf16_t*)out, window, nH, max_splits)
@@ -691,8 +703,8 @@ extern "C" int zf_attn_decode_bf16(const void* q, const void* k_pool, const void
 #define ZF_DEC(HD)                                                                              \
   hipLaunchKernelGGL(attn_decode_kernel<HD>, grid, dim3(256), 0, stream, (const bf16_t*)q,      \
                      (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, q_start,        \
-                     ctx_len, ws_o, ws_ml, scale_log2e, window, nH, nKV, page_size, max_pages,  \
-                     max_splits)
+                     ctx_len, ws_o, ws_ml, (bf16_t*)out, scale_log2e, window, nH, nKV,          \
+                     page_size, max_pages, max_splits)
   if (hd == 32) ZF_DEC(32);
   else if (hd == 64) ZF_DEC(64);
   else if (hd == 128) ZF_DEC(128);
@@ -730,8 +742,8 @@ extern "C" int zf_attn_decode_fused_bf16(const void* qkv, const float* q_gain,
 #define ZF_DEC(HD)                                                                              \
   hipLaunchKernelGGL(attn_decode_fused_kernel<HD>, grid, dim3(256), 0, stream,                  \
                      (const bf16_t*)qkv, (bf16_t*)k_pool, (bf16_t*)v_pool, block_table,         \
-                     ctx_len, ws_o, ws_ml, scale_log2e, window, nH, nKV, page_size, max_pages,  \
-                     max_splits, fu)
+                     ctx_len, ws_o, ws_ml, (bf16_t*)out, scale_log2e, window, nH, nKV,          \
+                     page_size, max_pages, max_splits, fu)
   if (hd == 32) ZF_DEC(32);
   else if (hd == 64) ZF_DEC(64);
   else if (hd == 128) ZF_DEC(128);

@@ -330,6 +330,10 @@ class Engine:
         max_ctx = max(ctx_lens) + extra_tokens
         if bucket_pages:      # a fixed table width (and context bound) per captured graph
             b = self.GRAPH_PAGE_BUCKET
+            from ..ops import DECODE_SPLIT_KEYS
+            short = max(1, DECODE_SPLIT_KEYS // ps)
+            if max_pages <= short:
+                b = short     # contexts within one split of the decode attention: no merge kernel
             max_pages = (max_pages + b - 1) // b * b
             max_ctx = max_pages * ps
 
