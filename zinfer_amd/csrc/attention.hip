@@ -422,12 +422,12 @@ struct DecodeFused {
 //
 // Order.  A lane's loads return in the order it asked for them, so whatever the norm and
 // rotation need from memory is asked for first and the keys right behind it: the arithmetic
-// then runs while the keys' loads are in flight and waits for none of them.  The values are
-// asked for behind the arithmetic (with both in flight beside what the norm holds, three
-// waves would no longer fit a SIMD's registers); they are needed last.  The wave that holds
-// the token's own position cannot read it from the cache (the stores come later than its
-// loads of the keys): it takes the new key and value from LDS into the operand registers of
-// the lanes that hold that position, once its loads have landed.
+// then runs while the keys' loads are in flight and waits for none of them.  At head size 128
+// half of the values are asked for with the keys and half behind the arithmetic (with all 48
+// loads in flight beside what the norm holds, three waves would no longer fit a SIMD's
+// registers); they are needed last.  The wave that holds the token's own position cannot
+// read it from the cache (the stores come later than its loads): decode_attend takes the new
+// key and value from LDS instead (PATCH).
 //
 // The page of a 16-key group is the same for a whole wave, so the look-ups and the blocks'
 // addresses are scalar and a load's address is one of them plus a lane's offset: the loads
