@@ -787,7 +787,9 @@ def mfma_attention_covers(dtype, n_heads, n_kv_heads, head_dim, page_size) -> bo
 # itself.  Measured on MI355X (Qwen3-8B shape, context 2100, per layer, against the two kernels
 # one after the other): 11.2 -> 8.2 us at batch 1, 15.0 -> 13.1 at 4, 19.1 -> 18.2 at 8,
 # 30.2 -> 29.3 at 16, 51.0 -> 50.0 at 32, but 94.6 -> 95.7 at 64, where the chip is busy
-# streaming keys and values and a workgroup's longer start costs more than a launch.
+# streaming keys and values and a workgroup's longer start costs more than a launch.  At
+# context 32768 it gains at batch 1, 8 and 16 alike (245 -> 255, 853 -> 864, 1008 -> 1012
+# tokens/s): what costs at batch 64 is the eighth of the workgroups that also store a key.
 FUSED_DECODE_MAX_SEQS = 32
 
 
