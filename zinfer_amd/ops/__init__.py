@@ -789,7 +789,7 @@ def mfma_attention_covers(dtype, n_heads, n_kv_heads, head_dim, page_size) -> bo
 # 30.2 -> 29.3 at 16, 51.0 -> 50.0 at 32, but 94.6 -> 95.7 at 64, where the chip is busy
 # streaming keys and values and a workgroup's longer start costs more than a launch.  At
 # context 32768 it gains at batch 1, 8 and 16 alike (245 -> 255, 853 -> 864, 1008 -> 1012
-# tokens/s): what costs at batch 64 is the eighth of the workgroups that also store a key.
+# tokens/s): there one workgroup in 128 also norms and stores a key, at context 2100 one in 9.
 FUSED_DECODE_MAX_SEQS = 32
 
 
