@@ -335,6 +335,41 @@ def test_graph_replays_with_forty_requests(tmp_path_factory):
         assert err <= LOGITS_TOL_BF16, (r, err)
 
 
+def test_forty_decode_tokens_with_the_partials_handed_on_or_added_first(tmp_path_factory, monkeypatch):
+    """Forty decode tokens at the served widths: the q/k/v product runs split along K and hands
+    its partials to the kernel that norms, rotates and stores; with that switched off a kernel
+    adds them first.  The same bits in the logits, step after step."""
+    from zinfer_amd import ops
+    from zinfer_amd.engine import Engine, StepEntry
+    from zinfer_amd.models.build import load_model
+    from zinfer_amd.parts.linear import Linear
+    name = "W"
+    path = tiny.model_dir_of(name, str(tmp_path_factory.getbasetemp()), torch.bfloat16)
+    cfg = tiny.CONFIGS[name]
+    V = cfg["vocab_size"]
+    width = (cfg["num_attention_heads"] + 2 * cfg["num_key_value_heads"]) * cfg["head_dim"]
+    reqs = {f"p{i}": tiny.random_tokens(3 + i % 5, V, 950 + i) for i in range(40)}
+    engines = []
+    for _ in range(2):
+        _, model = load_model(path, "bfloat16", DEV)
+        engines.append(Engine(model, page_size=16, num_pages=40 * 2 + 8, max_requests=48,
+                              use_graphs=False))
+    handed, added = engines
+    assert ops._small_plan(40, width, cfg["hidden_size"], True)[:1] == ("mid",), "not the product meant"
+    lg = None
+    for eng in engines:
+        lg = eng.step([StepEntry(r, t, [len(t) - 1]) for r, t in reqs.items()])
+    cur = handed.argmax(lg)
+    for k in range(4):
+        entries = [StepEntry(r, [t], [0]) for r, t in zip(reqs, cur)]
+        la = handed.step(entries)
+        monkeypatch.setattr(Linear, "forward_partials", lambda self, x: None)
+        lb = added.step(entries)
+        monkeypatch.undo()
+        assert torch.equal(la, lb), f"decode step {k}"
+        cur = handed.argmax(la)
+
+
 @pytest.mark.parametrize("name", ["D", "E"])
 def test_decode_attention_fused_or_not_gives_the_same_logits(name, tmp_path_factory, monkeypatch):
     """A decode step whose attention kernel norms and rotates q and k and writes the cache

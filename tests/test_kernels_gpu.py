@@ -645,6 +645,48 @@ def test_decode_attention_fused_equals_the_two_kernels(nH, nKV, hd, page_size, w
                                [1, 2, 16, 17, 100, 255, 256])
 
 
+@pytest.mark.parametrize("M,nH,nKV,hd,page_size,H", [(64, 32, 8, 128, 16, 4096), (40, 8, 2, 64, 16, 2048),
+                                                     (33, 4, 4, 128, 32, 4096), (128, 16, 2, 128, 16, 5120)])
+def test_qk_norm_rope_kv_write_from_a_split_products_partials(M, nH, nKV, hd, page_size, H):
+    """17 to 128 tokens: the q/k/v product runs split along K.  Its partials handed to the
+    kernel that norms, rotates and stores give the bits of the usual way (a kernel adds the
+    partials into bfloat16 rows, then that kernel): q and both pools."""
+    from zinfer_amd.parts.position import rotary_tables
+    ops, dtype = _ops(), torch.bfloat16
+    N = (nH + 2 * nKV) * hd
+    w = ops.pretile_weight((_rand((N, H), dtype, 41) * 0.05).to(DEV))
+    ks = ops.gemm_partials_plan(M, N, H, w, True)
+    assert ks is not None and ks > 1, "the test means a product that is split along K"
+    a = _rand((M, H), dtype, 42).to(DEV)
+    qg = (1 + 0.1 * _rand((hd,), torch.float32, 43)).to(DEV)
+    kg = (1 + 0.1 * _rand((hd,), torch.float32, 44)).to(DEV)
+    cos, sin = (t.to(DEV) for t in rotary_tables(hd, 10000.0, 400))
+    positions = torch.arange(M, dtype=torch.int32, device=DEV) * 3 % 400
+    num_pages = (M + page_size - 1) // page_size + 2
+    slots = torch.randperm(num_pages * page_size, generator=torch.Generator().manual_seed(2))[:M]
+    slots = slots.int().to(DEV)
+    row = nKV * page_size * hd
+    outs = []
+    for way in ("usual", "partials"):
+        kp = torch.zeros((num_pages, row), dtype=dtype, device=DEV)
+        vp = torch.zeros((num_pages, row), dtype=dtype, device=DEV)
+        q = torch.full((M, nH * hd), float("nan"), dtype=dtype, device=DEV)
+        if way == "usual":
+            qkv = torch.empty((M, N), dtype=dtype, device=DEV)
+            ops.gemm(a, w, qkv, w_tiled=True)
+        else:
+            qkv = ops.gemm_partials(a, w, ks)
+            assert qkv.shape == (ks, M, N)
+        ops.qk_norm_rope_kv_write(qkv, qg, kg, 1e-6, cos, sin, positions, slots, kp, vp, q, nH, nKV,
+                                  hd, page_size)
+        outs.append((q, kp, vp))
+    torch.cuda.synchronize()
+    bits = lambda t: t.view(torch.int16)
+    assert not torch.isnan(outs[0][0].float()).any()
+    for x, y in zip(*outs):
+        assert torch.equal(bits(x), bits(y))
+
+
 @pytest.mark.parametrize("nH,nKV,hd,page_size,window", [(32, 8, 128, 16, 0), (6, 2, 64, 32, 20),
                                                         (16, 1, 32, 16, 0), (6, 3, 256, 16, 0)])
 def test_decode_attention_one_split_writes_what_the_merge_would(nH, nKV, hd, page_size, window):

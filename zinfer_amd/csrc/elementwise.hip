@@ -226,13 +226,19 @@ __global__ void qk_norm_rope_kv_write_kernel(
 // under the rotation, LPH = the next power of two >= hd / 8 lanes work on a head and a wave
 // takes 64 / LPH heads of one token, so that loads and stores are 8 or 16 bytes wide and
 // there are far fewer waves than (token, head) pairs.
-template <typename T, int LPH>
+//
+// PART: the rows do not come as qkv but as the float32 partials [ksplit, T, (nH + 2 nKV) * hd]
+// that a product split along K left: a lane adds its elements' partials in split order and
+// rounds the sum to bfloat16, as the kernel that only adds partials would have written it, and
+// goes on from there (one launch less; q goes to q_out, k and v into the pools).
+template <typename T, int LPH, bool PART = false>
 __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_vec_kernel(
     T* __restrict__ qkv, const float* __restrict__ q_gain, const float* __restrict__ k_gain,
     float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int* __restrict__ positions, const int* __restrict__ slot_mapping,
     T* __restrict__ k_pool, T* __restrict__ v_pool, T* __restrict__ q_out, int nH, int nKV,
-    int hd, int page_size, int tiled) {
+    int hd, int page_size, int tiled, const float* __restrict__ partials, int ksplit,
+    size_t split_stride) {
   constexpr int HPW = 64 / LPH;
   const int t = blockIdx.x;
   const int lane = threadIdx.x % 64, li = lane % LPH;
@@ -244,7 +250,21 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_vec_kernel(
   const int row_width = (nH + 2 * nKV) * hd;
   T* src = qkv + (size_t)t * row_width + (size_t)min(head, nH + 2 * nKV - 1) * hd;
   float x0[4] = {0.f, 0.f, 0.f, 0.f}, x1[4] = {0.f, 0.f, 0.f, 0.f};
-  if (active) {
+  if (PART && active) {
+    const float* p = partials + (size_t)t * row_width +
+                     (size_t)min(head, nH + 2 * nKV - 1) * hd + 4 * li;
+    float4 s0 = float4{0.f, 0.f, 0.f, 0.f}, s1 = s0;
+    for (int k = 0; k < ksplit; ++k) {
+      const float4 a = *(const float4*)(p + (size_t)k * split_stride);
+      const float4 b = *(const float4*)(p + (size_t)k * split_stride + half);
+      s0.x += a.x; s0.y += a.y; s0.z += a.z; s0.w += a.w;
+      s1.x += b.x; s1.y += b.y; s1.z += b.z; s1.w += b.w;
+    }
+    x0[0] = bf16_to_float(float_to_bf16(s0.x)); x0[1] = bf16_to_float(float_to_bf16(s0.y));
+    x0[2] = bf16_to_float(float_to_bf16(s0.z)); x0[3] = bf16_to_float(float_to_bf16(s0.w));
+    x1[0] = bf16_to_float(float_to_bf16(s1.x)); x1[1] = bf16_to_float(float_to_bf16(s1.y));
+    x1[2] = bf16_to_float(float_to_bf16(s1.z)); x1[3] = bf16_to_float(float_to_bf16(s1.w));
+  } else if (active) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {     // consecutive: the compiler makes one load of each
       x0[e] = load_as_float<T>(src + 4 * li + e);
@@ -307,17 +327,20 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_vec_kernel(
   }
 }
 
-template <typename T>
+template <typename T, bool PART = false>
 static void launch_qk_vec(T* qkv, const float* q_gain, const float* k_gain, float eps,
                           const float* cos_t, const float* sin_t, const int* positions,
                           const int* slot_mapping, T* k_pool, T* v_pool, T* q_out, int Tn, int nH,
-                          int nKV, int hd, int page_size, int tiled, hipStream_t stream) {
+                          int nKV, int hd, int page_size, int tiled, hipStream_t stream,
+                          const float* partials = nullptr, int ksplit = 0) {
   const int lanes = hd / 8, heads = nH + 2 * nKV;
+  const size_t split_stride = (size_t)Tn * heads * hd;
 #define ZF_QKV(LPH)                                                                            \
-  hipLaunchKernelGGL((qk_norm_rope_kv_write_vec_kernel<T, LPH>),                               \
+  hipLaunchKernelGGL((qk_norm_rope_kv_write_vec_kernel<T, LPH, PART>),                         \
                      dim3(Tn, (heads + 256 / LPH - 1) / (256 / LPH)), dim3(256), 0, stream, qkv, \
                      q_gain, k_gain, eps, cos_t, sin_t, positions, slot_mapping, k_pool,       \
-                     v_pool, q_out, nH, nKV, hd, page_size, tiled)
+                     v_pool, q_out, nH, nKV, hd, page_size, tiled, partials, ksplit,           \
+                     split_stride)
   if (lanes <= 2) ZF_QKV(2);
   else if (lanes <= 4) ZF_QKV(4);
   else if (lanes <= 8) ZF_QKV(8);
@@ -332,9 +355,20 @@ extern "C" int zf_qk_norm_rope_kv_write(void* qkv, int dtype, const float* q_gai
                                         const float* sin_t, const int* positions,
                                         const int* slot_mapping, void* k_pool, void* v_pool,
                                         void* q_out, int T, int nH, int nKV, int hd,
-                                        int page_size, int tiled, hipStream_t stream) {
+                                        int page_size, int tiled, const float* partials,
+                                        int ksplit, hipStream_t stream) {
   if (T <= 0) return 0;
   if (tiled && (page_size % 16 != 0 || hd % 32 != 0)) return -2;
+  if (partials != nullptr) {
+    // rows from a split product's partials: bfloat16, q to q_out, k and v into the pools
+    if (dtype != ZF_BF16 || hd % 8 != 0 || hd > 512 || ksplit < 1 || q_out == nullptr ||
+        slot_mapping == nullptr)
+      return -2;
+    launch_qk_vec<bf16_t, true>(nullptr, q_gain, k_gain, eps, cos_t, sin_t, positions,
+                                slot_mapping, (bf16_t*)k_pool, (bf16_t*)v_pool, (bf16_t*)q_out,
+                                T, nH, nKV, hd, page_size, tiled, stream, partials, ksplit);
+    ZF_CHECK_LAUNCH();
+  }
   if (hd % 8 == 0 && hd <= 512) {
     if (dtype == ZF_F32)
       launch_qk_vec<float>((float*)qkv, q_gain, k_gain, eps, cos_t, sin_t, positions, slot_mapping,

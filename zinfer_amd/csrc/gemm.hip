@@ -1099,6 +1099,22 @@ extern "C" int zf_gemm_bf16_mid(const void* A, const void* W, void* C, void* ws,
   return launch_tile_wdirect<128, 128, 128, 32, 128>(A, W, C, M, N, K, epi, stream, ws, ksplit);
 }
 
+// The same product for 17 to 128 tokens with ksplit >= 2 workgroups along K, left as float32
+// partials [ksplit, M, N] in ws for a kernel of the caller's that adds them on its way.
+extern "C" int zf_gemm_bf16_mid_partials(const void* A, const void* W, void* ws, int M, int N,
+                                         int K, int ksplit, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (ksplit < 2 || ws == nullptr || M > 128) return -3;
+  if (M <= 32)
+    return launch_tile_wdirect<32, 128, 32, 32, 256>(A, W, ws, M, N, K, EPI_STORE_F32, stream, ws,
+                                                     ksplit, false);
+  if (M <= 64)
+    return launch_tile_wdirect<64, 128, 64, 32, 128>(A, W, ws, M, N, K, EPI_STORE_F32, stream, ws,
+                                                     ksplit, false);
+  return launch_tile_wdirect<128, 128, 128, 32, 128>(A, W, ws, M, N, K, EPI_STORE_F32, stream, ws,
+                                                     ksplit, false);
+}
+
 enum { NORM_NONE = 0, NORM_FOLD = 1, NORM_GIVEN = 2 };
 
 // What the weight-streaming kernel needs to know of an RMSNorm around it.

@@ -104,7 +104,21 @@ def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, cos, sin, positions, slot_ma
     with the [hd] gains, optional half-split rotation from the [max_pos, hd/2] tables at
     ``positions``; q goes to ``q_out`` [T, nH hd] (in place if None), k and v go into the
     pools at ``slot_mapping`` (k in place if None).  Pools of a shape the MFMA attention
-    kernels cover (``mfma_attention_covers``) are written in those kernels' own order."""
+    kernels cover (``mfma_attention_covers``) are written in those kernels' own order.
+
+    ``qkv`` may also be the float32 partials [ksplit, T, (nH + 2 nKV) hd] of a product split
+    along K (``gemm_partials``): the kernel adds them in split order and rounds to bfloat16
+    on its way, as the kernel that only adds them would have (bfloat16 pools, ``q_out`` and
+    ``slot_mapping`` given)."""
+    partials = qkv if qkv.dim() == 3 else None
+    if partials is not None:
+        if partials.dtype != torch.float32 or not partials.is_contiguous() or q_out is None \
+                or slot_mapping is None or k_pool.dtype != torch.bfloat16 \
+                or head_dim % 8 != 0 or head_dim > 512:
+            raise KernelUnavailable("qk_norm_rope_kv_write: partials must be contiguous float32 "
+                                    "[ksplit, T, width], with q_out, slot_mapping and bfloat16 "
+                                    "pools, head_dim a multiple of 8 up to 512")
+        qkv = partials[0]
     _need_gpu(qkv, q_gain, k_gain, cos, sin, positions, slot_mapping, k_pool, v_pool, q_out)
     T = qkv.shape[0]
     width = (n_heads + 2 * n_kv_heads) * head_dim
@@ -120,19 +134,23 @@ def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, cos, sin, positions, slot_ma
                             or cos.shape != sin.shape):
         raise KernelUnavailable("qk_norm_rope_kv_write: tables must be float32 [*, head_dim/2]")
     _i32(positions, "positions")
+    row_dtype = torch.bfloat16 if partials is not None else qkv.dtype
     if slot_mapping is not None:
         _i32(slot_mapping, "slot_mapping")
-        if k_pool.dtype != qkv.dtype or v_pool.dtype != qkv.dtype:
+        if k_pool.dtype != row_dtype or v_pool.dtype != row_dtype:
             raise KernelUnavailable("qk_norm_rope_kv_write: pools and qkv differ in dtype")
-    if q_out is not None and (q_out.dtype != qkv.dtype
+    if q_out is not None and (q_out.dtype != row_dtype
                               or q_out.shape != (T, n_heads * head_dim)):
         raise KernelUnavailable("qk_norm_rope_kv_write: q_out must be [T, nH * hd] of qkv's dtype")
     lib = build.load("elementwise")
     _check(lib.zf_qk_norm_rope_kv_write(
-        _ptr(qkv), _dt(qkv), _ptr(q_gain), _ptr(k_gain), ctypes.c_float(eps), _ptr(cos),
+        _ptr(None if partials is not None else qkv), 1 if partials is not None else _dt(qkv),
+        _ptr(q_gain), _ptr(k_gain),
+        ctypes.c_float(eps), _ptr(cos),
         _ptr(sin), _ptr(positions), _ptr(slot_mapping), _ptr(k_pool), _ptr(v_pool), _ptr(q_out),
         T, n_heads, n_kv_heads, head_dim, page_size,
-        1 if mfma_attention_covers(qkv.dtype, n_heads, n_kv_heads, head_dim, page_size) else 0,
+        1 if mfma_attention_covers(row_dtype, n_heads, n_kv_heads, head_dim, page_size) else 0,
+        _ptr(partials), 0 if partials is None else partials.shape[0],
         _stream()), "qk_norm_rope_kv_write")
 
 
@@ -576,6 +594,34 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         return
     _check(lib.zf_gemm_fma(_ptr(a), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), M, N, K,
                            1 if accumulate else 0, _stream()), "gemm")
+
+
+def gemm_partials_plan(M: int, N: int, K: int, w: torch.Tensor, w_tiled: bool):
+    """Workgroups along K if ``gemm`` would run a stored product a w^T through the kernel for
+    17 to 128 tokens split along K (whose partials a second kernel then adds), else None: the
+    partials can instead go to a kernel of the caller's that adds them on its way
+    (``gemm_partials``)."""
+    if not (w_tiled and w.dtype == torch.bfloat16 and w.is_cuda and 16 < M <= MID_MAX_M):
+        return None
+    plan = _small_plan(M, N, K, True)
+    return plan[1] if plan is not None and plan[0] == "mid" and plan[1] > 1 else None
+
+
+def gemm_partials(a: torch.Tensor, w: torch.Tensor, ksplit: int) -> torch.Tensor:
+    """The float32 partials [ksplit, M, N] of a w^T (``w`` pre-tiled, 17 to 128 rows of
+    ``a``) in a work buffer that the next split product overwrites; their sum in split order,
+    rounded, is what ``gemm`` stores."""
+    _need_gpu(a, w)
+    M, K = a.shape
+    N = w.shape[0]
+    if a.dtype != torch.bfloat16 or w.shape[1] != K or not can_pretile(w) \
+            or gemm_partials_plan(M, N, K, w, True) != ksplit:
+        raise KernelUnavailable("gemm_partials: not a product that gemm_partials_plan covers")
+    ws = _workspace("gemm_splitk", ksplit * M * N, torch.float32, a.device)
+    lib = build.load("gemm")
+    _check(lib.zf_gemm_bf16_mid_partials(_ptr(a), _ptr(w), _ptr(ws), M, N, K, ksplit, _stream()),
+           "gemm_partials")
+    return ws[:ksplit * M * N].view(ksplit, M, N)
 
 
 def norm_gemm_plan(M: int, N: int, K: int, w: torch.Tensor, w_tiled: bool):

@@ -8,8 +8,9 @@ from dataclasses import dataclass
 from typing import Callable, Dict
 
 from . import (advance_decode, apply_penalties, argmax, argmax_no_alloc, cast,
-               decode_attention_fused, embed, gather_rows, gemm, gemm_emit, gemm_given, gemm_sum_norm, gemm_swiglu, norm_gemm, paged_attention,
-               poison_pages, qk_norm_rope_kv_write, randinit, rmsnorm, sample_topk, scale_cap, swiglu)
+               decode_attention_fused, embed, gather_rows, gemm, gemm_emit, gemm_given,
+               gemm_partials, gemm_sum_norm, gemm_swiglu, norm_gemm, paged_attention, poison_pages,
+               qk_norm_rope_kv_write, randinit, rmsnorm, sample_topk, scale_cap, swiglu)
 
 
 @dataclass(frozen=True)
@@ -35,6 +36,7 @@ KERNELS: Dict[str, KernelEntry] = {
     "poison_pages": KernelEntry(poison_pages, "elementwise",
                                 "tests/test_kernels_gpu.py:test_cast_and_poison_pages"),
     "gemm": KernelEntry(gemm, "gemm", "tests/kernel_refs.py:gemm"),
+    "gemm_partials": KernelEntry(gemm_partials, "gemm", "tests/kernel_refs.py:gemm"),
     "gemm_swiglu": KernelEntry(gemm_swiglu, "gemm", "tests/kernel_refs.py:gemm_swiglu"),
     "norm_gemm": KernelEntry(norm_gemm, "gemm", "tests/kernel_refs.py:rmsnorm"),
     "gemm_emit": KernelEntry(gemm_emit, "gemm", "tests/kernel_refs.py:gemm"),

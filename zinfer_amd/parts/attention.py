@@ -76,15 +76,23 @@ class GqaAttention(Mixer):
         s = self.spec
         T = h.shape[0]
         act = self.ctx.act_dtype
-        qkv = step.scratch("qkv", (T, self.q_width + 2 * self.kv_width), act)
-        self.qkv.forward(h, qkv)
         tables = self.position.rotation_tables()
         kv = step.kv_tables(cache.group)
         eps = float(s.qk_norm_eps) if s.qk_norm_eps is not None else 0.0
         attn = step.scratch("attn", (T, self.q_width), act)
         window = 0 if s.window is None else int(s.window)
         plain_position = tables is not None or not self.position.custom_apply
-        if plain_position and step.max_q_len == 1 and cache.writes \
+        # 17 to 128 tokens: the product runs split along K, and the kernel that norms, rotates
+        # and stores takes its partials as they are (one launch less, the same bits)
+        partials = self.qkv.forward_partials(h) \
+            if plain_position and cache.writes and act == torch.bfloat16 \
+            and cache.k_pool.dtype == torch.bfloat16 and s.head_dim % 8 == 0 else None
+        if partials is not None:
+            qkv = partials
+        else:
+            qkv = step.scratch("qkv", (T, self.q_width + 2 * self.kv_width), act)
+            self.qkv.forward(h, qkv)
+        if partials is None and plain_position and step.max_q_len == 1 and cache.writes \
                 and step.n_seqs <= ops.FUSED_DECODE_MAX_SEQS and ops.mfma_attention_covers(
                     act, s.n_heads, s.n_kv_heads, s.head_dim, cache.page_size):
             # a decode step: the attention kernel norms and rotates q and k and stores the

@@ -56,6 +56,21 @@ class Linear:
         return out
 
 
+    def forward_partials(self, x):
+        """The float32 partials [ksplit, T, out] of x W^T where the product is one that runs
+        split along K and would need a kernel of its own to add them (17 to 128 tokens), for
+        a caller whose next kernel can add them on its way; else None (then ``forward``)."""
+        M, K = x.shape
+        ks = ops.gemm_partials_plan(M, self.out_features, K, self.weight, self.tiled)
+        if ks is None:
+            return None
+        if hasattr(x, "materialize"):
+            x = x.materialize()
+        if x.dtype != torch.bfloat16:
+            return None
+        return ops.gemm_partials(x, self.weight, ks)
+
+
 def place_matrix(t: torch.Tensor, ctx) -> torch.Tensor:
     """A matrix on the device: bfloat16 stays bfloat16 under a bfloat16 build, a tensor
     stored in 32-bit stays so; a float32 build widens everything."""
