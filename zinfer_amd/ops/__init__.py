@@ -398,9 +398,9 @@ def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = Fals
     memory (10: 128 x 256 tiles, two workgroups to a CU, when they fill the chip; else 128 x
     128 tiles, 16: with the waves side by side and k-tiles of 128, for a long K or when one
     round of the chip holds the tiles (weights from HBM, 512 tokens: qkv of the 8B shape 43 ->
-    38 us), 6: with 2 x 2 waves); otherwise the kernels that stage both operands through LDS (4: 256 x 256
-    when they still fill the chip, else 0: 128 x 128).  Measured on MI355X at the Qwen3-8B and
-    Qwen3-14B sizes."""
+    38 us), 6: with 2 x 2 waves); otherwise the kernels that stage both operands through LDS
+    (4: 256 x 256 when they still fill the chip, else 0: 128 x 128).  Measured on MI355X at the
+    Qwen3-8B and Qwen3-14B sizes."""
     if w_tiled:
         tiles_m = (M + 127) // 128
         tiles = tiles_m * ((N + 255) // 256)
