@@ -25,14 +25,19 @@ LENGTHS = {"A": (5, 17, 40, 70), "B": (1, 9, 33, 64, 130), "C": (3, 48, 65, 100)
 _plain_cache = {}
 
 
-def _setup(name, dtype, tmp_path_factory):
+def _setup(name, dtype, tmp_path_factory, twice=False):
+    """``twice``: every length a second time with other tokens, so that with four requests
+    live the later ones must take pages that the earlier ones gave back."""
     store = torch.float32 if dtype == "float32" else torch.bfloat16
     root = tmp_path_factory.getbasetemp()
     path = tiny.model_dir_of(name, str(root), store)
     cfg = tiny.CONFIGS[name]
     requests = {f"r{i}": tiny.random_tokens(n, cfg["vocab_size"], 100 + i)
                 for i, n in enumerate(LENGTHS[name])}
-    key = (name, dtype)
+    if twice:
+        requests.update({f"s{i}": tiny.random_tokens(n, cfg["vocab_size"], 200 + i)
+                         for i, n in enumerate(reversed(LENGTHS[name]))})
+    key = (name, dtype, twice)
     if key not in _plain_cache:
         w = tiny.weights_of(name, store)
         _plain_cache[key] = {rid: plain.model_forward_batched(cfg, w, toks).numpy()
@@ -51,6 +56,9 @@ def _replay(path, dtype, steps, page_size, max_tokens=None, poison=True):
                       poison_freed=poison)
     outputs = {}
     for st in steps:
+        for e in st["entries"]:
+            held = eng.length(e["id"]) if eng.has_request(e["id"]) else 0
+            assert e["start"] == held, f"step {st['step']}: {e['id']} holds {held}"
         entries = [StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]]
         logits = eng.step(entries, end=st["end"])
         if logits.shape[0]:
@@ -76,6 +84,22 @@ def _compare(steps, outputs, ref, vocab, tolerance):
     return worst
 
 
+def _pool_tokens(name, mode, steps):
+    """The pool of a mixed replay holds exactly the pages that are live at its fullest step
+    (requests rounded up to a page, not to 64 tokens): short requests then reuse pages too."""
+    return traces.peak_tokens(steps, tiny.PAGE_SIZE[name]) if mode == "mixed" else None
+
+
+def _assert_pages_were_used_again(eng, steps):
+    """The pool was made for the most tokens live at a time; the trace as a whole needs more
+    pages than it has, so later requests ran in pages that earlier ones gave back."""
+    assert max(len(st["entries"]) for st in steps) == 4, "four requests live at a time"
+    for grp in eng.cache.groups:
+        assert grp.pages.handed_out > grp.pages.num_pages, \
+            (f"{grp.pages.handed_out} pages handed out of a pool of {grp.pages.num_pages}: "
+             "no page was used again")
+
+
 MODES = {"whole": traces.whole, "prefill_then_32": traces.prefill_then_single,
          "portions": traces.changing_portions, "mixed": traces.mixed,
          "token_by_token": traces.token_by_token}
@@ -85,11 +109,13 @@ MODES = {"whole": traces.whole, "prefill_then_32": traces.prefill_then_single,
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_replay_modes(name, dtype, mode, tmp_path_factory):
-    path, cfg, requests, ref = _setup(name, dtype, tmp_path_factory)
+    path, cfg, requests, ref = _setup(name, dtype, tmp_path_factory, twice=mode == "mixed")
     steps = MODES[mode](requests)
-    outputs, eng = _replay(path, dtype, steps, tiny.PAGE_SIZE[name])
+    outputs, eng = _replay(path, dtype, steps, tiny.PAGE_SIZE[name], _pool_tokens(name, mode, steps))
     tolerance = LOGITS_TOL_F32 if dtype == "float32" else LOGITS_TOL_BF16
     worst = _compare(steps, outputs, ref, cfg["vocab_size"], tolerance)
+    if mode == "mixed":
+        _assert_pages_were_used_again(eng, steps)
     print(f"{name} {dtype} {mode}: worst error {worst:.3g}")
 
 
@@ -99,10 +125,13 @@ def test_serving_widths(mode, tmp_path_factory):
     (one kernel choice each: weight streaming, 17 to 128 tokens, tiled, with their splits along
     K), mixed batches, and decoding, against the plain implementation."""
     name = "W"
-    path, cfg, requests, ref = _setup(name, "bfloat16", tmp_path_factory)
+    path, cfg, requests, ref = _setup(name, "bfloat16", tmp_path_factory, twice=mode == "mixed")
     steps = MODES[mode](requests)
-    outputs, eng = _replay(path, "bfloat16", steps, tiny.PAGE_SIZE[name])
+    outputs, eng = _replay(path, "bfloat16", steps, tiny.PAGE_SIZE[name],
+                           _pool_tokens(name, mode, steps))
     worst = _compare(steps, outputs, ref, cfg["vocab_size"], LOGITS_TOL_BF16)
+    if mode == "mixed":
+        _assert_pages_were_used_again(eng, steps)
     print(f"{name} bfloat16 {mode}: worst error {worst:.3g}")
 
 
@@ -450,3 +479,86 @@ def test_decode_steps_in_a_row_equal_single_steps(dtype, tmp_path_factory):
         a.decode_steps([StepEntry(r, [1], [0]) for r in reqs], too_many)
     assert a.cache.num_free_pages() == free
     a.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_behind_two_thousand_tokens(dtype, tmp_path_factory):
+    """The benchmark's regime at narrow widths: a prompt of 2100 tokens in one step, then 40
+    tokens one by one (captured graphs; 9 splits of 256 keys and their merge), every logits row
+    against the plain implementation; then the same 40 tokens drawn on the device, several
+    steps in a row without the host, against the engine's own single steps."""
+    from zinfer_amd.engine import StepEntry
+    from zinfer_amd.engine.replay import make_engine
+    name = "L"
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    path = tiny.model_dir_of(name, str(tmp_path_factory.getbasetemp()), store)
+    cfg = tiny.CONFIGS[name]
+    V = cfg["vocab_size"]
+    toks = tiny.random_tokens(2140, V, 41)
+    ref = plain.model_forward_batched(cfg, tiny.weights_of(name, store), toks).numpy()
+    tolerance = LOGITS_TOL_F32 if dtype == "float32" else LOGITS_TOL_BF16
+    scale = np.abs(ref).max()
+    eng = make_engine(path, dtype, 2304 * 2, DEV, poison_freed=True)
+    lg = eng.step([StepEntry("long", toks[:2100], [2099])]).cpu().numpy()
+    assert np.abs(lg[0] - ref[2099]).max() <= tolerance * scale, "the prompt's last position"
+    for p in range(2100, 2140):
+        lg = eng.step([StepEntry("long", toks[p:p + 1], [0])]).cpu().numpy()
+        err = np.abs(lg[0].astype(np.float64) - ref[p]).max() / scale
+        assert np.isfinite(lg).all() and err <= tolerance, f"position {p}: error {err:.3g}"
+    assert eng.graph_replays >= 30
+    # greedy decoding from position 2100 on: single steps and steps in a row give the same tokens
+    eng.release("long")
+    singles, rows = [], []
+    for rid, many in (("one", False), ("many", True)):
+        lg = eng.step([StepEntry(rid, toks[:2100], [2099])])
+        cur = eng.argmax(lg)
+        out = []
+        while len(out) < 40:
+            if many:
+                drawn = eng.decode_steps([StepEntry(rid, cur, [0])], 8)
+                out += [d[0] for d in drawn]
+                cur = drawn[-1]
+            else:
+                cur = eng.argmax(eng.step([StepEntry(rid, cur, [0])]))
+                out.append(cur[0])
+        (rows if many else singles).extend(out)
+    assert singles == rows
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("name,dtype", [("E", "bfloat16"), ("L", "bfloat16"), ("B", "float32")])
+def test_a_decode_step_of_130_sequences(name, dtype, tmp_path_factory):
+    """More sequences in a decode-only step than the weight-streaming and the 17-to-128-token
+    products take (the tiled products then serve a step of single tokens, and the decode
+    attention's grid is 130 deep): three such steps against the plain implementation."""
+    from zinfer_amd.engine import StepEntry
+    from zinfer_amd.engine.replay import make_engine
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    path = tiny.model_dir_of(name, str(tmp_path_factory.getbasetemp()), store)
+    cfg = tiny.CONFIGS[name]
+    V = cfg["vocab_size"]
+    n = 130
+    reqs = {f"w{i}": tiny.random_tokens(4 + (i * 7) % 45, V, 3000 + i) for i in range(n)}
+    w = tiny.weights_of(name, store)
+    ps = tiny.PAGE_SIZE[name]
+    pages = sum((len(t) + ps - 1) // ps for t in reqs.values())
+    eng = make_engine(path, dtype, 0, DEVICE[0], page_size=ps, num_pages=pages, max_requests=n,
+                      poison_freed=True)
+    # the prompts but their last three tokens, 26 requests a step
+    ids = list(reqs)
+    for lo in range(0, n, 26):
+        eng.step([StepEntry(r, reqs[r][:-3], []) for r in ids[lo:lo + 26]])
+    got = {r: [] for r in ids}
+    for k in (3, 2, 1):
+        lg = eng.step([StepEntry(r, reqs[r][len(reqs[r]) - k:len(reqs[r]) - k + 1], [0])
+                       for r in ids]).cpu().numpy().copy()
+        assert lg.shape == (n, V) and np.isfinite(lg).all()
+        for i, r in enumerate(ids):
+            got[r].append(lg[i])
+    assert eng.cache.num_free_pages() == [0] and eng.cache.num_free_slots() == 0
+    tolerance = LOGITS_TOL_F32 if dtype == "float32" else LOGITS_TOL_BF16
+    for r in ids:
+        ref = plain.model_forward_batched(cfg, w, reqs[r]).numpy()[-3:]
+        err = np.abs(np.stack(got[r]).astype(np.float64) - ref).max() / np.abs(ref).max()
+        assert err <= tolerance, f"{r} ({len(reqs[r])} tokens): error {err:.3g}"
+    eng.cache.check()

@@ -20,14 +20,21 @@ def _emulated_kernels(monkeypatch):
 @pytest.mark.parametrize("mode", list(G.MODES))
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_replay_modes_host_logic(name, mode, tmp_path_factory):
-    path, cfg, requests, ref = G._setup(name, "float32", tmp_path_factory)
+    path, cfg, requests, ref = G._setup(name, "float32", tmp_path_factory, twice=mode == "mixed")
     steps = G.MODES[mode](requests)
-    outputs, eng = G._replay(path, "float32", steps, tiny.PAGE_SIZE[name])
+    outputs, eng = G._replay(path, "float32", steps, tiny.PAGE_SIZE[name],
+                             G._pool_tokens(name, mode, steps))
     G._compare(steps, outputs, ref, cfg["vocab_size"], 1e-5)
+    if mode == "mixed":
+        G._assert_pages_were_used_again(eng, steps)
 
 
 def test_mixed_reuse_host_logic(tmp_path_factory):
     G.test_mixed_many_requests_reuse_pages("float32", tmp_path_factory)
+
+
+def test_130_sequences_host_logic(tmp_path_factory):
+    G.test_a_decode_step_of_130_sequences("B", "float32", tmp_path_factory)
 
 
 def test_step_errors_host_logic(tmp_path_factory):

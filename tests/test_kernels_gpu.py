@@ -737,7 +737,8 @@ def _fused_against_two_kernels(ops, nH, nKV, hd, page_size, window, use_norm, us
     qkv = _rand((n, (nH + 2 * nKV) * hd), dtype, 22).to(DEV)
     qg = (1 + 0.1 * _rand((hd,), torch.float32, 23)).to(DEV) if use_norm else None
     kg = (1 + 0.1 * _rand((hd,), torch.float32, 24)).to(DEV) if use_norm else None
-    cos, sin = (t.to(DEV) for t in rotary_tables(hd, 10000.0, 1100)) if use_rope else (None, None)
+    cos, sin = (t.to(DEV) for t in rotary_tables(hd, 10000.0, max(1100, max(ctx_lens) + 8))) \
+        if use_rope else (None, None)
     positions = torch.tensor([c - 1 + 5 for c in ctx_lens], dtype=torch.int32, device=DEV)
     slot_mapping = torch.tensor(slots, dtype=torch.int32, device=DEV)
     d = {k: s[k].to(DEV) for k in ("block_table", "q_start", "ctx_len", "seq_index")}
@@ -1119,3 +1120,127 @@ def test_prefill_attention_splits_keys_over_workgroups(nH, nKV, hd, window, vari
             v_row = s["Vs"][0][target, (nH - 1) // (nH // nKV)].float()
             assert torch.allclose(got.cpu().float()[row, (nH - 1) * hd:nH * hd], v_row, atol=3e-2), target
             assert rel_err(got, want) <= 2 * tol(dtype)
+
+
+# ---------------------------------------------------------------- the served decode regime
+# Contexts of thousands of keys at the served head shapes: more than 8 splits of 256 keys (where
+# a lane of the merge kernel takes a second, third, ... load) and more than 64 (where it goes
+# round its loop again), which the short contexts above never reach.
+SERVED_HEADS = [(32, 8, 128, 16), (40, 8, 128, 16), (64, 8, 128, 16)]
+LONG_CONTEXTS = [2048, 2049, 2304, 4097, 8192, 32768]
+
+
+def _long_pools(nKV, hd, ps, ctx_lens, seed):
+    """Pools made on the device (rows [page, kv head, row, hd], values [page, kv head, hd,
+    row]) with pages dealt in a shuffled order and NaN in every row beyond a context."""
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    pages_per = [(c + ps - 1) // ps for c in ctx_lens]
+    num_pages = sum(pages_per) + 5
+    perm = torch.randperm(num_pages, generator=g, device=DEV)
+    k = torch.randn((num_pages, nKV, ps, hd), generator=g, device=DEV).to(torch.bfloat16)
+    v = torch.randn((num_pages, nKV, hd, ps), generator=g, device=DEV).to(torch.bfloat16)
+    bt = torch.full((len(ctx_lens), max(pages_per)), -1, dtype=torch.int32, device=DEV)
+    held = torch.zeros((num_pages,), dtype=torch.bool, device=DEV)
+    cur = 0
+    for i, (c, n) in enumerate(zip(ctx_lens, pages_per)):
+        pages = perm[cur:cur + n]
+        cur += n
+        bt[i, :n] = pages.int()
+        held[pages] = True
+        if c % ps:
+            k[pages[-1], :, c % ps:] = float("nan")
+            v[pages[-1], :, :, c % ps:] = float("nan")
+    k[~held] = float("nan")
+    v[~held] = float("nan")
+    return k, v, bt
+
+
+def _long_reference(q, k, v, bt, ctx_lens, nH, nKV, hd, ps, scale):
+    """softmax(q K^T scale) V of every sequence's one query over its whole context, in 64-bit."""
+    G = nH // nKV
+    out = torch.empty((len(ctx_lens), nH * hd), dtype=torch.float64, device=DEV)
+    for i, c in enumerate(ctx_lens):
+        pages = bt[i, :(c + ps - 1) // ps].long()
+        K = k[pages].permute(1, 0, 2, 3).reshape(nKV, -1, hd)[:, :c].double()
+        V = v[pages].permute(1, 0, 3, 2).reshape(nKV, -1, hd)[:, :c].double()
+        qi = q[i].view(nKV, G, hd).double()
+        a = torch.softmax(torch.einsum("kgd,knd->kgn", qi, K) * scale, dim=-1)
+        out[i] = torch.einsum("kgn,knd->kgd", a, V).reshape(-1)
+    return out
+
+
+def _long_decode(nH, nKV, hd, ps, ctx_lens, seed, stand_out=()):
+    """The decode attention kernels (splits + merge) against the 64-bit reference.
+    ``stand_out``: (sequence, position, query head) triples whose key is aligned with the query
+    and scaled up; returns output and reference."""
+    ops = _ops()
+    n = len(ctx_lens)
+    k, v, bt = _long_pools(nKV, hd, ps, ctx_lens, seed)
+    g = torch.Generator(device=DEV).manual_seed(seed + 1)
+    q = torch.randn((n, nH * hd), generator=g, device=DEV).to(torch.bfloat16)
+    G = nH // nKV
+    for i, pos, head in stand_out:
+        qv = q[i].view(nH, hd)[head].float()
+        k[bt[i, pos // ps].long(), head // G, pos % ps] = (qv / qv.norm() * 400.0).to(torch.bfloat16)
+    scale = 1.0 / math.sqrt(hd)
+    want = _long_reference(q, k, v, bt, ctx_lens, nH, nKV, hd, ps, scale)
+    num_pages = k.shape[0]
+    kt = ref.tile_k_pool(k.view(num_pages, -1), nKV, ps, hd)
+    vt = ref.tile_v_pool(v.view(num_pages, -1), nKV, ps, hd)
+    got = torch.full((n, nH * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    q_start = torch.arange(n + 1, dtype=torch.int32, device=DEV)
+    ctx = torch.tensor(ctx_lens, dtype=torch.int32, device=DEV)
+    ops.paged_attention(q, kt, vt, bt, q_start, ctx, q_start[:n].contiguous(), got, scale, 0, nH,
+                        nKV, hd, ps, 1, max(ctx_lens), n_single=n)
+    torch.cuda.synchronize()
+    return got, want, v, bt
+
+
+@pytest.mark.parametrize("nH,nKV,hd,ps", SERVED_HEADS)
+@pytest.mark.parametrize("batch", [1, 8, 64])
+def test_decode_attention_at_served_contexts(nH, nKV, hd, ps, batch):
+    """One token per sequence over 2048 to 32768 keys (9 to 128 splits): contexts that end at
+    a split's edge, one key beyond it, and deep in the merge kernel's second round."""
+    if batch == 1:
+        cases = [[c] for c in LONG_CONTEXTS]
+    elif batch == 8:
+        cases = [LONG_CONTEXTS + [1, 300], [16385, 16384, 20000, 257, 2047, 2050, 16640, 5]]
+    else:
+        cases = [[LONG_CONTEXTS[i % 5] + 7 * i for i in range(60)] + [32768, 16385, 1, 256]]
+    for ctx_lens in cases:
+        got, want, _, _ = _long_decode(nH, nKV, hd, ps, ctx_lens, seed=5 + len(ctx_lens))
+        assert not torch.isnan(got.float()).any(), f"contexts {ctx_lens[:8]}: NaN was read"
+        err = (got.double() - want).abs().amax(dim=1) / want.abs().amax(dim=1)
+        bad = torch.nonzero(err > 2 * tol(torch.bfloat16)).flatten().tolist()
+        assert not bad, f"sequences {bad} of contexts {ctx_lens}: error {err[bad[0]]:.3g}"
+
+
+@pytest.mark.parametrize("nH,nKV,hd,ps", SERVED_HEADS)
+def test_decode_attention_far_key_in_late_splits(nH, nKV, hd, ps):
+    """A key that takes all the weight at the first and at the last key of splits 8, 9 and 127
+    (the ninth and tenth partial of a lane's first round of loads, the last of its second):
+    the output is that position's value row."""
+    G = nH // nKV
+    for pos in (8 * 256, 9 * 256 - 1, 9 * 256, 10 * 256 - 1, 127 * 256, 128 * 256 - 1):
+        ctx_lens = [32768, max(pos + 1, 2305)]
+        head = (pos // 256 * 5) % nH
+        got, want, v, bt = _long_decode(nH, nKV, hd, ps, ctx_lens, seed=pos,
+                                        stand_out=[(0, pos, head), (1, pos, head)])
+        for i in (0, 1):
+            row = v[bt[i, pos // ps].long(), head // G, :, pos % ps].float()
+            mine = got[i].view(nH, hd)[head].float()
+            assert torch.allclose(mine, row, atol=3e-2), f"key {pos}, context {ctx_lens[i]}"
+        err = (got.double() - want).abs().max() / want.abs().max()
+        assert err <= 2 * tol(torch.bfloat16), f"key {pos}: error {err:.3g}"
+
+
+@pytest.mark.parametrize("nH,nKV,hd,ps", SERVED_HEADS)
+def test_decode_attention_fused_at_served_contexts(nH, nKV, hd, ps):
+    """The fused decode attention (steps of up to 32 sequences) against the two kernels it
+    replaces, bit for bit in output and pools, at 2048 to 32768 keys; alone (batch 1) and
+    eight together."""
+    ops = _ops()
+    _fused_against_two_kernels(ops, nH, nKV, hd, ps, 0, True, True,
+                               [2048, 2049, 2304, 4097, 8192, 32768, 16385, 300])
+    for c in (2049, 32768):
+        _fused_against_two_kernels(ops, nH, nKV, hd, ps, 0, True, True, [c])

@@ -19,9 +19,9 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 TOL = {"float32": 2e-5, "bfloat16": 2e-2}        # as in test_engine_gpu.py
 
 
-def run_trace(model_dir, dtype, steps, out_dir, max_tokens):
+def run_trace(model_dir, dtype, steps, out_dir, max_tokens, extra=()):
     cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir,
-           "--dtype", dtype, "--out", out_dir, "--max-tokens", str(max_tokens)]
+           "--dtype", dtype, "--out", out_dir, "--max-tokens", str(max_tokens)] + list(extra)
     p = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
     try:
         for st in steps:
@@ -59,7 +59,9 @@ def test_every_cutting_through_trace_run(name, dtype, tmp_path):
             st["step"] = len(steps)
             steps.append(st)
     peak = traces.peak_tokens(steps, 64)
-    outs = run_trace(model_dir, dtype, steps, str(tmp_path / "out"), peak)
+    # the configuration's own page size goes through the program's option (B: pages of 8)
+    outs = run_trace(model_dir, dtype, steps, str(tmp_path / "out"), peak,
+                     ["--page-size", str(tiny.PAGE_SIZE[name])])
     got = traces.collect(steps, outs, V)
     assert len(got) == 4 * len(requests)
     for rid_k, rows in got.items():
@@ -70,6 +72,55 @@ def test_every_cutting_through_trace_run(name, dtype, tmp_path):
     # the pool was made for `peak` tokens: pages were used again
     total = sum((len(t) + 63) // 64 * 64 for t in requests.values()) * 4
     assert peak < total
+
+
+def test_pool_and_slots_from_options(tmp_path):
+    """--num-pages and --max-requests size the pool and the slots themselves: a trace that
+    fits runs, one page or one slot fewer is CacheFull."""
+    model_dir = tiny.model_dir_of("B", str(tmp_path), torch.float32)
+    cfg = tiny.CONFIGS["B"]
+    V = cfg["vocab_size"]
+    reqs = {f"n{i}": tiny.random_tokens(n, V, 40 + i) for i, n in enumerate((20, 9, 17))}
+    w = tiny.weights_of("B", torch.float32)
+    steps = [{"step": 0, "entries": [{"id": r, "tokens": t, "want": [len(t) - 1], "start": 0}
+                                     for r, t in reqs.items()], "end": list(reqs)}]
+    pages = sum((len(t) + 3) // 4 for t in reqs.values())       # pages of 4 tokens
+    base = ["--page-size", "4"]
+    outs = run_trace(model_dir, "float32", steps, str(tmp_path / "o1"), 64,
+                     base + ["--num-pages", str(pages), "--max-requests", "3"])
+    got = outs[0].reshape(3, V)
+    for i, (r, t) in enumerate(reqs.items()):
+        ref = plain.model_forward_batched(cfg, w, t).numpy()[-1]
+        assert np.abs(got[i] - ref).max() <= TOL["float32"] * np.abs(ref).max()
+    for extra in (["--num-pages", str(pages - 1), "--max-requests", "3"],
+                  ["--num-pages", str(pages), "--max-requests", "2"]):
+        cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir,
+               "--dtype", "float32", "--out", str(tmp_path / "o2"), "--max-tokens", "64"] \
+            + base + extra
+        r = subprocess.run(cmd, input=json.dumps(steps[0]) + "\n", capture_output=True,
+                           text=True, timeout=300)
+        assert r.returncode == 1 and "CacheFull" in r.stderr and "done" not in r.stdout, extra
+
+
+def test_a_position_gap_is_an_error(tmp_path):
+    """An entry that says where it starts must start where the request's tokens end."""
+    model_dir = tiny.model_dir_of("A", str(tmp_path), torch.float32)
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir,
+           "--dtype", "float32", "--out", str(tmp_path / "o"), "--max-tokens", "128"]
+    first = {"step": 0, "entries": [{"id": "a", "tokens": [1, 2, 3], "want": [], "start": 0}],
+             "end": []}
+    for start, words in ((5, "tokens 3..4 were never given"), (2, "tokens 2..2 are held already")):
+        second = {"step": 1, "entries": [{"id": "a", "tokens": [4, 5], "want": [1],
+                                          "start": start}], "end": []}
+        r = subprocess.run(cmd, input=json.dumps(first) + "\n" + json.dumps(second) + "\n",
+                           capture_output=True, text=True, timeout=300)
+        assert r.returncode == 1 and "done 0" in r.stdout and "done 1" not in r.stdout
+        assert "PositionGap" in r.stderr and "'a'" in r.stderr and words in r.stderr, r.stderr
+    # a new request must start at 0
+    r = subprocess.run(cmd, input=json.dumps({"step": 0, "entries": [
+        {"id": "z", "tokens": [1], "want": [0], "start": 7}], "end": []}) + "\n",
+        capture_output=True, text=True, timeout=300)
+    assert r.returncode == 1 and "PositionGap" in r.stderr
 
 
 def test_errors_are_reported_not_papered_over(tmp_path):

@@ -53,9 +53,18 @@ WIDE = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_l
             intermediate_size=12288, vocab_size=8200, rope_theta=1000000.0, rms_norm_eps=1e-6,
             tie_word_embeddings=False, max_position_embeddings=1024, torch_dtype="bfloat16")
 
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "W": WIDE}
-PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 16, "W": 16}
-SEEDS = {"A": 11, "B": 22, "C": 33, "D": 44, "E": 55, "W": 66}
+# the served model's heads (4 query heads to a kv head, head size 128) under narrow widths and
+# a position table of 4096: contexts of thousands of keys, where the decode attention runs
+# more than 8 splits and the merge of their partials takes more than one load a lane
+LONG = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2,
+            hidden_size=256, num_attention_heads=8, num_key_value_heads=2, head_dim=128,
+            intermediate_size=768, vocab_size=1536, rope_theta=1000000.0, rms_norm_eps=1e-6,
+            tie_word_embeddings=False, max_position_embeddings=4096, torch_dtype="bfloat16")
+
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "W": WIDE,
+           "L": LONG}
+PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 16, "W": 16, "L": 16}
+SEEDS = {"A": 11, "B": 22, "C": 33, "D": 44, "E": 55, "W": 66, "L": 77}
 
 
 def config_of(name: str) -> Qwen3Config:

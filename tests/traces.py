@@ -9,7 +9,9 @@ from typing import Dict, List, Sequence
 
 
 def _entry(rid, tokens, lo, hi):
-    return {"id": rid, "tokens": list(tokens[lo:hi]), "want": list(range(hi - lo))}
+    # "start" is optional for the replay program; the traces give it, so that every replay
+    # also checks that the engine holds exactly the tokens the trace thinks it holds
+    return {"id": rid, "tokens": list(tokens[lo:hi]), "want": list(range(hi - lo)), "start": lo}
 
 
 def whole(requests: Dict[str, Sequence[int]]) -> List[dict]:
