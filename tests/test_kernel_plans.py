@@ -105,10 +105,32 @@ def test_weight_streaming_plans():
                 assert rg in (1, 2, 4) and 1 <= ks <= 16
 
 
-def test_the_flat_kernel_table_is_complete_and_its_references_exist():
+# which plain function (or, for kernels that are compared with other kernels or through the
+# engine, which test) each kernel of the table is checked against
+TESTED_AGAINST = {
+    "embed": "kernel_refs.py:embed", "rmsnorm": "kernel_refs.py:rmsnorm",
+    "qk_norm_rope_kv_write": "kernel_refs.py:qk_norm_rope_kv_write",
+    "swiglu": "kernel_refs.py:swiglu", "gather_rows": "kernel_refs.py:gather_rows",
+    "argmax": "kernel_refs.py:argmax", "argmax_no_alloc": "kernel_refs.py:argmax",
+    "scale_cap": "kernel_refs.py:scale_cap",
+    "advance_decode": "test_engine_gpu.py:test_decode_steps_in_a_row_equal_single_steps",
+    "cast": "test_kernels_gpu.py:test_cast_and_poison_pages",
+    "poison_pages": "test_kernels_gpu.py:test_cast_and_poison_pages",
+    "gemm": "kernel_refs.py:gemm", "gemm_partials": "kernel_refs.py:gemm",
+    "gemm_swiglu": "kernel_refs.py:gemm_swiglu", "norm_gemm": "kernel_refs.py:rmsnorm",
+    "gemm_emit": "kernel_refs.py:gemm", "gemm_given": "kernel_refs.py:rmsnorm",
+    "gemm_sum_norm": "kernel_refs.py:rmsnorm", "paged_attention": "kernel_refs.py:paged_attention",
+    "decode_attention_fused":
+        "test_kernels_gpu.py:test_decode_attention_fused_equals_the_two_kernels",
+    "apply_penalties": "plain.py:adjusted_logit", "sample_topk": "plain.py:sample_token",
+    "randinit": "test_kernels_gpu.py:test_randinit_is_the_numpy_draw_bit_for_bit",
+}
+
+
+def test_the_flat_kernel_table_is_complete_and_every_kernel_has_a_reference():
     """Every function of `zinfer_amd.ops` that launches a kernel is in the table once, its
-    module is one the build knows, and the reference it names exists."""
-    import importlib
+    module is one the build knows, it cites the reference's formula or says that it has
+    none, and the plain function or test it is checked against exists."""
     import inspect
     import os
     import re
@@ -116,16 +138,19 @@ def test_the_flat_kernel_table_is_complete_and_its_references_exist():
     launchers = {name for name, fn in vars(ops).items()
                  if inspect.isfunction(fn) and fn.__module__ == "zinfer_amd.ops"
                  and not name.startswith("_") and "build.load(" in inspect.getsource(fn)}
-    assert launchers == set(table.KERNELS), launchers ^ set(table.KERNELS)
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    assert launchers == set(table.KERNELS) == set(TESTED_AGAINST), \
+        launchers ^ set(table.KERNELS) ^ set(TESTED_AGAINST)
+    here = os.path.dirname(os.path.abspath(__file__))
     for name, entry in table.KERNELS.items():
         assert entry.launch is getattr(ops, name)
         assert entry.module in build.MODULES
-        path, fn = entry.reference.split(":")
-        with open(os.path.join(root, path)) as f:
-            assert re.search(rf"^def {fn}\(", f.read(), re.M), entry.reference
+        assert entry.formula.startswith(("src/", "own: ")), name
+        path, fn = TESTED_AGAINST[name].split(":")
+        with open(os.path.join(here, path)) as f:
+            assert re.search(rf"^def {fn}\(", f.read(), re.M), TESTED_AGAINST[name]
         source = inspect.getsource(entry.launch)
         assert f'build.load("{entry.module}")' in source, name
+        assert "tests/" not in entry.formula
 
 
 def test_measured_plans_are_plans_the_kernels_take():

@@ -287,6 +287,36 @@ def test_gemm_256_token_tiles_are_chosen_and_agree():
         assert torch.equal(chosen, forced) and torch.equal(chosen, small)
 
 
+@pytest.mark.parametrize("variant", [20, 21, 22, 10, 16])
+@pytest.mark.parametrize("K", [4096, 12288])
+def test_gemm_tiled_kernels_at_a_served_k(variant, K):
+    """The tiled kernels at the K the engine runs them with (4096: 128 trips round the
+    256-token tiles' ring of four k-tiles of 32; 12288: the down product's), where the offsets
+    into both operands are largest: against the plain product and, bit for bit, the 128 x 128
+    tiles; 64-token tiles of 128 outputs likewise."""
+    ops = _ops()
+    M, N = 512, 1024
+    a = _rand((M, K), torch.bfloat16, 71)
+    w = _rand((N, K), torch.bfloat16, 72, 0.02)
+    wt = ops.pretile_weight(w.to(DEV))
+    want = torch.empty((M, N), dtype=torch.float32)
+    ref.gemm(a, w, want, False)
+    got = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+    ops.gemm(a.to(DEV), wt, got, w_tiled=True, tile_variant=variant)
+    assert rel_err(got, want) <= 2e-5
+    small = torch.empty_like(got)
+    ops.gemm(a.to(DEV), wt, small, w_tiled=True, tile_variant=6)
+    assert torch.equal(got, small)
+    if variant == 20:
+        # and the residual sum with its 32-bit accumulate epilogue
+        base = _rand((M, N), torch.float32, 73)
+        want = base.clone()
+        ref.gemm(a, w, want, True)
+        got = base.clone().to(DEV)
+        ops.gemm(a.to(DEV), wt, got, True, w_tiled=True, tile_variant=variant)
+        assert rel_err(got, want) <= 2e-5
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64, 65, 200, 300])
 @pytest.mark.parametrize("I,K,tiled", [(32, 64, True), (12288 // 8, 320, True), (96, 136, False),
                                        (352, 4096, True), (8192, 192, True)])

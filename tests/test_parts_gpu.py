@@ -37,6 +37,16 @@ class _StubModel:
     def cache_needs(self):
         return self._needs
 
+    parts = ()      # the parts under test: they are asked for hints and shown their caches
+
+    def hint_providers(self):
+        return [q for p in self.parts for q in p.hint_providers()]
+
+    def accept_caches(self, caches):
+        for p, c in zip(self.parts, caches):
+            if hasattr(p, "accept_cache"):
+                p.accept_cache(c)
+
 
 class _context:
     """Step context for {request: n_tokens}: pages are reserved on entry, lengths are
@@ -128,6 +138,7 @@ def test_attention_part(dtype, qk_norm, window, rope):
     stub = _StubModel([None], dtype)
     part = build_part("mixer", spec, stub.ctx, "a.")
     stub._needs = [part.cache_need()]
+    stub.parts = (part,)
     eng = Engine(stub, page_size=16, num_pages=8, max_requests=2, poison_freed=True)
     w = {"a.q_proj.weight": _rand((nH * hd, H), 1, 0.1, dtype),
          "a.k_proj.weight": _rand((nKV * hd, H), 2, 0.1, dtype),
@@ -683,3 +694,195 @@ def test_toy_norm_position_and_routed_feed_forward(tmp_path):
         unregister_part("norm", ToyLayerNormSpec)
         unregister_part("position", ToyLearnedPositionSpec)
         unregister_part("feed_forward", ToyRoutedSpec)
+
+
+# ----------------------------------------------------------------------------- a mixer with a cache and hints of its own
+# One shared key row and one value row per token, of different widths, kept in 64-bit whatever
+# the engine's cache dtype is; and a way of its own to cut a step (tiles of 5 queries), which
+# it asks the engine to pack with the step's metadata.  Nothing in the framework knows of it.
+@dataclass(frozen=True)
+class ToyLatentSpec:
+    hidden_size: int
+    key_dim: int
+    value_dim: int
+    tile: int
+
+
+def _register_toy_latent(seen):
+    from zinfer_amd.parts import KVNeed, Mixer, StepHints, TensorDecl, register_part
+
+    class ToyLatentMixer(Mixer):
+        def __init__(self, spec, ctx, prefix):
+            super().__init__(spec, ctx, prefix)
+            self.hint_key = ("toy_latent", spec.tile)
+
+        def declare(self):
+            s, p = self.spec, self.prefix
+            return {p + "q.weight": TensorDecl((s.key_dim, s.hidden_size)),
+                    p + "k.weight": TensorDecl((s.key_dim, s.hidden_size)),
+                    p + "v.weight": TensorDecl((s.value_dim, s.hidden_size)),
+                    p + "o.weight": TensorDecl((s.hidden_size, s.value_dim))}
+
+        def bind(self, tensors):
+            self.w = {n: tensors[self.prefix + n + ".weight"].double().to(self.ctx.device)
+                      for n in "qkvo"}
+
+        def cache_need(self):
+            s = self.spec
+            return KVNeed(1, s.key_dim, None, value_dim=s.value_dim, dtype=torch.float64)
+
+        def accept_cache(self, cache):
+            seen["accepted"] = (cache.k_pool.dtype, cache.k_pool.shape[1], cache.v_pool.shape[1])
+
+        def step_hints(self, shape):
+            t = self.spec.tile
+            tiles = [(i, j) for i, n in enumerate(shape.q_lens) for j in range((n + t - 1) // t)]
+            seen["asked"] = seen.get("asked", 0) + 1
+            return StepHints({"tiles": np.asarray(tiles, dtype=np.int32).reshape(-1, 2)},
+                             {"n_tiles": len(tiles), "longest": max(shape.ctx_lens)})
+
+        def forward(self, h, residual, step, cache):
+            s, ps = self.spec, cache.page_size
+            hints = step.hints[self.hint_key]
+            tiles = hints.arrays["tiles"]
+            assert tiles.device.type == torch.device(DEV).type and tiles.dtype == torch.int32
+            assert tiles.shape == (hints.numbers["n_tiles"], 2)
+            assert hints.numbers["longest"] == max(step.ctx_lens)
+            kv = step.kv_tables(cache.group)
+            q, k, v = (h.double() @ self.w[n].T for n in "qkv")
+            slots = kv.slot_mapping.long()
+            cache.k_pool.view(-1, s.key_dim)[slots] = k
+            cache.v_pool.view(-1, s.value_dim)[slots] = v
+            first = [0]
+            for n in step.q_lens:
+                first.append(first[-1] + n)
+            done = 0
+            for i, j in tiles.cpu().tolist():        # the step, tile by tile as the hints cut it
+                n, c = step.q_lens[i], step.ctx_lens[i]
+                pages = kv.block_table[i, :(c + ps - 1) // ps].long()
+                K = cache.k_pool[pages].view(-1, s.key_dim)
+                V = cache.v_pool[pages].view(-1, s.value_dim)
+                for t in range(j * s.tile, min((j + 1) * s.tile, n)):
+                    pos = c - n + t
+                    a = torch.softmax(K[:pos + 1] @ q[first[i] + t] / s.key_dim ** 0.5, dim=0)
+                    residual[first[i] + t] += ((a @ V[:pos + 1]) @ self.w["o"].T).float()
+                    done += 1
+            assert done == step.n_tokens
+
+    register_part("mixer", ToyLatentSpec, ToyLatentMixer)
+
+
+@dataclass(frozen=True)
+class ToyLatentConfig:
+    hidden_size: int
+    key_dim: int
+    value_dim: int
+    vocab_size: int
+    model_type: str = "toy_latent"
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(**{k: raw[k] for k in ("hidden_size", "key_dim", "value_dim", "vocab_size")})
+
+    def to_dict(self):
+        return dict(architectures=["ToyLatentForCausalLM"], model_type="toy_latent",
+                    hidden_size=self.hidden_size, key_dim=self.key_dim, value_dim=self.value_dim,
+                    vocab_size=self.vocab_size)
+
+    def model_spec(self):
+        from zinfer_amd.config.specs import (GqaAttentionSpec, ModelSpec, PreNormBlockSpec,
+                                             RmsNormSpec, RotaryHalfSplitSpec, ScheduleEntry,
+                                             SwiGluSpec)
+        H = self.hidden_size
+        norm = RmsNormSpec(H, 1e-5)
+        ff = SwiGluSpec(H, 2 * H)
+        full = GqaAttentionSpec(H, 4, 2, 16, 1e-5, RotaryHalfSplitSpec(16, 1e4, 256), None)
+        latent = ToyLatentSpec(H, self.key_dim, self.value_dim, 5)
+        blk = lambda m: PreNormBlockSpec(mixer=m, feed_forward=ff, mixer_norm=norm, ff_norm=norm)
+        return ModelSpec(vocab_size=self.vocab_size, hidden_size=H, max_positions=256,
+                         layers=(blk(latent), blk(full), blk(latent)),
+                         schedule=tuple(ScheduleEntry(i) for i in range(3)), final_norm=norm,
+                         tie_word_embeddings=True)
+
+
+def _toy_latent_plain(cfg: ToyLatentConfig, w, toks):
+    caches = [([], []) for _ in range(3)]
+    rows = []
+    for p, tok in enumerate(toks):
+        x = w["model.embed_tokens.weight"][tok].to(F64)
+        for layer in range(3):
+            pre = f"model.layers.{layer}."
+            n = plain.rms_norm(x, w[pre + "input_layernorm.weight"], 1e-5)
+            if layer == 1:
+                q = plain.per_head_rms_norm(plain.linear(n, w[pre + "self_attn.q_proj.weight"]),
+                                            4, 16, w[pre + "self_attn.q_norm.weight"], 1e-5)
+                k = plain.per_head_rms_norm(plain.linear(n, w[pre + "self_attn.k_proj.weight"]),
+                                            2, 16, w[pre + "self_attn.k_norm.weight"], 1e-5)
+                v = plain.linear(n, w[pre + "self_attn.v_proj.weight"])
+                q, k = plain.rope_heads(q, 4, 16, p, 1e4), plain.rope_heads(k, 2, 16, p, 1e4)
+                caches[layer][0].append(k.reshape(2, 16)); caches[layer][1].append(v.reshape(2, 16))
+                o = plain.attention_single_query(q, torch.stack(caches[layer][0]),
+                                                 torch.stack(caches[layer][1]), 4, 2, 16, None)
+                x = x + plain.linear(o, w[pre + "self_attn.o_proj.weight"])
+            else:
+                q, k, v = (plain.linear(n, w[pre + f"self_attn.{m}.weight"]) for m in "qkv")
+                caches[layer][0].append(k); caches[layer][1].append(v)
+                a = plain.softmax(torch.stack(caches[layer][0]) @ q / cfg.key_dim ** 0.5)
+                x = x + plain.linear(a @ torch.stack(caches[layer][1]), w[pre + "self_attn.o.weight"])
+            mm = plain.rms_norm(x, w[pre + "post_attention_layernorm.weight"], 1e-5)
+            x = x + plain.linear(plain.swiglu(plain.linear(mm, w[pre + "mlp.gate_proj.weight"]),
+                                              plain.linear(mm, w[pre + "mlp.up_proj.weight"])),
+                                 w[pre + "mlp.down_proj.weight"])
+        rows.append(plain.linear(plain.rms_norm(x, w["model.norm.weight"], 1e-5),
+                                 w["model.embed_tokens.weight"]))
+    return torch.stack(rows).numpy()
+
+
+def test_toy_mixer_with_cache_widths_dtype_and_step_hints_of_its_own(tmp_path):
+    """A mixer defined here keeps keys 24 wide and values 40 wide in 64-bit pools under a
+    32-bit engine, beside an ordinary attention layer with pools of its own, and has the
+    engine pack its own way of cutting a step (tiles of 5 queries) into the step's upload:
+    built from a folder and stepped under every cutting without a change to the framework."""
+    from zinfer_amd.config import register_architecture, unregister_architecture
+    from zinfer_amd.engine import StepEntry
+    from zinfer_amd.engine.replay import make_engine
+    from zinfer_amd.parts import unregister_part
+    from zinfer_amd.weights import SafetensorsFile, write_model_dir
+    seen = {}
+    _register_toy_latent(seen)
+    register_architecture("ToyLatentForCausalLM", ToyLatentConfig, model_type="toy_latent")
+    try:
+        cfg = ToyLatentConfig(hidden_size=64, key_dim=24, value_dim=40, vocab_size=190)
+        path = write_model_dir(str(tmp_path / "toy_latent"), cfg, seed=13, dtype=torch.float32)
+        with SafetensorsFile(os.path.join(path, "model.safetensors")) as f:
+            w = {n: f.tensor(n) for n in f.names()}
+        requests = {f"l{i}": tiny.random_tokens(n, 190, 60 + i) for i, n in enumerate((37, 4, 66, 21))}
+        ref = {rid: _toy_latent_plain(cfg, w, t) for rid, t in requests.items()}
+        for mode in ("whole", "portions", "mixed", "prefill_then_32"):
+            steps = {"whole": traces.whole, "portions": traces.changing_portions,
+                     "mixed": traces.mixed, "prefill_then_32": traces.prefill_then_single}[mode](requests)
+            eng = make_engine(path, "float32", traces.peak_tokens(steps, 16), DEV)
+            # the two latent layers share a group (64-bit, 24 and 40 wide), the attention
+            # layer has its own (32-bit, 2 heads of 16 both ways)
+            assert len(eng.cache.groups) == 2 and not eng.use_graphs
+            lat, att = eng.cache.groups
+            assert lat.k.dtype == torch.float64 and att.k.dtype == torch.float32
+            assert lat.k.shape[2] == 16 * 24 and lat.v.shape[2] == 16 * 40 and lat.k.shape[0] == 2
+            assert att.k.shape[2] == att.v.shape[2] == 2 * 16 * 16
+            assert seen["accepted"] == (torch.float64, 16 * 24, 16 * 40)
+            asked = seen.get("asked", 0)
+            got_steps = {}
+            for st in steps:
+                lg = eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]],
+                              end=st["end"])
+                if lg.shape[0]:
+                    got_steps[st["step"]] = lg.cpu().numpy().copy()
+            assert seen["asked"] == asked + len(steps), "one call a step for both latent layers"
+            eng.cache.check()
+            out = traces.collect(steps, got_steps, 190)
+            for rid in requests:
+                err = np.abs(out[rid] - ref[rid]).max() / np.abs(ref[rid]).max()
+                assert err <= 2e-5, f"{mode} {rid}: {err:.3g}"
+    finally:
+        unregister_architecture("ToyLatentForCausalLM")
+        unregister_part("mixer", ToyLatentSpec)

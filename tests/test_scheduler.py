@@ -189,9 +189,26 @@ def test_a_request_id_in_use_is_refused():
     with pytest.raises(StepError, match="already in use"):
         s.add_request([3], request_id="x")                   # running
     s.run()
-    with pytest.raises(StepError, match="already in use"):
-        s.add_request([3], request_id="x")                   # finished
     assert s.finished["x"].generated == [3, 4]
+    # finished: the id is free again, the old record goes, nothing of it is carried over
+    s.add_request([7], SamplingParams(max_new_tokens=3, **GREEDY), request_id="x")
+    assert "x" not in s.finished
+    s.run()
+    assert s.finished["x"].prompt == [7] and s.finished["x"].generated == [8, 9, 10]
+    # a rejected request is finished at once; until step() has handed it back its id is taken
+    s.add_request([], request_id="y")
+    with pytest.raises(StepError, match="already in use"):
+        s.add_request([1], request_id="y")
+    s.run()
+    s.add_request([1], SamplingParams(max_new_tokens=1, **GREEDY), request_id="y")
+    s.run()
+    assert s.finished["y"].generated == [2]
+    # the caller takes finished requests out; nothing is kept for ever
+    assert s.pop_finished("x").generated == [8, 9, 10] and "x" not in s.finished
+    assert set(s.pop_finished()) == {"y"} and s.finished == {}
+    with pytest.raises(KeyError):
+        s.pop_finished("x")
+    eng.cache.check()
 
 
 def test_sampled_output_does_not_depend_on_the_batch():

@@ -130,6 +130,32 @@ def test_dtypes_are_kept(tmp_path):
     assert model32.embedding.dtype == torch.float32
 
 
+def test_float16_checkpoint_under_both_builds(tmp_path):
+    """A float16 checkpoint: the 32-bit build holds its values exactly, the bfloat16 build
+    rounds the matrices to bfloat16 (not 32-bit tensors of twice the bytes that would miss
+    the bfloat16 kernels); gains are 32-bit either way."""
+    cfg = tiny.config_of("A")
+    decls = declare_tensors(cfg.model_spec())
+    tensors = {k: t.to(torch.float16) for k, t in
+               draw_tensors(decls, 3, torch.float32, tied=True).items()}
+    (tmp_path / "config.json").write_text(json.dumps(tiny.TINY_A))
+    write_safetensors(str(tmp_path / "model.safetensors"), tensors)
+    got = load_tensors(str(tmp_path), decls)
+    down = "model.layers.0.mlp.down_proj.weight"
+    m32 = build_model(cfg.model_spec(), got, "float32", "cpu")
+    assert m32.blocks[0].feed_forward.down.weight.dtype == torch.float32
+    assert torch.equal(m32.blocks[0].feed_forward.down.weight, tensors[down].float())
+    assert torch.equal(m32.embedding, tensors["model.embed_tokens.weight"].float())
+    m16 = build_model(cfg.model_spec(), got, "bfloat16", "cpu")
+    assert m16.blocks[0].feed_forward.down.weight.dtype == torch.bfloat16
+    assert torch.equal(m16.blocks[0].feed_forward.down.weight, tensors[down].to(torch.bfloat16))
+    assert m16.blocks[1].mixer.qkv.weight.dtype == torch.bfloat16
+    assert m16.embedding.dtype == torch.bfloat16
+    for m in (m32, m16):
+        assert m.final_norm.gain.dtype == torch.float32
+        assert torch.equal(m.final_norm.gain, tensors["model.norm.weight"].float())
+
+
 def test_random_weights_mode(tmp_path):
     a = write_model_dir(str(tmp_path / "a"), tiny.config_of("B"), seed=5, dtype=torch.bfloat16)
     b = write_model_dir(str(tmp_path / "b"), tiny.config_of("B"), seed=5, dtype=torch.bfloat16)
@@ -223,8 +249,9 @@ def test_sharded_folder_loads_the_same_tensors(tmp_path):
 
 
 def test_float16_weights_widen_exactly(tmp_path):
-    """A float16 tensor becomes float32 (exact), never bfloat16 (3 bits of mantissa fewer):
-    under a 32-bit build the model computes with the stored values."""
+    """A float16 tensor is handed on as stored and a 32-bit build widens it exactly (it never
+    passes through bfloat16, 3 bits of mantissa fewer): the model computes with the stored
+    values."""
     cfg = tiny.config_of("A")
     decls = declare_tensors(cfg.model_spec())
     tensors = {k: v.to(torch.float16) for k, v in draw_tensors(decls, 2, torch.float32, tied=True).items()}
@@ -232,7 +259,7 @@ def test_float16_weights_widen_exactly(tmp_path):
     write_safetensors(str(tmp_path / "model.safetensors"), tensors)
     got = load_tensors(str(tmp_path), decls)
     for k, v in tensors.items():
-        assert got[k].dtype == torch.float32 and torch.equal(got[k], v.float()), k
+        assert got[k].dtype == torch.float16 and torch.equal(got[k], v), k
     assert not torch.equal(tensors["model.embed_tokens.weight"].float(),
                            tensors["model.embed_tokens.weight"].to(torch.bfloat16).float())
     model = build_model(cfg.model_spec(), got, "float32", "cpu")

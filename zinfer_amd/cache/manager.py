@@ -7,8 +7,9 @@ The reference keeps one contiguous buffer per request and layer, sized at creati
 that has run out.  Paging, groups and slots are this engine's own.
 
 Layout of a group's pool, per run of a layer: keys ``[num_pages, n_kv_heads, page_size,
-head_dim]`` and values ``[num_pages, n_kv_heads, head_dim, page_size]`` (the positions of a
-page contiguous, as the attention kernels' second matrix product reads them); token ``p`` of
+head_dim]`` and values ``[num_pages, n_kv_heads, value width, page_size]`` (the positions of a
+page contiguous, as the attention kernels' second matrix product reads them; the value
+width is the key's unless the need says otherwise, and so is the dtype); token ``p`` of
 a request lies in page ``table[p // page_size]`` at row ``p % page_size``.  The manager only
 hands out pages; the layout inside a page belongs to the kernels.
 """
@@ -31,8 +32,8 @@ class LayerCacheView:
     """What a mixer gets for one run of its layer."""
     group: int                       # index of the KV group (-1: none)
     page_size: int
-    k_pool: Optional[torch.Tensor]   # [num_pages, n_kv * page_size * head_dim] or None
-    v_pool: Optional[torch.Tensor]
+    k_pool: Optional[torch.Tensor]   # [num_pages, n_kv * page_size * key width] or None
+    v_pool: Optional[torch.Tensor]   # [num_pages, n_kv * page_size * value width] or None
     writes: bool                     # False: the run only reads another run's cache
     state: Optional[torch.Tensor]    # [max_requests, *shape] for a StateNeed
 
@@ -45,9 +46,12 @@ class KVGroup:
         self.page_size = page_size
         self.pages = PageAllocator(num_pages)
         self.tables: Dict[object, List[int]] = {}
-        row = need.n_kv_heads * page_size * need.head_dim
-        self.k = torch.zeros((len(runs), num_pages, row), dtype=dtype, device=device)
-        self.v = torch.zeros((len(runs), num_pages, row), dtype=dtype, device=device)
+        # a need may bring its own dtype and a value row of another width than a key's
+        dtype = need.dtype or dtype
+        self.k = torch.zeros((len(runs), num_pages, need.n_kv_heads * page_size * need.key_width),
+                             dtype=dtype, device=device)
+        self.v = torch.zeros((len(runs), num_pages, need.n_kv_heads * page_size * need.value_width),
+                             dtype=dtype, device=device)
 
     def first_needed_page(self, length: int) -> int:
         """Logical index of the first page a query at position >= ``length`` can still read."""
@@ -248,7 +252,8 @@ class CacheManager:
         return [g.pages.num_free for g in self.groups]
 
     def kv_bytes(self) -> int:
-        return sum(g.k.numel() * g.k.element_size() * 2 for g in self.groups)
+        return sum(g.k.numel() * g.k.element_size() + g.v.numel() * g.v.element_size()
+                   for g in self.groups)
 
     def check(self) -> None:
         """No page lost, none held twice: the pages in all tables are exactly the held ones."""

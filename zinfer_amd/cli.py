@@ -539,6 +539,7 @@ def cmd_serve_batch(args: List[str]) -> int:
                 n_tokens += len(req.generated)
                 out.write(json.dumps(rec, ensure_ascii=False) + "\n")
                 out.flush()
+                sched.pop_finished(req.id)      # written out: the scheduler keeps nothing of it
     finally:
         if out_path:
             out.close()
@@ -647,6 +648,9 @@ def cmd_bench(args: List[str], mode: str) -> int:
                     live[n] = t
         torch.cuda.synchronize()
         t2 = time.perf_counter()
+        for n in names:                       # what the requests hold goes back
+            eng.release(n)
+        eng.cache.check()
         if batch > 1:
             print(f"batch_size: {batch}")
         print(f"prompt_tokens: {len(ids)}")

@@ -80,13 +80,9 @@ class StepContext:
     q_lens: List[int]             # host copies, for parts that loop on the host
     ctx_lens: List[int]
     slots: List[int]
-    n_single: int = 0             # sequences with exactly one token in this step
-    # hints for kernels that cut their work by them: the 32-token tiles of the sequences with
-    # more than one token, as a number, as int32 pairs (sequence, tile) on the device with
-    # the tiles that read the most keys first, and those sequences' longest context
-    n_query_tiles: Optional[int] = None
-    q_tile_map: Optional[torch.Tensor] = None
-    prefill_max_ctx: Optional[int] = None
+    # what parts asked to know about the step's shape (``Part.step_hints``), by their
+    # ``hint_key``: ``StepHints`` whose arrays are int32 views on the device
+    hints: Dict[object, object] = field(default_factory=dict)
     meta_offset: int = 0          # address of the packed metadata (part of a graph's key)
     wants_all_rows: bool = False  # want_rows is 0, 1, ..., n_tokens - 1
     # A part that adds into the residual stream may, in the same kernel, leave what the norm

@@ -17,6 +17,7 @@ from ..cache import NO_PAGE, CacheManager
 from ..errors import (CacheFull, ConfigError, PositionOutOfBounds, StepError,
                       TokenIdOutOfBounds)
 from ..models.decoder import DecoderModel
+from ..parts.base import StepHints, StepShape
 from .batch import KVStepTables, Scratch, StepContext, StepEntry
 
 
@@ -28,6 +29,7 @@ class Engine:
     """Owns a model, its cache and work buffers; ``step`` is the only way tokens run."""
 
     GRAPH_PAGE_BUCKET = 64      # decode graphs are captured for block tables this many pages wide
+    STEP_TRACE_MAX = 65536      # most records ``step_trace`` keeps
     MAX_GRAPHS = 256            # the least recently replayed graph goes when there are more
 
     def __init__(self, model: DecoderModel, *, page_size: int = 16, num_pages: int = 256,
@@ -40,17 +42,16 @@ class Engine:
             from ..ops import build
             build.prepare(getattr(model, "kernel_modules", ()))
         spec = model.spec
-        if kv_dtype is not None and kv_dtype != model.ctx.compute_dtype:
-            # the cache-write and attention kernels keep keys and values in the activations'
-            # dtype; there is no converting write
-            raise ConfigError(f"the cache is kept in the compute dtype ({model.ctx.compute_dtype}"
-                              f"): a cache of {kv_dtype} needs a model built with that dtype")
         needs = model.cache_needs()
         reads = [e.cache_of for e in spec.schedule]
         self.cache = CacheManager(needs, reads, page_size, num_pages, max_requests,
                                   kv_dtype or model.ctx.compute_dtype, self.device,
                                   poison_freed=poison_freed)
         self.views = [self.cache.view(pos) for pos in range(len(spec.schedule))]
+        # a mixer whose kernels cannot serve the cache it was given says so now
+        model.accept_caches(self.views)
+        # the parts that want to know about a step's shape, one per kind
+        self._hint_providers = model.hint_providers()
         self.page_size = page_size
         self._scratch = Scratch(self.device)
         self._meta_host = None          # two pinned buffers that take turns
@@ -65,7 +66,9 @@ class Engine:
         self.graph_replays = 0
         # measurement: when a list, every step appends (tokens, sequences, seconds of host
         # packing, seconds of host launching, event before, event after the step's kernels,
-        # whether a request brought more than one token)
+        # whether a request brought more than one token).  Every record holds two events:
+        # whoever switches tracing on empties the list as it reads it (``drain_step_trace``);
+        # beyond STEP_TRACE_MAX records the oldest go.
         self.step_trace: Optional[list] = None
 
     # ------------------------------------------------------------------ requests
@@ -110,9 +113,8 @@ class Engine:
                     else self.model.forward(ctx, self.views)
                 if traced:
                     after.record()
-                    self.step_trace.append((ctx.n_tokens, ctx.n_seqs, t1 - t0,
-                                            time.perf_counter() - t1, before, after,
-                                            ctx.max_q_len > 1))
+                    self._trace((ctx.n_tokens, ctx.n_seqs, t1 - t0, time.perf_counter() - t1,
+                                 before, after, ctx.max_q_len > 1))
             except BaseException:
                 self._roll_back(wanted_len, added)
                 raise
@@ -125,6 +127,16 @@ class Engine:
         for rid in end:
             self.cache.release(rid)
         return logits
+
+    def _trace(self, record) -> None:
+        self.step_trace.append(record)
+        if len(self.step_trace) > self.STEP_TRACE_MAX:
+            del self.step_trace[:len(self.step_trace) - self.STEP_TRACE_MAX]
+
+    def drain_step_trace(self) -> list:
+        """The records gathered so far (the list is emptied; tracing stays on)."""
+        done, self.step_trace = self.step_trace or [], [] if self.step_trace is not None else None
+        return done
 
     def _reserve(self, wanted_len) -> List[object]:
         """Adds the requests that are new and reserves every request's pages; returns the
@@ -205,7 +217,7 @@ class Engine:
                             f"are free (free pages per group: {self.cache.num_free_pages()})")
         added = self._reserve(wanted_len)
         try:
-            traced = self.step_trace is not None
+            traced = self.step_trace is not None and self.device.type == "cuda"
             if traced:
                 import time
                 t0 = time.perf_counter()
@@ -233,8 +245,8 @@ class Engine:
                     ops.sample_topk(logits, rec[s], out[s])
             if traced:
                 after.record()
-                self.step_trace.append((n * n_steps, n, t1 - t0, time.perf_counter() - t1, before,
-                                        after, False))
+                self._trace((n * n_steps, n, t1 - t0, time.perf_counter() - t1, before, after,
+                             False))
             tokens = out.tolist()
         except BaseException:
             self._roll_back(wanted_len, added)
@@ -329,24 +341,29 @@ class Engine:
         max_pages = max((c + extra_tokens + ps - 1) // ps for c in ctx_lens)
         max_ctx = max(ctx_lens) + extra_tokens
         if bucket_pages:      # a fixed table width (and context bound) per captured graph
-            b = self.GRAPH_PAGE_BUCKET
-            from ..ops import DECODE_SPLIT_KEYS
-            short = max(1, DECODE_SPLIT_KEYS // ps)
-            if max_pages <= short:
-                b = short     # contexts within one split of the decode attention: no merge kernel
-            max_pages = (max_pages + b - 1) // b * b
+            # a part whose kernels' grids follow the width may ask for one of its own
+            asked = [w for w in (p.graph_table_pages(max_pages, ps) for p in self._hint_providers)
+                     if w is not None]
+            if asked:
+                max_pages = max(max_pages, *asked)
+            else:
+                b = self.GRAPH_PAGE_BUCKET
+                max_pages = (max_pages + b - 1) // b * b
             max_ctx = max_pages * ps
 
+        # what the parts want to know about the step's shape: their arrays ride in the upload
+        shape = StepShape(q_lens, starts, ctx_lens, ps, fixed_shapes=bucket_pages)
+        hinted = [(p.hint_key, p.step_hints(shape)) for p in self._hint_providers]
+        hinted = [(k, h) for k, h in hinted if h is not None]
+
         # one packed int32 buffer, one copy to the device
-        # the 32-token query tiles of the sequences that bring more than one token, those that
-        # read the most keys first
-        tiles = [(starts[i] + min(32 * (t + 1), q_lens[i]), i, t) for i in range(n_seqs)
-                 if q_lens[i] > 1 for t in range((q_lens[i] + 31) // 32)]
-        tiles.sort(key=lambda x: -x[0])
-        n_tiles = len(tiles)
         sizes = [("token_ids", T), ("positions", T), ("seq_index", T), ("q_start", n_seqs + 1),
-                 ("ctx_len", n_seqs), ("state_slots", n_seqs), ("want_rows", max(n_want, 1)),
-                 ("q_tile_map", 2 * n_tiles)]
+                 ("ctx_len", n_seqs), ("state_slots", n_seqs), ("want_rows", max(n_want, 1))]
+        for i, (_, h) in enumerate(hinted):
+            for name, arr in h.arrays.items():
+                if arr.dtype != np.int32:
+                    raise StepError(f"step hint {name!r} must be an int32 array, is {arr.dtype}")
+                sizes.append((f"hint{i}.{name}", arr.size))
         for g in range(n_groups):
             sizes += [(f"slot_mapping{g}", T), (f"block_table{g}", n_seqs * max_pages)]
         offs, total = {}, 0
@@ -374,8 +391,9 @@ class Engine:
         put("ctx_len", np.asarray(ctx_lens, dtype=np.int32))
         put("state_slots", np.asarray(slots, dtype=np.int32))
         put("want_rows", np.asarray(want_rows, dtype=np.int32))
-        if n_tiles:
-            put("q_tile_map", np.asarray([(i, t) for _, i, t in tiles], dtype=np.int32).reshape(-1))
+        for i, (_, h) in enumerate(hinted):
+            for name, arr in h.arrays.items():
+                put(f"hint{i}.{name}", arr.reshape(-1))
         for g in range(n_groups):
             bt = np.full((n_seqs, max_pages), NO_PAGE, dtype=np.int32)
             sm = np.empty((T,), dtype=np.int32)
@@ -408,10 +426,10 @@ class Engine:
             want_rows=view("want_rows")[:n_want], kv=kv, max_q_len=max(q_lens),
             max_ctx_len=max_ctx, q_lens=q_lens, ctx_lens=ctx_lens, slots=slots,
             meta_offset=self._meta_dev.data_ptr() if self._meta_dev is not None else 0,
-            n_single=sum(1 for n in q_lens if n == 1),
-            n_query_tiles=n_tiles,
-            q_tile_map=view("q_tile_map").view(n_tiles, 2) if n_tiles else None,
-            prefill_max_ctx=max((c for c, n in zip(ctx_lens, q_lens) if n > 1), default=None),
+            hints={k: StepHints({name: view(f"hint{i}.{name}").view(arr.shape)
+                                 for name, arr in h.arrays.items() if arr.size},
+                                dict(h.numbers))
+                   for i, (k, h) in enumerate(hinted)},
             wants_all_rows=want_rows == list(range(T)),
             _scratch=self._scratch)
 

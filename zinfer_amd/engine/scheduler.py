@@ -91,14 +91,17 @@ class Scheduler:
     # ------------------------------------------------------------------ requests
     def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None,
                     request_id=None) -> object:
-        """Queues a request and returns its id.  An id that is already in use is the caller's
-        mistake and raises; a request that can never run is rejected (see the module's text)."""
+        """Queues a request and returns its id.  An id that a live request (waiting, running
+        or holding pages) has is the caller's mistake and raises; the id of a request that has
+        finished may be used again, and its old record then goes.  A request that can never
+        run is rejected (see the module's text)."""
         prompt = [int(t) for t in prompt]
         params = params or SamplingParams()
         rid = request_id if request_id is not None else self._next_id
-        if rid in self.finished or self.cache.has_request(rid) or \
+        if self.cache.has_request(rid) or any(r.id == rid for r in self._rejected) or \
                 any(r.id == rid for r in self.running) or any(r.id == rid for r in self.waiting):
             raise StepError(f"request id {rid!r} is already in use")
+        self.finished.pop(rid, None)
         index = self._next_id
         self._next_id += 1
         # every request has a stream of its own, so its output does not depend on the batch
@@ -129,6 +132,16 @@ class Scheduler:
             return (f"CacheFull: a prompt of {len(req.prompt)} tokens needs {need} pages, the "
                     f"pool has {self.cache.num_pages()}")
         return None
+
+    def pop_finished(self, rid=None):
+        """Takes finished requests out of the scheduler: the one with this id (KeyError if it
+        has not finished), or, without an id, all of them as {id: request}.  ``finished``
+        otherwise keeps every request's prompt and tokens: a loop that serves for long calls
+        this once it has handed a result on."""
+        if rid is not None:
+            return self.finished.pop(rid)
+        done, self.finished = self.finished, {}
+        return done
 
     def has_work(self) -> bool:
         return bool(self.waiting or self.running or self._rejected)

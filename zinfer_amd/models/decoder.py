@@ -13,7 +13,6 @@ from ..config.specs import ModelSpec
 from ..errors import ConfigError
 from ..parts import BuildContext, TensorDecl, build_part
 from ..parts.linear import Linear, place_matrix
-from ..parts.norm import LazyRmsNorm, RmsNorm
 
 
 class DecoderModel:
@@ -64,6 +63,19 @@ class DecoderModel:
             # itself stays in rows for the gather); elsewhere both are one tensor.
             self.head = Linear(self.embedding)
 
+    def hint_providers(self):
+        """One part per ``hint_key`` among all the blocks' parts: the engine asks each once a
+        step for what its kernels want to know about the step's shape."""
+        seen = {}
+        for b in self.blocks:
+            for p in b.hint_providers():
+                seen.setdefault(p.hint_key, p)
+        return list(seen.values())
+
+    def accept_caches(self, caches) -> None:
+        for pos, e in enumerate(self.spec.schedule):
+            self.blocks[e.layer].accept_cache(caches[pos])
+
     # ---------------------------------------------------------------- cache needs
     def cache_needs(self) -> List[Optional[object]]:
         """For each schedule position: the cache need of the run, or None if it has none or
@@ -79,8 +91,6 @@ class DecoderModel:
         T = step.n_tokens
         x = step.scratch("residual", (T, s.hidden_size), torch.float32)
         ops.embed(self.embedding, step.token_ids, x, float(s.embedding_multiplier))
-        lazy_final = isinstance(self.final_norm, RmsNorm) and x.is_cuda \
-            and self.ctx.compute_dtype == torch.bfloat16
         step.norm_ready = None
         for pos, e in enumerate(s.schedule):
             # the norm that reads the stream after this block: the next block's first, or the
@@ -88,10 +98,11 @@ class DecoderModel:
             if pos + 1 < len(s.schedule):
                 after = getattr(self.blocks[s.schedule[pos + 1].layer], "entry_norm", None)
             else:
-                after = self.final_norm if lazy_final and step.wants_all_rows else None
+                after = self.final_norm if self.final_norm.defers and step.wants_all_rows \
+                    else None
             step.norm_after_block = after
             self.blocks[e.layer].forward(x, step, caches[pos])
-        ready, step.norm_ready, step.norm_after_block = step.norm_ready, None, None
+        left, step.norm_ready, step.norm_after_block = step.norm_ready, None, None
         n_rows = step.n_want
         logits = step.scratch("logits", (n_rows, s.vocab_size), torch.float32)
         if n_rows == 0:
@@ -99,15 +110,14 @@ class DecoderModel:
         if step.wants_all_rows:
             rows = x
         else:
-            ready = None
+            left = None
             rows = step.scratch("want_rows", (n_rows, s.hidden_size), torch.float32)
             ops.gather_rows(x, step.want_rows, rows)
         make = lambda: step.scratch("final_normed", (n_rows, s.hidden_size), self.ctx.act_dtype)
-        if lazy_final:
-            given = ready if ready is not None and ready.fits(self.final_norm, rows) else None
-            self.head.forward(LazyRmsNorm(self.final_norm, rows, make, given), logits)
-        else:
-            self.head.forward(self.final_norm.forward(rows, make()), logits)
+        normed = self.final_norm.deferred(rows, make, left)
+        if normed is None:
+            normed = self.final_norm.forward(rows, make())
+        self.head.forward(normed, logits)
         if s.logit_scale != 1.0 or s.logit_softcap is not None:
             ops.scale_cap(logits, float(s.logit_scale), float(s.logit_softcap or 0.0))
         return logits

@@ -818,6 +818,7 @@ def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bo
 # ------------------------------------------------------------------------- attention
 MAX_HEAD_DIM = 512          # the wave kernel keeps a head in registers: 8 values a lane
 DECODE_SPLIT_KEYS = 256     # keys per split of the decode kernel (DEC_SPLIT in attention.hip)
+PREFILL_QUERY_TILE = 32     # queries per tile of the kernels for prompt portions
 
 
 def mfma_attention_covers(dtype, n_heads, n_kv_heads, head_dim, page_size) -> bool:

@@ -1,7 +1,9 @@
 """One flat table of the engine's kernels: name -> (the function that launches it, the csrc
-module it lives in, the plain reference it is tested against).  The reference's counterpart is
-its table of ops that the per-op benchmark walks (`src/app/cli/tools/bench/ops.zig:12-49`).
-References are named, not imported: those under ``tests/`` are no part of the package."""
+module it lives in, where the reference implementation states the formula it computes).  The
+reference's counterpart is its table of ops that the per-op benchmark walks
+(`src/app/cli/tools/bench/ops.zig:12-49`).  Kernels without a counterpart there (paging,
+batching, fusions of two of the reference's operations) name the operations they are made of,
+or say "own"."""
 from __future__ import annotations
 
 from dataclasses import dataclass
@@ -17,39 +19,42 @@ from . import (advance_decode, apply_penalties, argmax, argmax_no_alloc, cast,
 class KernelEntry:
     launch: Callable
     module: str          # csrc/<module>.hip
-    reference: str       # "file:function" of the plain implementation its test compares with
+    formula: str         # file:lines of the reference implementation, or "own: ..."
 
+
+_LINEAR = "src/kernel/core/cpu.zig:21-36"
+_RMSNORM = "src/kernel/core/cpu.zig:38-48,73-110"
+_ATTENTION = "src/kernel/attention/basic.zig:5-76"
+_QK = "src/kernel/core/cpu.zig:50-71; src/kernel/attention/rope.zig:25-34,67-90"
 
 KERNELS: Dict[str, KernelEntry] = {
-    "embed": KernelEntry(embed, "elementwise", "tests/kernel_refs.py:embed"),
-    "rmsnorm": KernelEntry(rmsnorm, "elementwise", "tests/kernel_refs.py:rmsnorm"),
-    "qk_norm_rope_kv_write": KernelEntry(qk_norm_rope_kv_write, "elementwise",
-                                         "tests/kernel_refs.py:qk_norm_rope_kv_write"),
-    "swiglu": KernelEntry(swiglu, "elementwise", "tests/kernel_refs.py:swiglu"),
-    "gather_rows": KernelEntry(gather_rows, "elementwise", "tests/kernel_refs.py:gather_rows"),
-    "argmax": KernelEntry(argmax, "elementwise", "tests/kernel_refs.py:argmax"),
-    "argmax_no_alloc": KernelEntry(argmax_no_alloc, "elementwise", "tests/kernel_refs.py:argmax"),
-    "scale_cap": KernelEntry(scale_cap, "elementwise", "tests/kernel_refs.py:scale_cap"),
+    "embed": KernelEntry(embed, "elementwise", "src/model/layers/decoder_only_stack.zig:48-93"),
+    "rmsnorm": KernelEntry(rmsnorm, "elementwise", _RMSNORM),
+    "qk_norm_rope_kv_write": KernelEntry(
+        qk_norm_rope_kv_write, "elementwise",
+        _QK + "; src/model/runtime/optimized_kv_cache/cache.zig:21-107"),
+    "swiglu": KernelEntry(swiglu, "elementwise", "src/kernel/core/cpu.zig:130-147"),
+    "gather_rows": KernelEntry(gather_rows, "elementwise", "own: rows whose logits are wanted"),
+    "argmax": KernelEntry(argmax, "elementwise", "src/model/layers/logits.zig:47-59"),
+    "argmax_no_alloc": KernelEntry(argmax_no_alloc, "elementwise",
+                                   "src/model/layers/logits.zig:47-59"),
+    "scale_cap": KernelEntry(scale_cap, "elementwise", "own: logit scale and tanh cap"),
     "advance_decode": KernelEntry(advance_decode, "elementwise",
-                                  "tests/test_engine_gpu.py:test_decode_steps_in_a_row_equal_single_steps"),
-    "cast": KernelEntry(cast, "elementwise", "tests/test_kernels_gpu.py:test_cast_and_poison_pages"),
-    "poison_pages": KernelEntry(poison_pages, "elementwise",
-                                "tests/test_kernels_gpu.py:test_cast_and_poison_pages"),
-    "gemm": KernelEntry(gemm, "gemm", "tests/kernel_refs.py:gemm"),
-    "gemm_partials": KernelEntry(gemm_partials, "gemm", "tests/kernel_refs.py:gemm"),
-    "gemm_swiglu": KernelEntry(gemm_swiglu, "gemm", "tests/kernel_refs.py:gemm_swiglu"),
-    "norm_gemm": KernelEntry(norm_gemm, "gemm", "tests/kernel_refs.py:rmsnorm"),
-    "gemm_emit": KernelEntry(gemm_emit, "gemm", "tests/kernel_refs.py:gemm"),
-    "gemm_given": KernelEntry(gemm_given, "gemm", "tests/kernel_refs.py:rmsnorm"),
-    "gemm_sum_norm": KernelEntry(gemm_sum_norm, "gemm", "tests/kernel_refs.py:rmsnorm"),
-    "paged_attention": KernelEntry(paged_attention, "attention",
-                                   "tests/kernel_refs.py:paged_attention"),
-    "decode_attention_fused": KernelEntry(
-        decode_attention_fused, "attention",
-        "tests/test_kernels_gpu.py:test_decode_attention_fused_equals_the_two_kernels"),
+                                  "own: positions and slots of the next decode step"),
+    "cast": KernelEntry(cast, "elementwise", "src/tensor/formats/bfloat16.zig:3-13"),
+    "poison_pages": KernelEntry(poison_pages, "elementwise", "own: NaN into pages given back"),
+    "gemm": KernelEntry(gemm, "gemm", _LINEAR),
+    "gemm_partials": KernelEntry(gemm_partials, "gemm", _LINEAR),
+    "gemm_swiglu": KernelEntry(gemm_swiglu, "gemm", _LINEAR + "; src/kernel/core/cpu.zig:130-147"),
+    "norm_gemm": KernelEntry(norm_gemm, "gemm", _RMSNORM + "; " + _LINEAR),
+    "gemm_emit": KernelEntry(gemm_emit, "gemm", _LINEAR + "; " + _RMSNORM),
+    "gemm_given": KernelEntry(gemm_given, "gemm", _RMSNORM + "; " + _LINEAR),
+    "gemm_sum_norm": KernelEntry(gemm_sum_norm, "gemm", _LINEAR + "; " + _RMSNORM),
+    "paged_attention": KernelEntry(paged_attention, "attention", _ATTENTION),
+    "decode_attention_fused": KernelEntry(decode_attention_fused, "attention",
+                                          _QK + "; " + _ATTENTION),
     "apply_penalties": KernelEntry(apply_penalties, "sampling",
-                                   "zinfer_amd/sampling/sampler.py:adjust_logits"),
-    "sample_topk": KernelEntry(sample_topk, "sampling",
-                               "zinfer_amd/sampling/sampler.py:sample_token"),
-    "randinit": KernelEntry(randinit, "randinit", "zinfer_amd/weights/counter_rng.py:draw"),
+                                   "src/sampling/sampler.zig:186-201"),
+    "sample_topk": KernelEntry(sample_topk, "sampling", "src/sampling/sampler.zig:18-91"),
+    "randinit": KernelEntry(randinit, "randinit", "own: counter-based random weights"),
 }

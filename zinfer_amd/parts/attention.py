@@ -3,12 +3,13 @@ from __future__ import annotations
 import math
 from typing import Dict
 
+import numpy as np
 import torch
 
 from .. import ops
 from ..config.specs import GqaAttentionSpec
 from ..errors import ConfigError
-from .base import KVNeed, Mixer, TensorDecl, build_part, register_part
+from .base import KVNeed, Mixer, StepHints, TensorDecl, build_part, register_part
 from .linear import Linear, place_gain, place_matrix
 
 
@@ -40,6 +41,9 @@ class GqaAttention(Mixer):
         self.scale = s.scale if s.scale is not None else 1.0 / math.sqrt(float(s.head_dim))
         self.position = build_part("position", s.position, ctx, prefix)
         self.graph_safe = self.position.graph_safe
+        # every layer of this kind cuts a step the same way, whatever its heads: one set of
+        # hints a step serves them all
+        self.hint_key = ("gqa_attention", ops.PREFILL_QUERY_TILE, ops.DECODE_SPLIT_KEYS)
 
     def declare(self) -> Dict[str, TensorDecl]:
         s, p = self.spec, self.prefix
@@ -71,6 +75,38 @@ class GqaAttention(Mixer):
 
     def cache_need(self):
         return KVNeed(self.spec.n_kv_heads, self.spec.head_dim, self.spec.window)
+
+    def accept_cache(self, cache) -> None:
+        # the cache-write and attention kernels keep keys and values in the activations'
+        # dtype; there is no converting write
+        if cache.k_pool is not None and cache.k_pool.dtype != self.ctx.act_dtype:
+            raise ConfigError(f"the cache is kept in the compute dtype ({self.ctx.act_dtype}): "
+                              f"a cache of {cache.k_pool.dtype} needs a model built with that "
+                              "dtype")
+
+    def step_hints(self, shape) -> StepHints:
+        """How the attention kernels cut the step: the tiles of ``ops.PREFILL_QUERY_TILE``
+        queries of the sequences that bring more than one token, as (sequence, tile) pairs
+        with the tiles that read the most keys first; how many sequences bring exactly one
+        token; the longest context among the others."""
+        qt = ops.PREFILL_QUERY_TILE
+        tiles = [(shape.starts[i] + min(qt * (t + 1), n), i, t)
+                 for i, n in enumerate(shape.q_lens) if n > 1 for t in range((n + qt - 1) // qt)]
+        tiles.sort(key=lambda x: -x[0])
+        arrays = {}
+        if tiles:
+            arrays["q_tile_map"] = np.asarray([(i, t) for _, i, t in tiles], dtype=np.int32)
+        return StepHints(arrays, {
+            "n_single": sum(1 for n in shape.q_lens if n == 1),
+            "n_query_tiles": len(tiles),
+            "prefill_max_ctx": max((c for c, n in zip(shape.ctx_lens, shape.q_lens) if n > 1),
+                                   default=None)})
+
+    def graph_table_pages(self, pages: int, page_size: int):
+        # contexts within one split of the decode attention get a table width of their own:
+        # that kernel then writes the output itself and no merge kernel runs
+        short = max(1, ops.DECODE_SPLIT_KEYS // page_size)
+        return short if pages <= short else None
 
     def forward(self, h, residual, step, cache) -> None:
         s = self.spec
@@ -124,12 +160,15 @@ class GqaAttention(Mixer):
                                       kv.slot_mapping if cache.writes else None,
                                       cache.k_pool, cache.v_pool, q,
                                       s.n_heads, s.n_kv_heads, s.head_dim, cache.page_size)
+        hints = step.hints.get(self.hint_key)
+        cut = {} if hints is None else dict(
+            n_single=hints.numbers["n_single"], n_query_tiles=hints.numbers["n_query_tiles"],
+            q_tile_map=hints.arrays.get("q_tile_map"),
+            prefill_max_ctx=hints.numbers["prefill_max_ctx"])
         ops.paged_attention(q, cache.k_pool, cache.v_pool, kv.block_table, step.q_start,
                             step.ctx_len, step.seq_index, attn, float(self.scale), window,
                             s.n_heads, s.n_kv_heads, s.head_dim, cache.page_size,
-                            step.max_q_len, step.max_ctx_len, n_single=step.n_single,
-                            n_query_tiles=step.n_query_tiles, q_tile_map=step.q_tile_map,
-                            prefill_max_ctx=step.prefill_max_ctx)
+                            step.max_q_len, step.max_ctx_len, **cut)
         self.o.forward(attn, residual, accumulate=True, step=step)
 
 

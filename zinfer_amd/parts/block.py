@@ -6,7 +6,6 @@ import torch
 
 from ..config.specs import PreNormBlockSpec
 from .base import Block, TensorDecl, build_part, register_part
-from .norm import LazyRmsNorm, RmsNorm
 
 
 class PreNormBlock(Block):
@@ -40,22 +39,27 @@ class PreNormBlock(Block):
     def cache_need(self):
         return self.mixer.cache_need()
 
+    def accept_cache(self, cache) -> None:
+        self.mixer.accept_cache(cache)
+
+    def hint_providers(self):
+        return [q for p in self.parts for q in p.hint_providers()]
+
     def _normed(self, norm, consumer, x, step):
         """The consumer's input: the normed activations, or, for a consumer that says it can
-        fold an RMSNorm into its first product, the norm still to be run."""
+        take a norm that has not run, the norm's stand-in (``Norm.deferred``)."""
         make = lambda: step.scratch("normed", x.shape, self.ctx.act_dtype)
-        ready, step.norm_ready, step.norm_after = step.norm_ready, None, None
-        if isinstance(norm, RmsNorm) and getattr(consumer, "accepts_lazy_norm", False) \
-                and x.is_cuda and self.ctx.compute_dtype == torch.bfloat16:
-            given = ready if ready is not None and ready.fits(norm, x) else None
-            return LazyRmsNorm(norm, x, make, given)
+        left, step.norm_ready, step.norm_after = step.norm_ready, None, None
+        if getattr(consumer, "accepts_lazy_norm", False):
+            lazy = norm.deferred(x, make, left)
+            if lazy is not None:
+                return lazy
         return norm.forward(x, make())
 
     def _lazy(self, norm, consumer):
         """``norm`` if its reader takes a norm that has not run (and so what a residual sum
         leaves for it), else None."""
-        return norm if isinstance(norm, RmsNorm) and \
-            getattr(consumer, "accepts_lazy_norm", False) else None
+        return norm if norm.defers and getattr(consumer, "accepts_lazy_norm", False) else None
 
     def forward(self, x, step, cache) -> None:
         after_block = step.norm_after_block

@@ -20,41 +20,19 @@ class Linear:
 
     def forward(self, x, out: torch.Tensor, accumulate: bool = False, step=None) -> torch.Tensor:
         """out = x W^T, or out += x W^T (``out`` float32) when ``accumulate``.  ``x`` may be a
-        norm that has not run yet (``LazyRmsNorm``): it is folded into the product when the
-        weight-streaming kernel covers it, else it runs first.  With ``accumulate`` and a
-        ``step`` that names the norm reading ``out`` next (``step.norm_after``), the sum's
-        kernel leaves that norm's inputs in ``step.norm_ready`` when it can."""
+        norm that has not run yet (what ``Norm.deferred`` gave): it folds itself into the
+        product when it can, else it runs first.  With ``accumulate`` and a ``step`` that
+        names the norm reading ``out`` next (``step.norm_after``), that norm may have the sum's
+        kernel leave something for it (``Norm.residual_sum``, result in ``step.norm_ready``)."""
         if hasattr(x, "materialize"):
-            M, K = x.shape
-            if not x.done and not accumulate and \
-                    ops.norm_gemm_plan(M, self.out_features, K, self.weight, self.tiled) is not None:
-                if x.given is not None:
-                    ops.gemm_given(x.given.xg, x.given.sq, x.eps, self.weight, out)
-                else:
-                    ops.norm_gemm(x.x, x.gain, x.eps, self.weight, out)
+            if not accumulate and x.fold_into(self, out):
                 return out
             x = x.materialize()
         norm = getattr(step, "norm_after", None) if accumulate else None
-        if norm is not None and hasattr(norm, "gain") and x.dtype == torch.bfloat16 and \
-                ops.norm_emit_plan(x.shape[0], self.out_features, self.in_features, self.weight,
-                                   self.tiled) is not None:
-            from .norm import GivenRmsNorm
-            xg = step.scratch("normed_by_gain", out.shape, torch.bfloat16)
-            sq = step.scratch("normed_squares", (self.out_features // 16, 16), torch.float32)
-            ops.gemm_emit(x, self.weight, out, norm.gain, xg, sq)
-            step.norm_ready = GivenRmsNorm(norm, out, xg, sq)
-            return out
-        if norm is not None and hasattr(norm, "gain") and x.dtype == torch.bfloat16 and \
-                ops.sum_norm_plan(x.shape[0], self.out_features, self.in_features, self.weight,
-                                  self.tiled) is not None:
-            from .norm import DoneRmsNorm
-            normed = step.scratch("normed_by_sum", out.shape, torch.bfloat16)
-            ops.gemm_sum_norm(x, self.weight, out, norm.gain, float(norm.spec.eps), normed)
-            step.norm_ready = DoneRmsNorm(norm, out, normed)
+        if norm is not None and norm.residual_sum(self, x, out, step):
             return out
         ops.gemm(x, self.weight, out, accumulate, w_tiled=self.tiled)
         return out
-
 
     def forward_partials(self, x):
         """The float32 partials [ksplit, T, out] of x W^T where the product is one that runs
@@ -73,7 +51,9 @@ class Linear:
 
 def place_matrix(t: torch.Tensor, ctx) -> torch.Tensor:
     """A matrix on the device: bfloat16 stays bfloat16 under a bfloat16 build, a tensor
-    stored in 32-bit stays so; a float32 build widens everything."""
+    stored in 32-bit stays so; a float32 build widens everything (float16 exactly).  A
+    matrix stored in float16 or float64 is rounded to bfloat16 under a bfloat16 build: as
+    32-bit data it would take twice the bytes and miss the MFMA kernels."""
     if ctx.compute_dtype == torch.float32 and t.dtype == torch.bfloat16 \
             and torch.device(ctx.device).type == "cuda":
         # half the bytes go over the bus; the widening (exact) runs on the device
@@ -85,7 +65,7 @@ def place_matrix(t: torch.Tensor, ctx) -> torch.Tensor:
     if ctx.compute_dtype == torch.float32:
         t = t.to(torch.float32)
     elif t.dtype not in (torch.bfloat16, torch.float32):
-        t = t.to(torch.float32)
+        t = t.to(torch.bfloat16)
     return t.to(ctx.device).contiguous()
 
 

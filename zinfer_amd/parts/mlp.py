@@ -46,15 +46,11 @@ class SwiGluMlp(FeedForward):
         I = self.spec.intermediate_size
         act = self.ctx.act_dtype
         a = step.scratch("ff_act", (T, I), act)
-        if self.fused and hasattr(h, "materialize") and not h.done and self.gate_up.tiled \
-                and T <= ops.NORM_FOLD_MAX_M:
-            if h.given is not None:
-                ops.gemm_given(h.given.xg, h.given.sq, h.eps, self.gate_up.weight, a, swiglu=True)
-            else:
-                ops.norm_gemm(h.x, h.gain, h.eps, self.gate_up.weight, a, swiglu=True)
-            self.down.forward(a, residual, accumulate=True, step=step)
-            return
         if hasattr(h, "materialize"):
+            # a norm that has not run: the gate/up product folds it in where it can
+            if self.fused and h.fold_into(self.gate_up, a, swiglu=True):
+                self.down.forward(a, residual, accumulate=True, step=step)
+                return
             h = h.materialize()
         if self.fused and h.dtype == torch.bfloat16:
             ops.gemm_swiglu(h, self.gate_up.weight, a, w_tiled=self.gate_up.tiled)

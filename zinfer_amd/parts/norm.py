@@ -12,8 +12,14 @@ from .linear import place_gain
 
 class RmsNorm(Norm):
     """n = x * w / sqrt(mean(x^2) + eps) (`src/kernel/core/cpu.zig:38-48,73-110`); reads the
-    float32 residual stream, writes the activation dtype."""
+    float32 residual stream, writes the activation dtype.
+
+    Under bfloat16 on the GPU the norm can be taken apart by the products around it: the
+    weight-streaming product folds it in (``LazyRmsNorm.fold_into``), and the product that
+    last adds into the residual can leave the norm's inputs or its whole result
+    (``residual_sum``)."""
     graph_safe = True
+    defers = True
     kernel_modules = ("elementwise",)
 
 
@@ -26,6 +32,29 @@ class RmsNorm(Norm):
     def forward(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         ops.rmsnorm(x, self.gain, float(self.spec.eps), out)
         return out
+
+    def deferred(self, x: torch.Tensor, make_out, left=None):
+        if not (x.is_cuda and self.ctx.compute_dtype == torch.bfloat16):
+            return None
+        given = left if left is not None and left.fits(self, x) else None
+        return LazyRmsNorm(self, x, make_out, given)
+
+    def residual_sum(self, linear, a: torch.Tensor, out: torch.Tensor, step) -> bool:
+        if a.dtype != torch.bfloat16:
+            return False
+        M, N, K = a.shape[0], linear.out_features, linear.in_features
+        if ops.norm_emit_plan(M, N, K, linear.weight, linear.tiled) is not None:
+            xg = step.scratch("normed_by_gain", out.shape, torch.bfloat16)
+            sq = step.scratch("normed_squares", (N // 16, 16), torch.float32)
+            ops.gemm_emit(a, linear.weight, out, self.gain, xg, sq)
+            step.norm_ready = GivenRmsNorm(self, out, xg, sq)
+            return True
+        if ops.sum_norm_plan(M, N, K, linear.weight, linear.tiled) is not None:
+            normed = step.scratch("normed_by_sum", out.shape, torch.bfloat16)
+            ops.gemm_sum_norm(a, linear.weight, out, self.gain, float(self.spec.eps), normed)
+            step.norm_ready = DoneRmsNorm(self, out, normed)
+            return True
+        return False
 
 
 class GivenRmsNorm:
@@ -75,6 +104,25 @@ class LazyRmsNorm:
             self._out = self._make_out()
             self._norm.forward(self.x, self._out)
         return self._out
+
+    def fold_into(self, linear, out: torch.Tensor, swiglu: bool = False) -> bool:
+        """out = norm(x) W^T (with ``swiglu`` the activation of a stacked gate/up weight) in
+        the weight-streaming product, from the residual rows or from what their producer
+        left; False (and nothing done) where that kernel does not cover the sizes."""
+        M, K = self.shape
+        if self.done or not linear.tiled:
+            return False
+        if swiglu:
+            if M > ops.NORM_FOLD_MAX_M:
+                return False
+        elif ops.norm_gemm_plan(M, linear.out_features, K, linear.weight, True) is None:
+            return False
+        if self.given is not None:
+            ops.gemm_given(self.given.xg, self.given.sq, self.eps, linear.weight, out,
+                           swiglu=swiglu)
+        else:
+            ops.norm_gemm(self.x, self.gain, self.eps, linear.weight, out, swiglu=swiglu)
+        return True
 
 
 register_part("norm", RmsNormSpec, RmsNorm)

@@ -77,11 +77,9 @@ def load_tensors(model_dir: str, decls: Dict[str, TensorDecl]) -> Dict[str, torc
             info = where[n].infos[n]
             if info.dtype in _INT:
                 t = t.to(torch.int32)
-            elif info.dtype in ("F16", "F64"):
-                # float16 widens exactly; rounding it to bfloat16 here would take 3 bits of
-                # mantissa from a 32-bit build's weights.  What a bfloat16 build does with a
-                # 32-bit tensor is the parts' business.
-                t = t.to(torch.float32)
+            # float16 and float64 are handed on as they are stored: a 32-bit build widens
+            # float16 exactly (rounding it to bfloat16 here would take 3 bits of mantissa from
+            # its weights), a bfloat16 build rounds both to bfloat16 (``place_matrix``)
             out[n] = t
         return out
     finally:
