@@ -128,9 +128,11 @@ def decode_lead(batch: int, prompt_len: int, step_tokens: int) -> int:
     return batch * ((prompt_len + room - 1) // room)
 
 
-def run_decode(llm, cfg, batch: int, prompt_len: int, steps: int, warmup: int, seed: int):
+def run_decode(llm, cfg, batch: int, prompt_len: int, steps: int, warmup: int, seed: int,
+               classes: bool = False):
     """Prefills ``batch`` requests through the scheduler, runs ``warmup`` untimed decode
-    steps, then times exactly ``steps`` steps.  Returns (seconds, mean context length)."""
+    steps, then times exactly ``steps`` steps.  Returns (seconds, mean context length), and
+    with ``classes`` a third value: where a step's time goes (see ``step_classes``)."""
     import torch
     from zinfer_amd.sampling import SamplingParams
     g = torch.Generator().manual_seed(seed)
@@ -164,22 +166,59 @@ def run_decode(llm, cfg, batch: int, prompt_len: int, steps: int, warmup: int, s
     run_exactly(warmup)
     torch.cuda.synchronize()
     ctx0 = sum(r.n_computed for r in sched.running) / batch
+    if classes:
+        llm.engine.step_trace = []
     t0 = time.perf_counter()
     run_exactly(steps)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ctx1 = sum(r.n_computed for r in sched.running) / batch
     assert len(sched.running) == batch and sched.n_preemptions == 0
+    where = None
+    if classes:
+        trace, llm.engine.step_trace = llm.engine.step_trace, None
+        where = step_classes(llm.engine, sched, trace, steps, dt)
     for r in list(sched.running):
         sched._finish(r, "bench")
-    return dt, (ctx0 + ctx1) / 2 + 0.5
+    return (dt, (ctx0 + ctx1) / 2 + 0.5) + ((where,) if classes else ())
 
 
-def decode_roofline(cfg, elem: int, batch: int, mean_ctx: float, seconds_per_step: float) -> dict:
+def step_classes(eng, sched, trace, steps: int, seconds: float) -> dict:
+    """Where a decode step's time goes, in milliseconds a step.  ``host``: the host's work for
+    the timed steps (packing metadata, launching), which runs beside the device's;
+    ``device``: between the events around the timed steps' kernels; the classes: a graph of
+    the same step with only that class's kernels, replayed (``Engine.class_times``: products =
+    the layers' matrix products with what is fused into them (norms, SwiGLU, residual sums),
+    attention = attention over the cache, in steps of up to 32 sequences with the per-head
+    norm, rotation and cache write; norm_rope_write = those as kernels of their own;
+    head_sampling = final norm, head, arg-max)."""
+    from zinfer_amd.engine import StepEntry
+    host = sum(r[2] + r[3] for r in trace) / steps
+    device = sum(r[4].elapsed_time(r[5]) for r in trace) / 1e3 / steps
+    entries = [StepEntry(r.id, [r.generated[-1]], [0]) for r in sched.running]
+    t = eng.class_times(entries)
+    out = {k + "_ms": round(v * 1e3, 4) for k, v in t.items() if k != "step"}
+    out["classes_sum_ms"] = round(sum(v for k, v in t.items() if k != "step") * 1e3, 4)
+    out["graph_step_ms"] = round(t["step"] * 1e3, 4)
+    out["device_ms"] = round(device * 1e3, 4)
+    out["host_ms"] = round(host * 1e3, 4)
+    out["wall_ms"] = round(seconds / steps * 1e3, 4)
+    return out
+
+
+def decode_roofline(cfg, elem: int, batch: int, mean_ctx: float, seconds_per_step: float,
+                    measured_gbs: float = None) -> dict:
+    """``measured``: what a kernel that only reads (16-byte non-temporal loads, 8 in flight a
+    lane, a workgroup 64 KB in a row, 2 GiB from HBM, the best pass between two events over 256
+    to 4096 workgroups) reaches on this card."""
     step_bytes = weight_bytes_per_step(cfg, elem) + batch * mean_ctx * kv_bytes_per_token(cfg, elem)
     achieved = step_bytes / seconds_per_step / 1e9
-    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-            "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)}
+    out = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+           "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)}
+    if measured_gbs:
+        out["measured_read"] = round(measured_gbs, 1)
+        out["frac_of_measured"] = round(achieved / measured_gbs, 4)
+    return out
 
 
 def config_of(cfg, shape: str, **more) -> dict:
@@ -355,28 +394,49 @@ def main_long_context(args) -> int:
 
 
 # --------------------------------------------------------------------------- the default line
-def check_fp32(llm, cfg, raw, args) -> dict:
-    """The same random weights (bfloat16 values widened) through the 32-bit path: FMA
-    products, wave attention, 32-bit cache.  Reports the largest difference of the last
-    position's logits relative to their largest magnitude, and whether the arg-max agrees."""
+def check_fp32(llm, cfg, raw, seed: int, T: int) -> dict:
+    """What bfloat16 costs at this shape: the same random weights (bfloat16 values widened)
+    through the true 32-bit path (FMA products, 32-bit attention, 32-bit cache) beside the
+    serving engine, on one prompt of ``T`` tokens: its first 512 tokens as one step, the rest
+    as a second, then one decode token (the 32-bit arg-max) at context ``T``.  For each of the
+    three places: the largest difference of the logits relative to their largest magnitude,
+    the root-mean-square difference relative to their root-mean-square, and whether the
+    arg-max agrees."""
     import torch
     from zinfer_amd.engine import Engine, StepEntry
     from zinfer_amd.models.build import random_model
-    T = args.check_fp32
-    g = torch.Generator().manual_seed(args.seed + 99)
+    g = torch.Generator().manual_seed(seed + 99)
     toks = torch.randint(0, cfg.vocab_size, (T,), generator=g).tolist()
-    want = [T - 1]
-    lb = llm.engine.step([StepEntry("chk", toks, want)], end=["chk"]).float().clone()
+    head = min(512, T)
     # same seed, same draws, rounded to bfloat16 as the serving model's, then widened
-    _, model32 = random_model(raw, args.seed, "float32", "cuda:0", store_dtype="bfloat16")
-    eng32 = Engine(model32, page_size=PAGE, num_pages=(T + PAGE - 1) // PAGE + 1, max_requests=2)
+    _, model32 = random_model(raw, seed, "float32", "cuda:0", store_dtype="bfloat16")
+    eng32 = Engine(model32, page_size=PAGE, num_pages=(T + 1 + PAGE - 1) // PAGE + 1,
+                   max_requests=2)
+    out = {"tokens": T}
     t0 = time.perf_counter()
-    lf = eng32.step([StepEntry("chk", toks, want)], end=["chk"]).float()
+    cuts = [("prefill_%d" % head, toks[:head])]
+    if T > head:
+        cuts.append(("prefill_%d" % T, toks[head:]))
+    nxt = None
+    for name, part in cuts + [("decode_ctx%d" % T, None)]:
+        part = [nxt] if part is None else part
+        entry = [StepEntry("chk", part, [len(part) - 1])]
+        lb = llm.engine.step(entry).float().clone()
+        lf = eng32.step(entry).float()
+        nxt = int(lf.argmax())
+        out[name] = {
+            "rel_max_diff": round(float((lb - lf).abs().max() / lf.abs().max()), 5),
+            "rel_rms_diff": round(float((lb - lf).pow(2).mean().sqrt() / lf.pow(2).mean().sqrt()), 5),
+            "argmax_equal": bool(int(lb.argmax()) == nxt)}
     torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    err = float((lb - lf).abs().max() / lf.abs().max())
-    return {"tokens": T, "rel_max_diff": round(err, 5), "fp32_ms": round(dt * 1e3, 1),
-            "argmax_equal": bool(int(lb.argmax()) == int(lf.argmax()))}
+    out["seconds"] = round(time.perf_counter() - t0, 2)
+    llm.engine.release("chk")
+    eng32.release("chk")
+    del eng32, model32
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()
+    return out
 
 
 def main_decode(args) -> int:
@@ -398,9 +458,11 @@ def main_decode(args) -> int:
     elem = 2 if args.dtype == "bfloat16" else 4
     peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
 
+    import zinfer_amd.ops as ops
+    measured_gbs = ops.measure_read_bandwidth("cuda:0") / 1e9
     pre_s = run_prefill(llm, cfg, args.prefill_tokens, args.seed + 1)
-    dt, mean_ctx = run_decode(llm, cfg, args.batch, args.prompt_len, args.steps, args.warmup,
-                              args.seed + 2)
+    dt, mean_ctx, where = run_decode(llm, cfg, args.batch, args.prompt_len, args.steps,
+                                     args.warmup, args.seed + 2, classes=True)
     value = args.batch * args.steps / dt
     points = {}
     if not args.no_points:
@@ -426,12 +488,16 @@ def main_decode(args) -> int:
         "prefill": {"value": round(args.prefill_tokens / pre_s, 1), "tokens": args.prefill_tokens,
                     "ms": round(pre_s * 1e3, 3),
                     "frac": round(prefill_flops(cfg, args.prefill_tokens) / pre_s / peak, 4)},
-        "roofline": decode_roofline(cfg, elem, args.batch, mean_ctx, dt / args.steps),
+        "roofline": decode_roofline(cfg, elem, args.batch, mean_ctx, dt / args.steps,
+                                    measured_gbs),
+        "classes": where,
         "points": points,
         "build_s": round(build_s, 1),
     }
-    if args.check_fp32:
-        line["fp32_check"] = check_fp32(llm, cfg, raw, args)
+    check_tokens = args.check_fp32 if args.check_fp32 is not None else \
+        (0 if args.no_points or args.dtype != "bfloat16" else 2048)
+    if check_tokens:
+        line["fp32_check"] = check_fp32(llm, cfg, raw, args.seed, check_tokens)
     if not args.no_points and args.layers is None and args.dtype == "bfloat16":
         # the other two workloads in short form (their own modes report them in full)
         drop(llm)
@@ -480,9 +546,10 @@ def main() -> int:
                     help="only the headline: no other batches, prompt lengths or workloads")
     ap.add_argument("--no-long-context-points", dest="long_context_points", action="store_false",
                     help="leave the 32B-shape points out of the default line")
-    ap.add_argument("--check-fp32", type=int, default=0, metavar="TOKENS",
-                    help="also run a prompt of TOKENS tokens through a true 32-bit engine with "
-                         "the same weights and report how far the logits are apart")
+    ap.add_argument("--check-fp32", type=int, default=None, metavar="TOKENS",
+                    help="also run a prompt of TOKENS tokens and one decode token through a true "
+                         "32-bit engine with the same weights and report how far the logits "
+                         "are apart (default: 2048, with --no-points 0 = not at all)")
     ap.add_argument("--requests", type=int, default=32, help="continuous: requests")
     ap.add_argument("--prompt-min", type=int, default=128)
     ap.add_argument("--prompt-max", type=int, default=4096)

@@ -223,7 +223,14 @@ def model_forward(cfg: dict, weights: Dict[str, torch.Tensor], token_ids: Sequen
 # tests check it against ``model_forward`` and then use it for the longer sequences.
 def model_forward_batched(cfg: dict, weights: Dict[str, torch.Tensor],
                           token_ids: Sequence[int], window: Optional[int] = None,
-                          return_hidden: bool = False) -> torch.Tensor:
+                          return_hidden: bool = False, act_round=None) -> torch.Tensor:
+    """``act_round``: a rounding (such as ``bf16_round``) applied wherever an engine that
+    keeps its activations in bfloat16 between kernels stores one: the normed rows, q/k/v,
+    q and k after norm and rotation, the soft-max terms before they meet the values, the
+    attention's output, the feed-forward's activation, the final normed rows.  The residual
+    stream and every sum stay exact.  It models what such an engine's distance from the exact
+    result should be; it is no reference for values."""
+    rnd = (lambda t: act_round(t).to(F64)) if act_round is not None else (lambda t: t)
     H = cfg["hidden_size"]; nH = cfg["num_attention_heads"]; nKV = cfg["num_key_value_heads"]
     hd = cfg["head_dim"]; eps = cfg["rms_norm_eps"]; theta = cfg["rope_theta"]
     L = cfg["num_hidden_layers"]; G = nH // nKV
@@ -252,26 +259,31 @@ def model_forward_batched(cfg: dict, weights: Dict[str, torch.Tensor],
         allowed &= pos[None, :] > pos[:, None] - window
     for l in range(L):
         w = lambda s: weights[layer_name(l, s)].to(F64)
-        n = rms_norm(x, w("input_layernorm.weight"), eps)
-        q = n @ w("self_attn.q_proj.weight").T
-        k = n @ w("self_attn.k_proj.weight").T
-        v = n @ w("self_attn.v_proj.weight").T
-        q = rot(headnorm(q, nH, w("self_attn.q_norm.weight")), nH)      # [T, nH, hd]
-        k = rot(headnorm(k, nKV, w("self_attn.k_norm.weight")), nKV)    # [T, nKV, hd]
+        n = rnd(rms_norm(x, w("input_layernorm.weight"), eps))
+        q = rnd(n @ w("self_attn.q_proj.weight").T)
+        k = rnd(n @ w("self_attn.k_proj.weight").T)
+        v = rnd(n @ w("self_attn.v_proj.weight").T)
+        q = rnd(rot(headnorm(q, nH, w("self_attn.q_norm.weight")), nH))      # [T, nH, hd]
+        k = rnd(rot(headnorm(k, nKV, w("self_attn.k_norm.weight")), nKV))    # [T, nKV, hd]
         v = v.reshape(T, nKV, hd)
         kx = k.repeat_interleave(G, dim=1)  # query head h reads kv head h // G
         vx = v.repeat_interleave(G, dim=1)
         s = torch.einsum("thd,shd->hts", q, kx) * (1.0 / math.sqrt(float(hd)))
         s = s.masked_fill(~allowed[None], float("-inf"))
-        a = torch.softmax(s, dim=-1)
-        o = torch.einsum("hts,shd->thd", a, vx).reshape(T, nH * hd)
+        if act_round is None:
+            a = torch.softmax(s, dim=-1)
+            o = torch.einsum("hts,shd->thd", a, vx).reshape(T, nH * hd)
+        else:       # the terms are rounded, their sum is not
+            e = torch.exp(s - s.max(dim=-1, keepdim=True).values)
+            o = torch.einsum("hts,shd->thd", rnd(e), vx) / e.sum(-1).T[:, :, None]
+            o = rnd(o.reshape(T, nH * hd))
         r = x + o @ w("self_attn.o_proj.weight").T
-        m = rms_norm(r, w("post_attention_layernorm.weight"), eps)
-        act = swiglu(m @ w("mlp.gate_proj.weight").T, m @ w("mlp.up_proj.weight").T)
+        m = rnd(rms_norm(r, w("post_attention_layernorm.weight"), eps))
+        act = rnd(swiglu(m @ w("mlp.gate_proj.weight").T, m @ w("mlp.up_proj.weight").T))
         x = r + act @ w("mlp.down_proj.weight").T
     if return_hidden:
         return x
-    n = rms_norm(x, weights["model.norm.weight"], eps)
+    n = rnd(rms_norm(x, weights["model.norm.weight"], eps))
     return n @ lm_head_weight(cfg, weights).to(F64).T
 
 

@@ -124,6 +124,7 @@ TESTED_AGAINST = {
         "test_kernels_gpu.py:test_decode_attention_fused_equals_the_two_kernels",
     "apply_penalties": "plain.py:adjusted_logit", "sample_topk": "plain.py:sample_token",
     "randinit": "test_kernels_gpu.py:test_randinit_is_the_numpy_draw_bit_for_bit",
+    "stream_read": "test_kernels_gpu.py:test_stream_read_reads_every_byte_once",
 }
 
 
@@ -143,6 +144,7 @@ def test_the_flat_kernel_table_is_complete_and_every_kernel_has_a_reference():
     here = os.path.dirname(os.path.abspath(__file__))
     for name, entry in table.KERNELS.items():
         assert entry.launch is getattr(ops, name)
+        assert entry.launch.kernel_class in ops.KERNEL_CLASSES, name
         assert entry.module in build.MODULES
         assert entry.formula.startswith(("src/", "own: ")), name
         path, fn = TESTED_AGAINST[name].split(":")
@@ -190,3 +192,54 @@ def test_measured_plans_are_plans_the_kernels_take():
     assert ops._skinny_plan(8, 5120, 5120, True) == (2, 1) and ops._skinny_plan(8, 4096, 4096, True) == (1, 1)
     assert ops._skinny_plan(8, 10240, 5120, True) == (4, 1) and ops._skinny_plan(8, 6144, 4096, True) == (2, 1)
     assert ops._skinny_plan(1, 151936, 4096, True) == (2, 1)
+
+
+def test_widths_without_an_entry_get_plans_the_launchers_accept():
+    """The measured table is an override, not the rule: for widths it does not list (other
+    models' projections, odd multiples of 64) the rules give, for every number of tokens from
+    17 to 64, a plan that passes the same check as a table entry."""
+    table = ops._measured_plans()["plans"]
+    widths = [(2048, 1024), (1024, 2048), (6144, 1024), (2048, 6144), (4096, 2560), (2560, 4096),
+              (19456, 2560), (2560, 9728), (4160, 1088), (192, 4096), (8192, 8192), (64, 64)]
+    for N, K in widths:
+        for swiglu in (False, True):
+            key = f"{N}x{K}" + (":swiglu" if swiglu else "")
+            assert key not in table, key
+            if swiglu and N % 64:
+                continue
+            for M in range(17, 65):
+                plan = ops._small_plan(M, N, K, True, swiglu=swiglu)
+                assert plan is not None and plan[0] in ("mid", "skinny"), (key, M)
+                if plan[0] == "skinny" and not swiglu:
+                    assert N % (16 * plan[1]) == 0 and plan[2] <= 16, (key, M, plan)
+                ops.check_plans({"plans": {key: {str(ops.plan_bucket(M)): list(plan)}}})
+            # the decode plans of such widths come from the rules as well
+            for M in (1, 8, 16):
+                rg, ks = ops._skinny_plan(M, N, K, True)
+                assert rg in (1, 2, 4) and N % (16 * rg) == 0 and 1 <= ks <= 16
+                assert ops._decode_acc_plan(M, N, K) is None
+
+
+def test_a_model_folders_plans_are_checked_and_override_the_table(tmp_path, monkeypatch):
+    import copy
+    import json
+    monkeypatch.setattr(ops, "_measured", copy.deepcopy(ops._measured_plans()))
+    before = ops._small_plan(40, 2048, 1024, True)
+    good = {"plans": {"2048x1024": {"48": ["skinny", 1, 2], "17": ["skinny", 2, 1]}},
+            "decode_acc": {"2048x6144": ["skinny", 2, 3], "_": "a remark"}}
+    p = tmp_path / ops.PLAN_FILE
+    p.write_text(json.dumps(good))
+    assert ops.load_plans(str(p)) == 2
+    assert ops._small_plan(40, 2048, 1024, True) == ("skinny", 1, 2) != before
+    assert ops._small_plan(64, 2048, 1024, True) == ("skinny", 1, 2)     # the nearest bucket above 32
+    assert ops._small_plan(20, 2048, 1024, True) == ("skinny", 2, 1)
+    assert ops._decode_acc_plan(8, 2048, 6144) == ("skinny", 2, 3)
+    for bad in ({"plans": {"2048x1024": {"48": ["skinny", 3, 1]}}},
+                {"plans": {"2048x1024": {"40": ["mid", 1]}}},
+                {"plans": {"2048x1024": {"48": ["mid", 9]}}},
+                {"plans": {"2048x1024:swiglu": {"48": ["mid", 2]}}},
+                {"plans": {"2048 by 1024": {"48": ["mid", 1]}}},
+                {"decode_acc": {"2048x6144": ["skinny", 2, 1]}}):
+        p.write_text(json.dumps(bad))
+        with pytest.raises(Exception, match="kernel plans"):
+            ops.load_plans(str(p))

@@ -3,6 +3,7 @@ other than the engine's tiny configurations: widths and vocabularies that are no
 two, head sizes in steps of 16, any number of heads and groups."""
 import math
 
+import numpy as np
 import pytest
 import torch
 
@@ -1073,6 +1074,40 @@ def test_mfma_prefill_window_edge_and_far_key(hd, variant):
                 assert close == inside, f"window {window}, query {p}, key {target}"
                 assert rel_err(got, want) <= 2 * tol(dtype), \
                     f"window {window}, query {p}, key {target}"
+
+
+def test_stream_read_reads_every_byte_once():
+    """The measurement kernel's xor over the buffer is the xor of all its words, for sizes
+    that are and are not a multiple of what one round of the grid takes."""
+    ops = _ops()
+    for n_words, wgs in ((4 * 1000, 7), (4 * 512 * 8 * 3, 3), (4 * 123457, 64), (1 << 22, 2048)):
+        g = torch.Generator().manual_seed(n_words)
+        buf = torch.randint(-2 ** 31, 2 ** 31 - 1, (n_words,), generator=g, dtype=torch.int32)
+        want = int(np.bitwise_xor.reduce(buf.numpy().view(np.uint32)))
+        sink = torch.zeros((wgs,), dtype=torch.int32, device=DEV)
+        ops.stream_read(buf.to(DEV), sink, wgs)
+        got = int(np.bitwise_xor.reduce(sink.cpu().numpy().view(np.uint32)))
+        assert got == want, (n_words, wgs)
+    assert ops.measure_read_bandwidth(DEV, nbytes=1 << 28, repeats=2) > 1e12
+
+
+def test_only_the_kernels_of_a_class_are_launched():
+    """Under `only_classes` a launcher of another class leaves its output alone."""
+    ops = _ops()
+    x = _rand((3, 64), torch.float32, 1).to(DEV)
+    gain = torch.ones(64, device=DEV)
+    out = torch.full((3, 64), 7.0, device=DEV)
+    with ops.only_classes({"attention"}):
+        ops.rmsnorm(x, gain, 1e-6, out)
+        assert float(out.min()) == 7.0
+        with ops.kernel_class("attention"):            # a caller's label wins
+            ops.rmsnorm(x, gain, 1e-6, out)
+        assert float(out.abs().max()) < 7.0
+    out.fill_(7.0)
+    ops.rmsnorm(x, gain, 1e-6, out)
+    assert float(out.abs().max()) < 7.0
+    with pytest.raises(Exception, match="unknown kernel classes"):
+        ops.only_classes({"nonsense"})
 
 
 def test_cast_and_poison_pages():

@@ -61,10 +61,17 @@ LONG = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_l
             intermediate_size=768, vocab_size=1536, rope_theta=1000000.0, rms_norm_eps=1e-6,
             tie_word_embeddings=False, max_position_embeddings=4096, torch_dtype="bfloat16")
 
+# the served model's depth and heads (36 layers, 32 query heads on 8 kv heads of 128) under
+# narrow widths: how far bfloat16 drifts from the exact result over a real number of layers
+DEEP = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=36,
+            hidden_size=256, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+            intermediate_size=512, vocab_size=1024, rope_theta=1000000.0, rms_norm_eps=1e-6,
+            tie_word_embeddings=False, max_position_embeddings=512, torch_dtype="bfloat16")
+
 CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "W": WIDE,
-           "L": LONG}
-PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 16, "W": 16, "L": 16}
-SEEDS = {"A": 11, "B": 22, "C": 33, "D": 44, "E": 55, "W": 66, "L": 77}
+           "L": LONG, "P": DEEP}
+PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 16, "W": 16, "L": 16, "P": 16}
+SEEDS = {"A": 11, "B": 22, "C": 33, "D": 44, "E": 55, "W": 66, "L": 77, "P": 88}
 
 
 def config_of(name: str) -> Qwen3Config:

@@ -653,3 +653,51 @@ extern "C" int zf_advance_decode(int* token_ids, int* positions, int* ctx_len, c
                      max_pages, page_size, advance);
   ZF_CHECK_LAUNCH();
 }
+
+// ---------------------------------------------------------------- measurement: a read stream
+// Reads `bytes` (a multiple of 16) once and does nothing else of weight: every lane takes
+// 16-byte non-temporal loads, 8 in flight, a workgroup 64 KB in a row at a time, and xors
+// what it read into one word per workgroup (so that no load can be dropped).  The rate
+// this reaches from HBM is what the weight-streaming kernels are measured against.
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t zf_u32x4_t;
+__global__ __launch_bounds__(512) void stream_read_kernel(const zf_u32x4_t* __restrict__ src,
+                                                          size_t n16, uint32_t* __restrict__ sink) {
+  // a workgroup takes chunks of 8 x 512 x 16 bytes = 64 KB in a row, chunk after chunk
+  const size_t chunk = (size_t)8 * blockDim.x;
+  uint32_t acc = 0;
+  size_t c = (size_t)blockIdx.x * chunk;
+  for (; c + chunk <= n16; c += (size_t)gridDim.x * chunk) {
+    zf_u32x4_t v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      v[u] = __builtin_nontemporal_load(src + c + (size_t)u * blockDim.x + threadIdx.x);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc ^= v[u][0] ^ v[u][1] ^ v[u][2] ^ v[u][3];
+  }
+  // the last, partial chunk belongs to exactly one workgroup
+  if (c < n16)
+    for (size_t i = c + threadIdx.x; i < n16; i += blockDim.x) {
+      const zf_u32x4_t v = __builtin_nontemporal_load(src + i);
+      acc ^= v[0] ^ v[1] ^ v[2] ^ v[3];
+    }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) acc ^= __shfl_xor(acc, o, 64);
+  __shared__ uint32_t part[8];
+  if (threadIdx.x % 64 == 0) part[threadIdx.x / 64] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t a = 0;
+    for (int w = 0; w < (int)blockDim.x / 64; ++w) a ^= part[w];
+    sink[blockIdx.x] = a;
+  }
+}
+
+// sink: at least `workgroups` words.  bytes % 16 == 0, 1 <= workgroups <= 65536.
+extern "C" int zf_stream_read(const void* src, long long bytes, uint32_t* sink, int workgroups,
+                              hipStream_t stream) {
+  if (bytes <= 0) return 0;
+  if (bytes % 16 != 0 || workgroups < 1 || workgroups > 65536) return 1;
+  hipLaunchKernelGGL(stream_read_kernel, dim3(workgroups), dim3(512), 0, stream,
+                     (const zf_u32x4_t*)src, (size_t)(bytes / 16), sink);
+  ZF_CHECK_LAUNCH();
+}

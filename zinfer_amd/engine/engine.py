@@ -256,6 +256,55 @@ class Engine:
         self.steps_run += n_steps
         return tokens
 
+    def class_times(self, entries: Sequence[StepEntry], repeats: int = 20) -> Dict[str, float]:
+        """Seconds a decode step of ``entries`` (one token each) spends in each class of kernels
+        (``ops.KERNEL_CLASSES``), and in all of them together under "step": for each class a
+        graph of the step with only that class's kernels launched is captured and replayed
+        ``repeats`` times between two events.  What the runs compute means nothing (the kernels
+        of the other classes did not run) and nothing of it is kept: the requests hold what
+        they held before.  The reference's per-op timing harness is
+        `src/app/cli/tools/bench/ops.zig:516-543`."""
+        from .. import ops
+        if not self.use_graphs:
+            raise StepError("class_times needs a model whose decode steps replay as a graph")
+        if not entries or any(len(e.tokens) != 1 for e in entries):
+            raise StepError("class_times: every entry brings one token")
+        _, wanted_len = self._check_entries(entries)
+        if not self.cache.can_reserve(wanted_len):
+            raise CacheFull("CacheFull: the step needs more pages or request slots than are free")
+        added = self._reserve(wanted_len)
+        out: Dict[str, float] = {}
+        try:
+            ctx = self._build_context(entries, bucket_pages=True)
+            self.model.forward(ctx, self.views)           # settles every work buffer's size
+            stream = torch.cuda.current_stream(self.device)
+            for cls in ops.KERNEL_CLASSES + ("step",):
+                only = ops.KERNEL_CLASSES if cls == "step" else (cls,)
+                n0 = ops.launch_count()
+                with ops.only_classes(only):
+                    self.model.forward(ctx, self.views)
+                if ops.launch_count() == n0:              # the step has no kernel of this class
+                    out[cls] = 0.0
+                    continue
+                stream.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with ops.only_classes(only):
+                    with torch.cuda.graph(graph):
+                        self.model.forward(ctx, self.views)
+                graph.replay()
+                before = torch.cuda.Event(enable_timing=True)
+                after = torch.cuda.Event(enable_timing=True)
+                before.record()
+                for _ in range(repeats):
+                    graph.replay()
+                after.record()
+                after.synchronize()
+                out[cls] = before.elapsed_time(after) * 1e-3 / repeats
+                del graph
+        finally:
+            self._roll_back(wanted_len, added)
+        return out
+
     def _generations(self) -> tuple:
         from .. import ops
         return (self._scratch.generation, ops.workspace_generation(), self._meta_generation)

@@ -42,9 +42,15 @@ def build_model(spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype, device
 def load_model(model_dir: str, dtype="bfloat16", device="cuda:0"):
     """(typed configuration, bound model) of a folder with config.json and model.safetensors;
     the architecture is chosen by config.json."""
+    import os
     config = load_config(model_dir)
     spec = config.model_spec()
     ctx = BuildContext(parse_dtype(dtype), torch.device(device))
+    # kernel plans measured at this model's own widths (``bench-ops --tune`` writes them)
+    from .. import ops
+    plans = os.path.join(model_dir, ops.PLAN_FILE)
+    if os.path.exists(plans):
+        ops.load_plans(plans)
     model = DecoderModel(spec, ctx)
     tensors = load_tensors(model_dir, model.declare())
     model.bind(tensors)

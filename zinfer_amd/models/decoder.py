@@ -114,10 +114,11 @@ class DecoderModel:
             rows = step.scratch("want_rows", (n_rows, s.hidden_size), torch.float32)
             ops.gather_rows(x, step.want_rows, rows)
         make = lambda: step.scratch("final_normed", (n_rows, s.hidden_size), self.ctx.act_dtype)
-        normed = self.final_norm.deferred(rows, make, left)
-        if normed is None:
-            normed = self.final_norm.forward(rows, make())
-        self.head.forward(normed, logits)
-        if s.logit_scale != 1.0 or s.logit_softcap is not None:
-            ops.scale_cap(logits, float(s.logit_scale), float(s.logit_softcap or 0.0))
+        with ops.kernel_class("head_sampling"):      # what a per-class measurement counts these as
+            normed = self.final_norm.deferred(rows, make, left)
+            if normed is None:
+                normed = self.final_norm.forward(rows, make())
+            self.head.forward(normed, logits)
+            if s.logit_scale != 1.0 or s.logit_softcap is not None:
+                ops.scale_cap(logits, float(s.logit_scale), float(s.logit_softcap or 0.0))
         return logits

@@ -61,7 +61,76 @@ def _i32(t: torch.Tensor, what: str) -> None:
         raise KernelUnavailable(f"{what} must be int32, is {t.dtype}")
 
 
+# ------------------------------------------------------------------------- kernel classes
+# Every launcher belongs to a class of a step's work; the per-class benchmark
+# (``Engine.class_times``, the reference's per-op harness is `src/app/cli/tools/bench/
+# ops.zig:516-543`) runs a step with only one class's kernels launched, the others left out.
+# The outputs of such a run mean nothing; only its time does.
+KERNEL_CLASSES = ("products", "attention", "norm_rope_write", "head_sampling", "other")
+_class_filter = None        # None: everything launches; else the set of classes that do
+_class_override = None      # a caller's label for the launches inside it (the head's product)
+_launch_count = 0           # launcher calls that went through
+
+
+def launch_count() -> int:
+    return _launch_count
+
+
+class only_classes:
+    """Within this context only kernels of ``classes`` are launched."""
+
+    def __init__(self, classes):
+        unknown = set(classes) - set(KERNEL_CLASSES)
+        if unknown:
+            raise KernelUnavailable(f"unknown kernel classes {sorted(unknown)}")
+        self.classes = frozenset(classes)
+
+    def __enter__(self):
+        global _class_filter
+        self._before, _class_filter = _class_filter, self.classes
+
+    def __exit__(self, *exc):
+        global _class_filter
+        _class_filter = self._before
+
+
+class kernel_class:
+    """Launches inside this context count as ``name`` whatever their launcher's own class."""
+
+    def __init__(self, name: str):
+        self.name = name
+
+    def __enter__(self):
+        global _class_override
+        self._before, _class_override = _class_override, self.name
+
+    def __exit__(self, *exc):
+        global _class_override
+        _class_override = self._before
+
+
+def _left_out(cls: str) -> bool:
+    return _class_filter is not None and (_class_override or cls) not in _class_filter
+
+
+def _launches(cls: str):
+    """Marks a launcher with its class; under ``only_classes`` a launcher of another class
+    returns without launching."""
+    def deco(fn):
+        @functools.wraps(fn)
+        def launcher(*args, **kwargs):
+            global _launch_count
+            if _class_filter is not None and (_class_override or cls) not in _class_filter:
+                return None
+            _launch_count += 1
+            return fn(*args, **kwargs)
+        launcher.kernel_class = cls
+        return launcher
+    return deco
+
+
 # ------------------------------------------------------------------------- elementwise
+@_launches("other")
 def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
     """out[t, :] = table[ids[t], :] widened to float32, times ``scale``."""
     _need_gpu(table, ids, out)
@@ -75,6 +144,7 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: floa
                         ctypes.c_float(scale), _stream()), "embed")
 
 
+@_launches("head_sampling")
 def scale_cap(x: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> None:
     """In place on float32: x = x * scale, then with cap > 0: x = cap * tanh(x / cap)."""
     _need_gpu(x)
@@ -85,6 +155,7 @@ def scale_cap(x: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> None:
                             ctypes.c_float(cap), _stream()), "scale_cap")
 
 
+@_launches("norm_rope_write")
 def rmsnorm(x: torch.Tensor, gain: torch.Tensor, eps: float, out: torch.Tensor) -> None:
     """out = x * gain / sqrt(mean(x^2) + eps) over the last axis; x and gain float32."""
     _need_gpu(x, gain, out)
@@ -98,6 +169,7 @@ def rmsnorm(x: torch.Tensor, gain: torch.Tensor, eps: float, out: torch.Tensor) 
                           _stream()), "rmsnorm")
 
 
+@_launches("norm_rope_write")
 def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, cos, sin, positions, slot_mapping, k_pool,
                           v_pool, q_out, n_heads, n_kv_heads, head_dim, page_size) -> None:
     """Per token and head of ``qkv`` [T, (nH + 2 nKV) hd]: optional RMSNorm of q and k heads
@@ -154,6 +226,7 @@ def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, cos, sin, positions, slot_ma
         _stream()), "qk_norm_rope_kv_write")
 
 
+@_launches("norm_rope_write")
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     """out[t, j] = silu(gate_up[t, j]) * gate_up[t, I + j]."""
     _need_gpu(gate_up, out)
@@ -164,6 +237,7 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     _check(lib.zf_swiglu(_ptr(gate_up), _ptr(out), _dt(out), T, I, _stream()), "swiglu")
 
 
+@_launches("other")
 def cast(src: torch.Tensor, out: torch.Tensor) -> None:
     """out = src in the other storage type (bfloat16 <-> float32), element by element."""
     _need_gpu(src, out)
@@ -175,6 +249,7 @@ def cast(src: torch.Tensor, out: torch.Tensor) -> None:
                        _stream()), "cast")
 
 
+@_launches("other")
 def poison_pages(pool: torch.Tensor, pages: torch.Tensor) -> None:
     """pool[:, pages, :] = NaN: ``pool`` [runs, pages, row] float32 or bfloat16, ``pages`` int32."""
     _need_gpu(pool, pages)
@@ -187,6 +262,7 @@ def poison_pages(pool: torch.Tensor, pages: torch.Tensor) -> None:
                                _stream()), "poison_pages")
 
 
+@_launches("head_sampling")
 def gather_rows(x: torch.Tensor, idx: torch.Tensor, out: torch.Tensor) -> None:
     _need_gpu(x, idx, out)
     _i32(idx, "idx")
@@ -197,6 +273,7 @@ def gather_rows(x: torch.Tensor, idx: torch.Tensor, out: torch.Tensor) -> None:
     _check(lib.zf_gather_rows(_ptr(x), _ptr(idx), _ptr(out), n, H, _stream()), "gather_rows")
 
 
+@_launches("head_sampling")
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     """out[r] = index of the first maximum of logits[r, :]."""
     _need_gpu(logits, out)
@@ -212,6 +289,7 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
 ARGMAX_NO_ALLOC_MAX_PARTIALS = 32768    # ZF_ARGMAX_NO_ALLOC_MAX_PARTIALS in zf_no_alloc.h
 
 
+@_launches("head_sampling")
 def argmax_no_alloc(logits: torch.Tensor, out: torch.Tensor) -> None:
     """``argmax`` for callers that cannot allocate: the partial results live in a fixed device
     array of the library (shared by all calls on a GPU: overlapping calls race), so at most
@@ -228,6 +306,7 @@ def argmax_no_alloc(logits: torch.Tensor, out: torch.Tensor) -> None:
     _check(lib.zf_argmax_no_alloc(_ptr(logits), _ptr(out), n, V, _stream()), "argmax_no_alloc")
 
 
+@_launches("other")
 def advance_decode(token_ids: torch.Tensor, positions: torch.Tensor, ctx_len: torch.Tensor,
                    sampled: torch.Tensor, slot_mapping: torch.Tensor, block_table: torch.Tensor,
                    page_size: int, advance: bool) -> None:
@@ -252,6 +331,7 @@ def advance_decode(token_ids: torch.Tensor, positions: torch.Tensor, ctx_len: to
            "advance_decode")
 
 
+@_launches("other")
 def randinit(out: torch.Tensor, key: int, start: int, kind: str, std: float = 0.02) -> None:
     """out[i] = element ``start + i`` of the random tensor with ``key``
     (`weights/counter_rng.py`: 'normal' = N(0, std), 'gain' = 1 + U(-0.1, 0.1), 'zeros')."""
@@ -263,6 +343,43 @@ def randinit(out: torch.Tensor, key: int, start: int, kind: str, std: float = 0.
     _check(lib.zf_randinit(_ptr(out), _dt(out), ctypes.c_ulonglong(key & ((1 << 64) - 1)),
                            ctypes.c_ulonglong(start), ctypes.c_ulonglong(out.numel()),
                            KIND[kind], ctypes.c_double(std), _stream()), "randinit")
+
+
+@_launches("other")
+def stream_read(buf: torch.Tensor, sink: torch.Tensor, workgroups: int = 2048) -> None:
+    """Reads ``buf`` once (16-byte non-temporal loads, 8 in flight a lane) and xors it into
+    ``sink`` (int32, one word per workgroup): the read stream the weight-streaming kernels are
+    measured against (``measure_read_bandwidth``)."""
+    _need_gpu(buf, sink)
+    _i32(sink, "sink")
+    nbytes = buf.numel() * buf.element_size()
+    if nbytes % 16 != 0 or sink.numel() < workgroups or not 1 <= workgroups <= 65536:
+        raise KernelUnavailable("stream_read: a buffer of a multiple of 16 bytes and a sink of "
+                                "one int32 per workgroup (1 to 65536)")
+    lib = build.load("elementwise")
+    _check(lib.zf_stream_read(_ptr(buf), ctypes.c_longlong(nbytes), _ptr(sink), int(workgroups),
+                              _stream()), "stream_read")
+
+
+def measure_read_bandwidth(device, nbytes: int = 2 << 30, repeats: int = 3) -> float:
+    """Bytes a second of the best of ``repeats`` passes of ``stream_read`` over a buffer of
+    ``nbytes`` (far more than the last-level cache holds, so it comes from HBM), each pass
+    timed by a pair of events; the best of 256 to 4096 workgroups."""
+    buf = torch.empty((nbytes // 4,), dtype=torch.int32, device=device)
+    buf.zero_()
+    sink = torch.zeros((4096,), dtype=torch.int32, device=device)
+    best = 0.0
+    for wgs in (256, 512, 768, 1024, 2048, 4096):
+        stream_read(buf, sink, wgs)                       # warm-up
+        for _ in range(repeats):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            stream_read(buf, sink, wgs)
+            b.record()
+            b.synchronize()
+            best = max(best, nbytes / (a.elapsed_time(b) * 1e-3))
+    del buf
+    return best
 
 
 # ------------------------------------------------------------------------- work buffers
@@ -357,13 +474,81 @@ def _measured_plans() -> dict:
     return _measured
 
 
+PLAN_FILE = "kernel_plans.json"     # a model folder may bring plans measured at its own widths
+PLAN_BUCKETS = (17, 24, 32, 48, 64)
+
+
+def plan_bucket(M: int) -> int:
+    """The bucket of a number of tokens in 17..64: a plan is kept per bucket, not per M."""
+    return 17 if M <= 20 else 24 if M <= 28 else 32 if M <= 32 else 48 if M <= 56 else 64
+
+
+def check_plans(plans: dict) -> None:
+    """Raises ``KernelUnavailable`` unless every entry of a plan table names a configuration
+    the launchers accept (what ``load_plans`` takes, and what the tuner writes)."""
+    def bad(why):
+        raise KernelUnavailable(f"kernel plans: {why}")
+    for key, entry in plans.get("plans", {}).items():
+        shape, _, kind = key.partition(":")
+        try:
+            N, K = (int(x) for x in shape.split("x"))
+        except ValueError:
+            bad(f"{key!r} is not 'NxK' or 'NxK:swiglu'")
+        if kind not in ("", "swiglu"):
+            bad(f"{key!r}: unknown kind {kind!r}")
+        for bucket, plan in entry.items():
+            M = int(bucket)
+            if M not in PLAN_BUCKETS:
+                bad(f"{key}: bucket {bucket} is none of {PLAN_BUCKETS}")
+            if plan[0] == "mid" and len(plan) == 2:
+                # k-tiles of 256 (up to 32 tokens) or 128, dealt over the workgroups along K
+                ks, tk = int(plan[1]), (256 if M <= 32 else 128)
+                ok = K % tk == 0 and 1 <= ks <= K // tk and N % 16 == 0
+            elif plan[0] == "skinny" and len(plan) == 3:
+                rg, ks = int(plan[1]), int(plan[2])
+                ok = rg in (1, 2, 4) and N % (16 * rg) == 0 and 1 <= ks <= 16 and K % 64 == 0
+            else:
+                ok = False
+            if ok and kind == "swiglu":
+                ok = plan[-1] == 1 and (plan[0] == "mid" or plan[1] >= 2) and N % 32 == 0
+            if not ok:
+                bad(f"{key} at {bucket} tokens: {plan} is no plan the kernels take")
+    for key, plan in plans.get("decode_acc", {}).items():
+        if key == "_":
+            continue
+        N, K = (int(x) for x in key.split("x"))
+        if plan is not None and not (
+                len(plan) == 3 and plan[0] == "skinny" and plan[1] in (1, 2, 4)
+                and N % (16 * plan[1]) == 0 and 2 <= plan[2] <= 16 and N <= 8192 and K % 64 == 0):
+            bad(f"decode_acc {key}: {plan} is no plan the kernels take")
+
+
+def load_plans(path: str) -> int:
+    """Merges a plan file (``bench-ops --tune`` writes one) over the built-in table: its
+    entries win for their widths.  Returns the number of entries taken."""
+    import json
+    with open(path, "r", encoding="utf-8") as f:
+        plans = json.load(f)
+    check_plans(plans)
+    table = _measured_plans()
+    n = 0
+    for key, entry in plans.get("plans", {}).items():
+        table["plans"][key] = {str(b): list(p) for b, p in entry.items()}
+        n += 1
+    for key, plan in plans.get("decode_acc", {}).items():
+        if key != "_":
+            table["decode_acc"][key] = None if plan is None else list(plan)
+            n += 1
+    return n
+
+
 def _small_plan(M: int, N: int, K: int, w_tiled: bool, swiglu: bool = False):
     """Which kernel takes a product of 17 to 128 tokens (None: the tiled kernels):
     ('mid', workgroups along K) or ('skinny', row groups per workgroup, workgroups along K).
     The widths of the served models have measured entries in ``plans_mi355x.json``; other
     widths follow the rules of ``_mid_plan`` and ``_skinny_plan``."""
     if w_tiled and 16 < M <= SKINNY_MAX_M:
-        bucket = 17 if M <= 20 else 24 if M <= 28 else 32 if M <= 32 else 48 if M <= 56 else 64
+        bucket = plan_bucket(M)
         entry = _measured_plans()["plans"].get(f"{N}x{K}" + (":swiglu" if swiglu else ""))
         if entry is not None:
             # a width measured at fewer numbers of tokens: the nearest one on the same side of
@@ -532,6 +717,7 @@ def pretile_weight(w: torch.Tensor) -> torch.Tensor:
     return t.view(N, K)
 
 
+@_launches("products")
 def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
          w_tiled: bool = False, tile_variant: Optional[int] = None) -> None:
     """out = a w^T (w is [N, K]); with ``accumulate`` out += a w^T, in 32-bit.  ``w_tiled``:
@@ -619,9 +805,15 @@ def gemm_partials(a: torch.Tensor, w: torch.Tensor, ksplit: int) -> torch.Tensor
         raise KernelUnavailable("gemm_partials: not a product that gemm_partials_plan covers")
     ws = _workspace("gemm_splitk", ksplit * M * N, torch.float32, a.device)
     lib = build.load("gemm")
-    _check(lib.zf_gemm_bf16_mid_partials(_ptr(a), _ptr(w), _ptr(ws), M, N, K, ksplit, _stream()),
-           "gemm_partials")
+    if not _left_out("products"):
+        global _launch_count
+        _launch_count += 1
+        _check(lib.zf_gemm_bf16_mid_partials(_ptr(a), _ptr(w), _ptr(ws), M, N, K, ksplit,
+                                             _stream()), "gemm_partials")
     return ws[:ksplit * M * N].view(ksplit, M, N)
+
+
+gemm_partials.kernel_class = "products"     # (it hands its work buffer on even when left out)
 
 
 def norm_gemm_plan(M: int, N: int, K: int, w: torch.Tensor, w_tiled: bool):
@@ -635,6 +827,7 @@ def norm_gemm_plan(M: int, N: int, K: int, w: torch.Tensor, w_tiled: bool):
     return rg if ks == 1 else None
 
 
+@_launches("products")
 def norm_gemm(x: torch.Tensor, gain: torch.Tensor, eps: float, w: torch.Tensor,
               out: torch.Tensor, swiglu: bool = False) -> None:
     """out = rmsnorm(x, gain, eps) w^T with the norm folded into the weight-streaming product
@@ -676,6 +869,7 @@ def sum_norm_plan(M: int, N: int, K: int, w: torch.Tensor, w_tiled: bool):
     return ("tile", ks) if ks >= 2 else None
 
 
+@_launches("products")
 def gemm_sum_norm(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, gain: torch.Tensor,
                   eps: float, normed: torch.Tensor) -> None:
     """residual += a w^T in 32-bit (``w`` pre-tiled) and normed = bfloat16(rmsnorm(residual,
@@ -717,6 +911,7 @@ def norm_emit_plan(M: int, N: int, K: int, w: torch.Tensor, w_tiled: bool):
     return rg if (ks == 1 and rg <= 2) else None
 
 
+@_launches("products")
 def gemm_emit(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, gain: torch.Tensor,
               xg: torch.Tensor, sq: torch.Tensor) -> None:
     """residual += a w^T in 32-bit (``w`` pre-tiled) and, for the RMSNorm that reads the sum
@@ -739,6 +934,7 @@ def gemm_emit(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, gain: to
                                         _ptr(sq), M, N, K, rg, _stream()), "gemm_emit")
 
 
+@_launches("products")
 def gemm_given(xg: torch.Tensor, sq: torch.Tensor, eps: float, w: torch.Tensor,
                out: torch.Tensor, swiglu: bool = False) -> None:
     """out = rmsnorm(x) w^T from what ``gemm_emit`` left of x: xg = bfloat16(x * gain) and the
@@ -778,6 +974,7 @@ def can_fuse_swiglu(w: torch.Tensor) -> bool:
     return w.is_cuda and w.dtype == torch.bfloat16 and w.shape[0] % 64 == 0 and w.shape[1] % 8 == 0
 
 
+@_launches("products")
 def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bool = False,
                 tile_variant: Optional[int] = None) -> None:
     """out[M, I] = silu(a Wg^T) * (a Wu^T) as bfloat16, with ``w`` [2 I, K] from
@@ -840,6 +1037,7 @@ def mfma_attention_covers(dtype, n_heads, n_kv_heads, head_dim, page_size) -> bo
 FUSED_DECODE_MAX_SEQS = 32
 
 
+@_launches("attention")
 def decode_attention_fused(qkv, q_gain, k_gain, eps, cos, sin, positions, slot_mapping, k_pool,
                            v_pool, block_table, q_start, ctx_len, out, scale, window, n_heads,
                            n_kv_heads, head_dim, page_size, max_ctx_len) -> None:
@@ -905,6 +1103,7 @@ def _prefill_key_split(n_query_tiles: int, n_kv_heads: int, max_ctx_len: int):
     return (keys, splits) if splits >= 2 else None
 
 
+@_launches("attention")
 def paged_attention(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index, out, scale,
                     window, n_heads, n_kv_heads, head_dim, page_size, max_q_len,
                     max_ctx_len, n_single=None, n_query_tiles=None, q_tile_map=None,
@@ -999,6 +1198,7 @@ SAMPLE_ROW_DTYPE = [("temperature", "<f4"), ("top_p", "<f4"), ("min_p", "<f4"), 
                     ("u", "<f8")]
 
 
+@_launches("head_sampling")
 def apply_penalties(logits, rows, tokens, counts, params) -> None:
     """In place, for every triple (rows[i], tokens[i], counts[i]): the repetition, presence
     and frequency penalties of ``params[row] = (repetition, presence, frequency)``."""
@@ -1014,6 +1214,7 @@ def apply_penalties(logits, rows, tokens, counts, params) -> None:
                                   _ptr(params), n, V, _stream()), "apply_penalties")
 
 
+@_launches("head_sampling")
 def sample_topk(logits: torch.Tensor, params: torch.Tensor, out: torch.Tensor) -> None:
     """out[r] = a token of row r drawn as the reference's sampler draws it: the top_k
     (1..1024) largest logits, temperature, min-p, top-p, and the uniform number u of the
