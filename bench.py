@@ -342,7 +342,7 @@ def run_long_context(llm, cfg, elem: int, context: int, batches, steps: int, see
     end at ``context``."""
     out = {}
     for b in batches:
-        warm = 8
+        warm = 16
         prompt_len = context - steps - warm - b * ((context + 8191) // 8192) - 8
         dt, mean_ctx = run_decode(llm, cfg, b, prompt_len, steps, warm, seed + b)
         out[f"decode_b{b}"] = round(b * steps / dt, 1)
@@ -374,7 +374,7 @@ def main_long_context(args) -> int:
     hb = 8 if 8 in batches else max(batches)      # the batch of the headline
     line = {"metric": f"decode tok/s at context {context}, {SHAPE_NAMES[shape]} shape, batch {hb}",
             "value": res[f"decode_b{hb}"], "unit": "tokens/s", "n_gpus": 1, "steps": steps,
-            "warmup": 8, "ms_per_step": res[f"decode_b{hb}_ms"], "higher_is_better": True,
+            "warmup": 16, "ms_per_step": res[f"decode_b{hb}_ms"], "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
             "config": config_of(cfg, shape, global_batch=hb, seq_len=context,
@@ -455,6 +455,7 @@ def main_decode(args) -> int:
                     max_step_tokens=step_tokens, multi_step=args.multi_step)
     cfg = llm.config
     build_s = time.perf_counter() - t_build
+    llm.engine.capture_runs = not args.no_run_graphs
     elem = 2 if args.dtype == "bfloat16" else 4
     peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
 
@@ -468,8 +469,7 @@ def main_decode(args) -> int:
     if not args.no_points:
         for b in (1, 64):
             k = max(16, args.steps // 4)
-            d, ctx = run_decode(llm, cfg, b, args.prompt_len, k, min(args.warmup, 4),
-                                args.seed + 3 + b)
+            d, ctx = run_decode(llm, cfg, b, args.prompt_len, k, args.warmup, args.seed + 3 + b)
             points[f"decode_b{b}"] = round(b * k / d, 1)
             points[f"decode_b{b}_hbm_frac"] = decode_roofline(cfg, elem, b, ctx, d / k)["frac"]
         for T in (512, 8192):
@@ -535,7 +535,7 @@ def main() -> int:
     ap.add_argument("--multi-step", type=int, default=8,
                     help="most decode steps in a row on the device without the host between")
     ap.add_argument("--steps", type=int, default=128)
-    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=2048)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
@@ -562,6 +562,8 @@ def main() -> int:
     ap.add_argument("--batches", default="1,8,64",
                     help="long-context: the batch sizes decoded at (the pool holds the largest)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-run-graphs", action="store_true",
+                    help="decode steps in a row replay one graph per step instead of one for the run")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py runs on one GPU only (asked for {args.gpus}): this engine has no "

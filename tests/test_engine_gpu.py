@@ -453,7 +453,10 @@ def test_decode_steps_in_a_row_equal_single_steps(dtype, tmp_path_factory):
         lg = eng.step([StepEntry(r, t, [len(t) - 1]) for r, t in reqs.items()])
         cur = eng.argmax(lg)
     rng = np.random.default_rng(5)
-    for n_steps, sampled in ((19, False), (1, False), (9, True), (2, True)):
+    # (a run of steps is captured as one graph the second time its shape comes: the repeats
+    # below go through the first, eager, pass, the capture and a replay of it)
+    for n_steps, sampled in ((19, False), (1, False), (9, True), (2, True), (5, False), (5, False),
+                             (5, False), (4, True), (4, True), (4, True)):
         records = None
         if sampled:
             records = np.zeros((n_steps, len(reqs)), dtype=ops.SAMPLE_ROW_DTYPE)
@@ -474,7 +477,7 @@ def test_decode_steps_in_a_row_equal_single_steps(dtype, tmp_path_factory):
     # refused before anything runs: too many steps for the pages that are free
     free = a.cache.num_free_pages()
     too_many = 4 * free[0] + 32         # four requests, pages of 16: more pages than are free
-    assert too_many < 450               # still inside the position table
+    assert too_many < 400               # still inside the position table
     with pytest.raises(Exception, match="CacheFull"):
         a.decode_steps([StepEntry(r, [1], [0]) for r in reqs], too_many)
     assert a.cache.num_free_pages() == free

@@ -225,13 +225,13 @@ def test_a_model_folders_plans_are_checked_and_override_the_table(tmp_path, monk
     import json
     monkeypatch.setattr(ops, "_measured", copy.deepcopy(ops._measured_plans()))
     before = ops._small_plan(40, 2048, 1024, True)
-    good = {"plans": {"2048x1024": {"48": ["skinny", 1, 2], "17": ["skinny", 2, 1]}},
+    good = {"plans": {"2048x1024": {"48": ["skinny", 2, 4], "17": ["skinny", 2, 1]}},
             "decode_acc": {"2048x6144": ["skinny", 2, 3], "_": "a remark"}}
     p = tmp_path / ops.PLAN_FILE
     p.write_text(json.dumps(good))
     assert ops.load_plans(str(p)) == 2
-    assert ops._small_plan(40, 2048, 1024, True) == ("skinny", 1, 2) != before
-    assert ops._small_plan(64, 2048, 1024, True) == ("skinny", 1, 2)     # the nearest bucket above 32
+    assert ops._small_plan(40, 2048, 1024, True) == ("skinny", 2, 4) != before
+    assert ops._small_plan(64, 2048, 1024, True) == ("skinny", 2, 4)     # the nearest bucket above 32
     assert ops._small_plan(20, 2048, 1024, True) == ("skinny", 2, 1)
     assert ops._decode_acc_plan(8, 2048, 6144) == ("skinny", 2, 3)
     for bad in ({"plans": {"2048x1024": {"48": ["skinny", 3, 1]}}},

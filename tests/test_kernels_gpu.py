@@ -654,6 +654,64 @@ def test_qk_norm_rope_kv_write(dtype, nH, nKV, hd, page_size, use_norm, use_rope
     assert rel_err(got_inplace, want_inplace) <= tol(dtype)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nH,nKV,hd,page_size", [(32, 8, 128, 16), (6, 2, 64, 32), (3, 1, 48, 16),
+                                                 (8, 2, 32, 8), (4, 4, 256, 16)])
+def test_qk_norm_rope_kv_write_of_hundreds_of_tokens(dtype, nH, nKV, hd, page_size):
+    """From 256 tokens on a workgroup takes four tokens in a row and stores the values of four
+    consecutive rows at once: portions that start at a page's edge, in the middle of a group of
+    four rows and one row before a page's end, single tokens between them, slots in no order
+    at all, and a number of tokens that is no multiple of four."""
+    from zinfer_amd.parts.position import rotary_tables
+    ops, eps = _ops(), 1e-6
+    width = (nH + 2 * nKV) * hd
+    runs = [(0, 130), (3, 57), (-1, 70), (1, 1), (2, 2), (0, 4), (5, 3)]   # (start row in a fresh page, tokens)
+    slots, positions, page = [], [], 0
+    for start, n in runs:
+        first = page * page_size + (start % page_size)
+        slots += list(range(first, first + n))
+        positions += list(range(7 + start % page_size, 7 + start % page_size + n))
+        page = (first + n + page_size - 1) // page_size + 1
+    g = torch.Generator().manual_seed(3)
+    extra = (torch.randperm(8 * page_size, generator=g)[:40] + page * page_size).tolist()
+    slots += extra
+    positions += [int(x) % 300 for x in extra]
+    page += 9
+    T = len(slots)
+    assert T >= 256 and T % 4 != 0
+    qkv = _rand((T, width), dtype, 12)
+    qg, kg = (1 + 0.1 * _rand((hd,), torch.float32, 13)), (1 + 0.1 * _rand((hd,), torch.float32, 14))
+    cos, sin = rotary_tables(hd, 10000.0, 400)
+    slots_t = torch.tensor(slots, dtype=torch.int32)
+    pos_t = torch.tensor(positions, dtype=torch.int32)
+    row = nKV * page_size * hd
+    pools = [torch.zeros((page, row), dtype=dtype) for _ in range(4)]
+    q_want = torch.empty((T, nH * hd), dtype=dtype)
+    ref.qk_norm_rope_kv_write(qkv.clone(), qg, kg, eps, cos, sin, pos_t, slots_t, pools[0],
+                              pools[1], q_want, nH, nKV, hd, page_size)
+    q_got = torch.full((T, nH * hd), float("nan"), dtype=dtype, device=DEV)
+    kp, vp = pools[2].to(DEV), pools[3].to(DEV)
+    ops.qk_norm_rope_kv_write(qkv.to(DEV), qg.to(DEV), kg.to(DEV), eps, cos.to(DEV), sin.to(DEV),
+                              pos_t.to(DEV), slots_t.to(DEV), kp, vp, q_got, nH, nKV, hd, page_size)
+    assert rel_err(q_got, q_want) <= tol(dtype)
+    if ops.mfma_attention_covers(dtype, nH, nKV, hd, page_size):
+        pools[0] = ref.tile_k_pool(pools[0], nKV, page_size, hd)
+        pools[1] = ref.tile_v_pool(pools[1], nKV, page_size, hd)
+    assert rel_err(kp, pools[0]) <= tol(dtype)
+    assert torch.equal(vp.cpu(), pools[1])
+    # the same tokens one at a time give the same bits (the kernel's other path)
+    q_one = torch.empty_like(q_got)
+    kp1, vp1 = pools[2].to(DEV), pools[3].to(DEV)
+    for lo in range(0, T, 100):
+        hi = min(T, lo + 100)
+        ops.qk_norm_rope_kv_write(qkv[lo:hi].to(DEV), qg.to(DEV), kg.to(DEV), eps, cos.to(DEV),
+                                  sin.to(DEV), pos_t[lo:hi].to(DEV), slots_t[lo:hi].to(DEV), kp1,
+                                  vp1, q_one[lo:hi], nH, nKV, hd, page_size)
+    bits = lambda t: t.view(torch.int16 if dtype == torch.bfloat16 else torch.int32)
+    assert torch.equal(bits(q_one), bits(q_got)) and torch.equal(bits(kp1), bits(kp))
+    assert torch.equal(bits(vp1), bits(vp))
+
+
 @pytest.mark.parametrize("nH,nKV,hd,page_size,window,use_norm,use_rope", [
     (32, 8, 128, 16, 0, True, True), (8, 2, 32, 16, 0, True, True), (6, 6, 64, 32, 0, True, False),
     (16, 1, 64, 16, 37, False, True), (9, 3, 256, 16, 0, True, True), (10, 2, 128, 48, 300, True, True),
@@ -676,7 +734,7 @@ def test_decode_attention_fused_equals_the_two_kernels(nH, nKV, hd, page_size, w
                                [1, 2, 16, 17, 100, 255, 256])
 
 
-@pytest.mark.parametrize("M,nH,nKV,hd,page_size,H", [(64, 32, 8, 128, 16, 4096), (40, 8, 2, 64, 16, 2048),
+@pytest.mark.parametrize("M,nH,nKV,hd,page_size,H", [(64, 32, 8, 128, 16, 4096), (40, 8, 2, 64, 16, 2560), (60, 8, 2, 64, 16, 2048),
                                                      (33, 4, 4, 128, 32, 4096), (128, 16, 2, 128, 16, 5120)])
 def test_qk_norm_rope_kv_write_from_a_split_products_partials(M, nH, nKV, hd, page_size, H):
     """17 to 128 tokens: the q/k/v product runs split along K.  Its partials handed to the

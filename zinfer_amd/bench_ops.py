@@ -212,7 +212,8 @@ def tune(cfg: dict, dev: str, log=print) -> dict:
         if not (N % 64 == 0 and K % 64 == 0):
             log(f"{name}: {N} x {K} does not pre-tile, no plans apply")
             continue
-        copies = max(3, min(16, int(1.5e9 // (N * K * 2))))
+        # more copies in turn than the 256 MB last-level cache holds: the weights come from HBM
+        copies = max(3, min(96, -(-600_000_000 // (N * K * 2))))
         ws = [ops.pretile_weight((torch.randn(N, K, device=dev) * 0.02).to(torch.bfloat16))
               for _ in range(copies)]
         key = f"{N}x{K}" + (":swiglu" if kind == "swiglu" else "")

@@ -221,6 +221,27 @@ __global__ void qk_norm_rope_kv_write_kernel(
   }
 }
 
+// Four consecutive elements as one 8-byte (bfloat16) or 16-byte (float32) access; the
+// address is a multiple of that size wherever the kernel below uses them (head sizes that
+// are multiples of 8, rows and pools that start on 256-byte boundaries).
+template <typename T> __device__ __forceinline__ void load4(const T* p, float (&x)[4]);
+template <> __device__ __forceinline__ void load4<float>(const float* p, float (&x)[4]) {
+  const float4 v = *(const float4*)p;
+  x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+}
+template <> __device__ __forceinline__ void load4<bf16_t>(const bf16_t* p, float (&x)[4]) {
+  const uint2 v = *(const uint2*)p;
+  x[0] = __uint_as_float(v.x << 16); x[1] = __uint_as_float(v.x & 0xffff0000u);
+  x[2] = __uint_as_float(v.y << 16); x[3] = __uint_as_float(v.y & 0xffff0000u);
+}
+template <typename T> __device__ __forceinline__ void store4(T* p, const float (&x)[4]);
+template <> __device__ __forceinline__ void store4<float>(float* p, const float (&x)[4]) {
+  *(float4*)p = float4{x[0], x[1], x[2], x[3]};
+}
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, const float (&x)[4]) {
+  *(uint2*)p = uint2{pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3])};
+}
+
 // The same for head sizes that are a multiple of 8 (every size in steps of 16 is): a lane
 // takes 4 consecutive elements of the first half of a head and the 4 that pair with them
 // under the rotation, LPH = the next power of two >= hd / 8 lanes work on a head and a wave
@@ -231,99 +252,142 @@ __global__ void qk_norm_rope_kv_write_kernel(
 // that a product split along K left: a lane adds its elements' partials in split order and
 // rounds the sum to bfloat16, as the kernel that only adds partials would have written it, and
 // goes on from there (one launch less; q goes to q_out, k and v into the pools).
-template <typename T, int LPH, bool PART = false>
+template <typename T, int LPH, bool PART = false, int TPB = 1>
 __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_vec_kernel(
     T* __restrict__ qkv, const float* __restrict__ q_gain, const float* __restrict__ k_gain,
     float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int* __restrict__ positions, const int* __restrict__ slot_mapping,
     T* __restrict__ k_pool, T* __restrict__ v_pool, T* __restrict__ q_out, int nH, int nKV,
     int hd, int page_size, int tiled, const float* __restrict__ partials, int ksplit,
-    size_t split_stride) {
+    size_t split_stride, int Tn) {
+  // TPB: a workgroup takes this many tokens in a row, the same lanes the same head of each:
+  // what all of them need from memory is asked for before any arithmetic, and a quarter of
+  // the workgroups are handed out (2048 tokens of 48 heads, one token a workgroup: 33 us for
+  // 50 MB; the kernel waited for one load after the other).
   constexpr int HPW = 64 / LPH;
-  const int t = blockIdx.x;
+  const int t0 = blockIdx.x * TPB;
   const int lane = threadIdx.x % 64, li = lane % LPH;
   // four waves to a workgroup (a quarter of the workgroups to hand out: 2048 tokens of 48
   // heads took 25 us as 24576 workgroups of one wave)
   const int head = (blockIdx.y * 4 + threadIdx.x / 64) * HPW + lane / LPH;
   const int half = hd / 2;
-  const bool active = head < nH + 2 * nKV && 4 * li < half;
-  const int row_width = (nH + 2 * nKV) * hd;
-  T* src = qkv + (size_t)t * row_width + (size_t)min(head, nH + 2 * nKV - 1) * hd;
-  float x0[4] = {0.f, 0.f, 0.f, 0.f}, x1[4] = {0.f, 0.f, 0.f, 0.f};
-  if (PART && active) {
-    const float* p = partials + (size_t)t * row_width +
-                     (size_t)min(head, nH + 2 * nKV - 1) * hd + 4 * li;
-    float4 s0 = float4{0.f, 0.f, 0.f, 0.f}, s1 = s0;
-    for (int k = 0; k < ksplit; ++k) {
-      const float4 a = *(const float4*)(p + (size_t)k * split_stride);
-      const float4 b = *(const float4*)(p + (size_t)k * split_stride + half);
-      s0.x += a.x; s0.y += a.y; s0.z += a.z; s0.w += a.w;
-      s1.x += b.x; s1.y += b.y; s1.z += b.z; s1.w += b.w;
-    }
-    x0[0] = bf16_to_float(float_to_bf16(s0.x)); x0[1] = bf16_to_float(float_to_bf16(s0.y));
-    x0[2] = bf16_to_float(float_to_bf16(s0.z)); x0[3] = bf16_to_float(float_to_bf16(s0.w));
-    x1[0] = bf16_to_float(float_to_bf16(s1.x)); x1[1] = bf16_to_float(float_to_bf16(s1.y));
-    x1[2] = bf16_to_float(float_to_bf16(s1.z)); x1[3] = bf16_to_float(float_to_bf16(s1.w));
-  } else if (active) {
+  const int n_heads = nH + 2 * nKV;
+  const bool active = head < n_heads && 4 * li < half;
+  const int row_width = n_heads * hd;
+  const int hh = min(head, n_heads - 1);
+  const bool is_q = head < nH, is_v = head >= nH + nKV;
+  float x0[TPB][4], x1[TPB][4];
+  int slot[TPB], pos[TPB];
+  bool live[TPB];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {     // consecutive: the compiler makes one load of each
-      x0[e] = load_as_float<T>(src + 4 * li + e);
-      x1[e] = load_as_float<T>(src + half + 4 * li + e);
+  for (int tt = 0; tt < TPB; ++tt) {
+    const int t = min(t0 + tt, Tn - 1);
+    live[tt] = active && t0 + tt < Tn;
+    slot[tt] = slot_mapping ? slot_mapping[t] : 0;
+    pos[tt] = (cos_t && !is_v) ? positions[t] : 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) x0[tt][e] = x1[tt][e] = 0.f;
+    T* src = qkv + (size_t)t * row_width + (size_t)hh * hd;
+    if (PART && live[tt]) {
+      const float* p = partials + (size_t)t * row_width + (size_t)hh * hd + 4 * li;
+      float4 s0 = float4{0.f, 0.f, 0.f, 0.f}, s1 = s0;
+      for (int k = 0; k < ksplit; ++k) {
+        const float4 a = *(const float4*)(p + (size_t)k * split_stride);
+        const float4 b = *(const float4*)(p + (size_t)k * split_stride + half);
+        s0.x += a.x; s0.y += a.y; s0.z += a.z; s0.w += a.w;
+        s1.x += b.x; s1.y += b.y; s1.z += b.z; s1.w += b.w;
+      }
+      x0[tt][0] = bf16_to_float(float_to_bf16(s0.x)); x0[tt][1] = bf16_to_float(float_to_bf16(s0.y));
+      x0[tt][2] = bf16_to_float(float_to_bf16(s0.z)); x0[tt][3] = bf16_to_float(float_to_bf16(s0.w));
+      x1[tt][0] = bf16_to_float(float_to_bf16(s1.x)); x1[tt][1] = bf16_to_float(float_to_bf16(s1.y));
+      x1[tt][2] = bf16_to_float(float_to_bf16(s1.z)); x1[tt][3] = bf16_to_float(float_to_bf16(s1.w));
+    } else if (live[tt]) {
+      load4<T>(src + 4 * li, x0[tt]);
+      load4<T>(src + half + 4 * li, x1[tt]);
     }
   }
-  const bool is_q = head < nH, is_v = head >= nH + nKV;
-  int slot = 0;
-  if (slot_mapping) slot = slot_mapping[t];
-  const int page = slot / page_size, r = slot % page_size;
   if (is_v) {
     if (!active || slot_mapping == nullptr) return;
-    T* blk = v_pool + ((size_t)page * nKV + (head - nH - nKV)) * page_size * hd;
+    const int kvh = head - nH - nKV;
+    if (TPB == 4 && tiled && sizeof(T) == 2 && live[3] && slot[0] % 4 == 0 &&
+        slot[1] == slot[0] + 1 && slot[2] == slot[0] + 2 && slot[3] == slot[0] + 3) {
+      // The tiled pool keeps the rows r .. r + 3 (r % 4 == 0) of a head element side by side
+      // (8 bytes), and a portion's tokens lie in consecutive rows: four tokens' values of an
+      // element go out as one store.  (Rows that follow one another inside a group of 4 are
+      // one request's: another request's rows lie in another page.)
+      const int page = slot[0] / page_size, r = slot[0] % page_size;
+      uint16_t* grp = (uint16_t*)v_pool + ((size_t)page * nKV + kvh) * page_size * hd +
+                      (size_t)(r / 16) * 16 * hd + ((r % 16) / 4) * 64;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int d0 = 4 * li + e, d1 = half + 4 * li + e;
-      if (tiled) {
-        T* grp = blk + (size_t)(r / 16) * 16 * hd + ((r % 16) / 4) * 64 + r % 4;
-        store_from_float<T>(grp + (d0 / 16) * 256 + (d0 % 16) * 4, x0[e]);
-        store_from_float<T>(grp + (d1 / 16) * 256 + (d1 % 16) * 4, x1[e]);
-      } else {
-        store_from_float<T>(blk + (size_t)d0 * page_size + r, x0[e]);
-        store_from_float<T>(blk + (size_t)d1 * page_size + r, x1[e]);
+      for (int e = 0; e < 4; ++e) {
+        const int d0 = 4 * li + e, d1 = half + 4 * li + e;
+        *(uint2*)(grp + (d0 / 16) * 256 + (d0 % 16) * 4) =
+            uint2{pack_bf16x2(x0[0][e], x0[1][e]), pack_bf16x2(x0[2][e], x0[3][e])};
+        *(uint2*)(grp + (d1 / 16) * 256 + (d1 % 16) * 4) =
+            uint2{pack_bf16x2(x1[0][e], x1[1][e]), pack_bf16x2(x1[2][e], x1[3][e])};
+      }
+      return;
+    }
+#pragma unroll
+    for (int tt = 0; tt < TPB; ++tt) {
+      if (!live[tt]) continue;
+      const int page = slot[tt] / page_size, r = slot[tt] % page_size;
+      T* blk = v_pool + ((size_t)page * nKV + kvh) * page_size * hd;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int d0 = 4 * li + e, d1 = half + 4 * li + e;
+        if (tiled) {
+          T* grp = blk + (size_t)(r / 16) * 16 * hd + ((r % 16) / 4) * 64 + r % 4;
+          store_from_float<T>(grp + (d0 / 16) * 256 + (d0 % 16) * 4, x0[tt][e]);
+          store_from_float<T>(grp + (d1 / 16) * 256 + (d1 % 16) * 4, x1[tt][e]);
+        } else {
+          store_from_float<T>(blk + (size_t)d0 * page_size + r, x0[tt][e]);
+          store_from_float<T>(blk + (size_t)d1 * page_size + r, x1[tt][e]);
+        }
       }
     }
     return;
   }
   // query and key heads (lanes of value heads have left: the shuffles below stay inside
   // groups of LPH lanes, which are all of one head)
-  HeadCoef cf;
-  load_head_coef(cf, active ? li : 0, hd, is_q ? q_gain : k_gain, cos_t, sin_t,
-                 cos_t ? positions[t] : 0);
-  head_norm_rotate<LPH>(x0, x1, hd, active, eps, cf);
-  if (!active) return;
-  T* dst0;
-  T* dst1;
-  if (is_q) {
-    T* base = q_out ? q_out + (size_t)t * nH * hd + (size_t)head * hd : src;
-    dst0 = base + 4 * li;
-    dst1 = base + half + 4 * li;
-  } else if (slot_mapping) {
-    T* blk = k_pool + ((size_t)page * nKV + (head - nH)) * page_size * hd;
-    if (tiled) {      // element d of row r: [d / 32][16 * ((d % 32) / 8) + r % 16][d % 8]
-      T* grp = blk + (size_t)(r / 16) * 16 * hd;
-      const int d0 = 4 * li, d1 = half + 4 * li;
-      dst0 = grp + (d0 / 32) * 512 + (((d0 % 32) / 8) * 16 + r % 16) * 8 + d0 % 8;
-      dst1 = grp + (d1 / 32) * 512 + (((d1 % 32) / 8) * 16 + r % 16) * 8 + d1 % 8;
-    } else {
-      dst0 = blk + (size_t)r * hd + 4 * li;
-      dst1 = blk + (size_t)r * hd + half + 4 * li;
-    }
-  } else {
-    dst0 = src + 4 * li;
-    dst1 = src + half + 4 * li;
+  HeadCoef cf[TPB];
+  load_head_coef(cf[0], active ? li : 0, hd, is_q ? q_gain : k_gain, cos_t, sin_t, pos[0]);
+#pragma unroll
+  for (int tt = 1; tt < TPB; ++tt) {
+    cf[tt] = cf[0];
+    load_head_rotation(cf[tt], active ? li : 0, hd, cos_t, sin_t, pos[tt]);
   }
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    store_from_float<T>(dst0 + e, x0[e]);
-    store_from_float<T>(dst1 + e, x1[e]);
+  for (int tt = 0; tt < TPB; ++tt) head_norm_rotate<LPH>(x0[tt], x1[tt], hd, live[tt], eps, cf[tt]);
+#pragma unroll
+  for (int tt = 0; tt < TPB; ++tt) {
+    if (!live[tt]) continue;
+    const int t = t0 + tt;
+    T* src = qkv + (size_t)t * row_width + (size_t)hh * hd;
+    T* dst0;
+    T* dst1;
+    if (is_q) {
+      T* base = q_out ? q_out + (size_t)t * nH * hd + (size_t)head * hd : src;
+      dst0 = base + 4 * li;
+      dst1 = base + half + 4 * li;
+    } else if (slot_mapping) {
+      const int page = slot[tt] / page_size, r = slot[tt] % page_size;
+      T* blk = k_pool + ((size_t)page * nKV + (head - nH)) * page_size * hd;
+      if (tiled) {      // element d of row r: [d / 32][16 * ((d % 32) / 8) + r % 16][d % 8]
+        T* grp = blk + (size_t)(r / 16) * 16 * hd;
+        const int d0 = 4 * li, d1 = half + 4 * li;
+        dst0 = grp + (d0 / 32) * 512 + (((d0 % 32) / 8) * 16 + r % 16) * 8 + d0 % 8;
+        dst1 = grp + (d1 / 32) * 512 + (((d1 % 32) / 8) * 16 + r % 16) * 8 + d1 % 8;
+      } else {
+        dst0 = blk + (size_t)r * hd + 4 * li;
+        dst1 = blk + (size_t)r * hd + half + 4 * li;
+      }
+    } else {
+      dst0 = src + 4 * li;
+      dst1 = src + half + 4 * li;
+    }
+    store4<T>(dst0, x0[tt]);
+    store4<T>(dst1, x1[tt]);
   }
 }
 
@@ -335,12 +399,20 @@ static void launch_qk_vec(T* qkv, const float* q_gain, const float* k_gain, floa
                           const float* partials = nullptr, int ksplit = 0) {
   const int lanes = hd / 8, heads = nH + 2 * nKV;
   const size_t split_stride = (size_t)Tn * heads * hd;
+  // from a few hundred tokens on a workgroup takes four tokens in a row
+  const bool rows4 = !PART && Tn >= 256;
+#define ZF_QKV_T(LPH, TPB)                                                                     \
+  hipLaunchKernelGGL((qk_norm_rope_kv_write_vec_kernel<T, LPH, PART, TPB>),                    \
+                     dim3((Tn + TPB - 1) / TPB, (heads + 256 / LPH - 1) / (256 / LPH)),        \
+                     dim3(256), 0, stream, qkv, q_gain, k_gain, eps, cos_t, sin_t, positions,  \
+                     slot_mapping, k_pool, v_pool, q_out, nH, nKV, hd, page_size, tiled,       \
+                     partials, ksplit, split_stride, Tn)
 #define ZF_QKV(LPH)                                                                            \
-  hipLaunchKernelGGL((qk_norm_rope_kv_write_vec_kernel<T, LPH, PART>),                         \
-                     dim3(Tn, (heads + 256 / LPH - 1) / (256 / LPH)), dim3(256), 0, stream, qkv, \
-                     q_gain, k_gain, eps, cos_t, sin_t, positions, slot_mapping, k_pool,       \
-                     v_pool, q_out, nH, nKV, hd, page_size, tiled, partials, ksplit,           \
-                     split_stride)
+  do {                                                                                         \
+    if constexpr (PART) ZF_QKV_T(LPH, 1);                                                      \
+    else if (rows4) ZF_QKV_T(LPH, 4);                                                          \
+    else ZF_QKV_T(LPH, 1);                                                                     \
+  } while (0)
   if (lanes <= 2) ZF_QKV(2);
   else if (lanes <= 4) ZF_QKV(4);
   else if (lanes <= 8) ZF_QKV(8);
@@ -348,6 +420,7 @@ static void launch_qk_vec(T* qkv, const float* q_gain, const float* k_gain, floa
   else if (lanes <= 32) ZF_QKV(32);
   else ZF_QKV(64);
 #undef ZF_QKV
+#undef ZF_QKV_T
 }
 
 extern "C" int zf_qk_norm_rope_kv_write(void* qkv, int dtype, const float* q_gain,

@@ -56,20 +56,43 @@ __device__ __forceinline__ void load_head_coef(HeadCoef& cf, int li, int hd,
                                                const float* __restrict__ gain,
                                                const float* __restrict__ cos_t,
                                                const float* __restrict__ sin_t, int pos) {
+  // hd % 8 == 0 and 4 li < hd / 2: each group of four is one 16-byte load (as four 4-byte
+  // loads they were two thirds of the load instructions of the kernels that call this)
   const int half = hd / 2;
   cf.has_gain = gain != nullptr;
   cf.has_rotation = cos_t != nullptr;
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    cf.g0[e] = cf.has_gain ? gain[4 * li + e] : 1.f;
-    cf.g1[e] = cf.has_gain ? gain[half + 4 * li + e] : 1.f;
-    cf.c[e] = cf.has_rotation ? cos_t[(size_t)pos * half + 4 * li + e] : 1.f;
-    cf.sn[e] = cf.has_rotation ? sin_t[(size_t)pos * half + 4 * li + e] : 0.f;
+  float4 g0 = float4{1.f, 1.f, 1.f, 1.f}, g1 = g0, c = g0, sn = float4{0.f, 0.f, 0.f, 0.f};
+  if (cf.has_gain) {
+    g0 = *(const float4*)(gain + 4 * li);
+    g1 = *(const float4*)(gain + half + 4 * li);
   }
+  if (cf.has_rotation) {
+    c = *(const float4*)(cos_t + (size_t)pos * half + 4 * li);
+    sn = *(const float4*)(sin_t + (size_t)pos * half + 4 * li);
+  }
+  cf.g0[0] = g0.x; cf.g0[1] = g0.y; cf.g0[2] = g0.z; cf.g0[3] = g0.w;
+  cf.g1[0] = g1.x; cf.g1[1] = g1.y; cf.g1[2] = g1.z; cf.g1[3] = g1.w;
+  cf.c[0] = c.x; cf.c[1] = c.y; cf.c[2] = c.z; cf.c[3] = c.w;
+  cf.sn[0] = sn.x; cf.sn[1] = sn.y; cf.sn[2] = sn.z; cf.sn[3] = sn.w;
+}
+// the same head at another position: the gains stay, cosines and sines are loaded anew
+__device__ __forceinline__ void load_head_rotation(HeadCoef& cf, int li, int hd,
+                                                   const float* __restrict__ cos_t,
+                                                   const float* __restrict__ sin_t, int pos) {
+  if (!cf.has_rotation) return;
+  const int half = hd / 2;
+  const float4 c = *(const float4*)(cos_t + (size_t)pos * half + 4 * li);
+  const float4 sn = *(const float4*)(sin_t + (size_t)pos * half + 4 * li);
+  cf.c[0] = c.x; cf.c[1] = c.y; cf.c[2] = c.z; cf.c[3] = c.w;
+  cf.sn[0] = sn.x; cf.sn[1] = sn.y; cf.sn[2] = sn.z; cf.sn[3] = sn.w;
 }
 template <int LPH>
 __device__ __forceinline__ void head_norm_rotate(float (&x0)[4], float (&x1)[4], int hd,
                                                  bool active, float eps, const HeadCoef& cf) {
+  // every product and sum below is rounded on its own: fused multiply-adds, formed or not as
+  // the code around a call happens to be scheduled, would let two kernels that call this
+  // disagree in the last bit
+#pragma clang fp contract(off)
   if (cf.has_gain) {
     float ss = 0.f;
 #pragma unroll

@@ -64,6 +64,10 @@ class Engine:
             and getattr(model, "graph_safe", False)
         self._graphs: Dict[tuple, tuple] = {}
         self.graph_replays = 0
+        # several decode steps in a row (``decode_steps``) are also recorded as one graph, from
+        # the second time a shape of run comes
+        self.capture_runs = True
+        self._run_shapes: Dict[tuple, int] = {}
         # measurement: when a list, every step appends (tokens, sequences, seconds of host
         # packing, seconds of host launching, event before, event after the step's kernels,
         # whether a request brought more than one token).  Every record holds two events:
@@ -230,19 +234,60 @@ class Engine:
             out = self._scratch.get("decoded", (n_steps, n), torch.int32)
             rec = None
             if records is not None:
-                rec = torch.from_numpy(records.view(np.uint8).reshape(n_steps, -1).copy()) \
-                    .to(self.device)
-            for s in range(n_steps):
-                if s:
-                    for g, tables in enumerate(ctx.kv):
-                        ops.advance_decode(ctx.token_ids, ctx.positions, ctx.ctx_len, out[s - 1],
-                                           tables.slot_mapping, tables.block_table, self.page_size,
-                                           advance=(g == 0))
-                logits = self._forward_graphed(ctx)
-                if rec is None:
-                    ops.argmax(logits, out[s])
-                else:
-                    ops.sample_topk(logits, rec[s], out[s])
+                # at a fixed address, so that a captured run of steps can be replayed
+                rec = self._scratch.get("sample_records", (n_steps, n * 24), torch.uint8)
+                rec.copy_(torch.from_numpy(records.view(np.uint8).reshape(n_steps, -1).copy()),
+                          non_blocking=False)
+
+            def run_steps():
+                for s in range(n_steps):
+                    if s:
+                        for g, tables in enumerate(ctx.kv):
+                            ops.advance_decode(ctx.token_ids, ctx.positions, ctx.ctx_len,
+                                               out[s - 1], tables.slot_mapping,
+                                               tables.block_table, self.page_size,
+                                               advance=(g == 0))
+                    logits = self.model.forward(ctx, self.views) if capturing[0] \
+                        else self._forward_graphed(ctx)
+                    if rec is None:
+                        ops.argmax(logits, out[s])
+                    else:
+                        ops.sample_topk(logits, rec[s], out[s])
+
+            # The whole run of steps as one graph.  A call with a new shape runs step by step
+            # (each step's own graph, the kernels between them launched one by one), which
+            # settles every work buffer.  The second call with that shape does the same and
+            # then records the run once more without running it (some tens of milliseconds,
+            # which a shape that comes only once is not worth); later calls replay that
+            # record, so that nothing is launched between the steps.
+            capturing = [False]
+            key = ("run", n, n_steps, rec is not None, tuple(t.max_pages for t in ctx.kv),
+                   ctx.meta_offset)
+            held = self._graphs.get(key)
+            if n_steps > 1 and held is not None and held[2] == self._generations():
+                self._graphs[key] = self._graphs.pop(key)
+                held[0].replay()
+                self.graph_replays += n_steps
+            else:
+                run_steps()
+                seen = self._run_shapes.get(key, 0)
+                if len(self._run_shapes) > 4 * self.MAX_GRAPHS:
+                    self._run_shapes.clear()
+                self._run_shapes[key] = seen + 1
+                if n_steps > 1 and self.capture_runs and seen >= 1:
+                    torch.cuda.current_stream(self.device).synchronize()
+                    graph = torch.cuda.CUDAGraph()
+                    capturing[0] = True
+                    try:
+                        with torch.cuda.graph(graph):
+                            run_steps()
+                    finally:
+                        capturing[0] = False
+                    self._graphs = {k: g for k, g in self._graphs.items()
+                                    if g[2] == self._generations() and k != key}
+                    while len(self._graphs) >= self.MAX_GRAPHS:
+                        self._graphs.pop(next(iter(self._graphs)))
+                    self._graphs[key] = (graph, None, self._generations())
             if traced:
                 after.record()
                 self._trace((n * n_steps, n, t1 - t0, time.perf_counter() - t1, before, after,

@@ -425,11 +425,23 @@ def _skinny_plan(M: int, N: int, K: int, tiled: bool):
                 if N % (16 * rg) == 0 and 128 <= N // (16 * rg) <= 256:
                     return rg, 1
             return (2 if N >= 6144 else 1), 1
+        # 17 to 64 tokens.  A wide output fills the chip by its row groups alone.  A narrow one
+        # takes about 256 workgroups: the longer K is, the more rows a workgroup keeps (the
+        # tokens are read again by every workgroup), and a split along K makes up for the
+        # workgroups that costs (4096 x 1024: 256 of one row group; 1024 x 2048: 64 x 4 along
+        # K; 2048 x 6144: 64 of two row groups x 4; 4096 x 12288: 64 of four x 4).  Measured on
+        # MI355X at the projection widths of the Qwen3 0.6B to 8B shapes.
         if N >= 16384:
             return 4, 1
         if N >= 6144:
             return 2, 1
-        return (4, 4) if K >= 8192 else (2, 2)
+        rg = 1 if K < 4096 else 2 if K < 8192 else 4
+        while rg > 1 and N % (16 * rg) != 0:
+            rg //= 2
+        wgs, ks = N // (16 * rg), 1
+        while 2 * ks * wgs <= 256 and 2 * ks <= 16 and K >= 1024 * ks:
+            ks *= 2
+        return rg, ks
     if M <= 16:
         rg = 4 if N // 64 >= 256 else 1
         ks = 2 if (rg == 4 and N // 64 < 1024) else 1
@@ -458,7 +470,8 @@ def _mid_plan(M: int, N: int, K: int, w_tiled: bool, swiglu: bool = False):
     if swiglu:
         return 1
     tiles = (N + 127) // 128
-    return max(1, min(256 // tiles, K // 1024))
+    # up to 64 tokens a workgroup has half the work per k-tile: it may keep as little as 512 of K
+    return max(1, min(256 // tiles, K // (512 if M <= 64 else 1024)))
 
 
 _measured = None
@@ -558,11 +571,14 @@ def _small_plan(M: int, N: int, K: int, w_tiled: bool, swiglu: bool = False):
                 plan = entry[str(min(same, key=lambda b: abs(b - bucket)))]
                 return tuple(plan)
     mid = _mid_plan(M, N, K, w_tiled, swiglu)
-    if mid is not None:
+    # a short K: what the weight-streaming kernel reads again per workgroup is little, and it
+    # stays ahead of the kernel that stages the tokens up to 56 tokens (64 at K <= 1024)
+    short_k = w_tiled and 32 < M <= SKINNY_MAX_M and K <= 2048 and (M <= 56 or K <= 1024)
+    if mid is not None and not short_k:
         return ("mid", mid)
     if M <= SKINNY_MAX_M:
         if swiglu:
-            return ("skinny", 4 if (M > 16 and N >= 16384) else 2, 1)
+            return ("skinny", 4 if (M > 16 and N >= 12288 and N % 64 == 0) else 2, 1)
         return ("skinny",) + tuple(_skinny_plan(M, N, K, w_tiled))
     return None
 
