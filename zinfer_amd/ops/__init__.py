@@ -608,7 +608,8 @@ def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = Fals
         # between one and two 128 x 256 tiles per CU half the CUs hold two workgroups and half
         # one, and the smaller tiles finish sooner (2048 tokens into 6144 outputs); with few
         # tiles along the tokens (512 tokens into 24576 outputs) the large tiles still win
-        if tiles >= 160 and not (256 < tiles < 512 and tiles_m > 4):
+        # (five rows of tiles: 544 tokens into 24576 outputs, 480 large tiles, 143 -> 115 us)
+        if tiles >= 160 and not (256 < tiles < 512 and tiles_m > 5):
             return 10
         one_round = tiles_m * ((N + 127) // 128) <= 256
         return 16 if K > 0 and K % 128 == 0 and (K >= 8192 or one_round) else 6
