@@ -41,17 +41,20 @@ PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 PAGE = 16
 
 
-def _shape(layers, hidden, heads, inter):
+def _shape(layers, hidden, heads, inter, tied=False):
     return dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=layers,
                 hidden_size=hidden, num_attention_heads=heads, num_key_value_heads=8,
                 head_dim=128, intermediate_size=inter, vocab_size=151936, rope_theta=1000000.0,
-                rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960,
+                rms_norm_eps=1e-6, tie_word_embeddings=tied, max_position_embeddings=40960,
                 torch_dtype="bfloat16")
 
 
-SHAPES = {"8b": _shape(36, 4096, 32, 12288), "14b": _shape(40, 5120, 40, 17408),
-          "32b": _shape(64, 5120, 64, 25600)}
-SHAPE_NAMES = {"8b": "Qwen3-8B", "14b": "Qwen3-14B", "32b": "Qwen3-32B"}
+# (the three smaller shapes tie the head to the embedding)
+SHAPES = {"0.6b": _shape(28, 1024, 16, 3072, True), "1.7b": _shape(28, 2048, 16, 6144, True),
+          "4b": _shape(36, 2560, 32, 9728, True), "8b": _shape(36, 4096, 32, 12288),
+          "14b": _shape(40, 5120, 40, 17408), "32b": _shape(64, 5120, 64, 25600)}
+SHAPE_NAMES = {"0.6b": "Qwen3-0.6B", "1.7b": "Qwen3-1.7B", "4b": "Qwen3-4B", "8b": "Qwen3-8B",
+               "14b": "Qwen3-14B", "32b": "Qwen3-32B"}
 
 
 def build_llm(raw: dict, dtype: str, seed: int, pool_tokens: int, max_seqs: int, **sched):

@@ -630,3 +630,22 @@ def test_bfloat16_drift_over_36_layers_is_what_its_roundings_explain(tmp_path):
     # the depth costs what a random walk costs: three times the distance for nine times the layers
     assert seen[(36, "prompt")][0] <= 1.25 * 3.0 * seen[(4, "prompt")][0]
     assert 0.02 <= seen[(36, "prompt")][1] <= 0.05, "the model of the served shape's 3.9 %"
+
+
+def test_debug_tables_finds_a_page_that_is_not_the_pools(tmp_path_factory):
+    """With the debugging check on, a block table that names a page beyond the pool (here: put
+    there by the test) is an error that names group, sequence and page index before any of
+    the step's kernels runs; a sound step passes."""
+    from zinfer_amd import StepError
+    from zinfer_amd.engine import StepEntry
+    from zinfer_amd.engine.replay import make_engine
+    path = tiny.model_dir_of("D", str(tmp_path_factory.getbasetemp()), torch.bfloat16)
+    eng = make_engine(path, "bfloat16", 256, DEV)
+    eng.debug_tables = True
+    lg = eng.step([StepEntry("x", [1] * 40, [39]), StepEntry("y", [2] * 5, [4])])
+    assert lg.shape[0] == 2
+    eng.step([StepEntry("x", [3], [0]), StepEntry("y", [4], [0])])      # a graph-captured step
+    table = eng.cache.table(0, "x")
+    table[1] = eng.cache.groups[0].pages.num_pages + 7
+    with pytest.raises(StepError, match=r"BlockTableOutOfBounds: group 0, sequence 1, page index 1"):
+        eng.step([StepEntry("y", [5], [0]), StepEntry("x", [6], [0])])

@@ -1149,6 +1149,31 @@ def test_stream_read_reads_every_byte_once():
     assert ops.measure_read_bandwidth(DEV, nbytes=1 << 28, repeats=2) > 1e12
 
 
+def test_check_tables_reports_and_never_traps():
+    """The debugging check of a step's tables: a page beyond the pool, a page that is not held
+    (-1) inside a context, a context longer than the row, a slot beyond the pool are reported;
+    entries beyond a context are not looked at."""
+    ops = _ops()
+    ps, num_pages = 16, 10
+    bt = torch.tensor([[3, 9, -1, -1], [0, 1, 2, -1]], dtype=torch.int32)
+    ctx = torch.tensor([20, 48], dtype=torch.int32)
+    slots = torch.tensor([3 * 16 + 4, 2 * 16 + 15], dtype=torch.int32)
+
+    def run(bt, ctx, slots):
+        rep = torch.zeros(4, dtype=torch.int32, device=DEV)
+        ops.check_tables(bt.to(DEV), ctx.to(DEV), None if slots is None else slots.to(DEV), ps,
+                         num_pages, rep)
+        return rep.tolist()
+    assert run(bt, ctx, slots) == [0, 0, 0, 0]
+    assert run(bt, ctx, None) == [0, 0, 0, 0]
+    bad = bt.clone(); bad[0, 1] = 10
+    assert run(bad, ctx, slots) == [1, 0, 1, 10]
+    bad = bt.clone(); bad[1, 2] = -1
+    assert run(bad, ctx, slots) == [1, 1, 2, -1]
+    assert run(bt, torch.tensor([20, 65], dtype=torch.int32), slots)[:2] == [1, 1]
+    assert run(bt, ctx, torch.tensor([5, 160], dtype=torch.int32)) == [2, 1, 0, 160]
+
+
 def test_only_the_kernels_of_a_class_are_launched():
     """Under `only_classes` a launcher of another class leaves its output alone."""
     ops = _ops()

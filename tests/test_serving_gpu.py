@@ -171,3 +171,31 @@ def test_thirty_six_layers_against_the_plain_model(dtype, tolerance, tmp_path):
     got = np.concatenate(got)
     err = np.abs(got - ref).max(axis=1) / np.abs(ref).max()
     assert err.max() <= tolerance, f"position {int(err.argmax())}: {err.max():.3g}"
+
+
+def test_bench_commands_print_the_reference_keys_and_class_times(tmp_path, capsys):
+    """`zinfer bench` and `bench-batch` over a tiny model: the reference's report keys
+    (`src/app/cli/tools/bench/runtime.zig:81-98`), with --classes a decode step's time per
+    class of kernels, and nothing held afterwards (the command checks its cache itself)."""
+    from zinfer_amd import cli
+    path = tiny.model_dir_of("D", str(tmp_path), torch.bfloat16)
+    for cmd, extra, batch in (("bench", [], 1), ("bench-batch", ["3"], 3)):
+        rc = cli.main([cmd, path, "5,6,7,8,9"] + extra + ["6", "--ignore-eos", "--classes",
+                                                          "--max-tokens", "512"])
+        out = capsys.readouterr().out
+        assert rc == 0, out
+        keys = {line.split(":")[0] for line in out.splitlines() if ":" in line}
+        for key in ("model_dir", "backend", "kv_cache", "q8_layout", "kernel_isa", "threads",
+                    "prompt_tokens", "decode_tokens", "tokenize_ms", "prefill_ms", "decode_ms",
+                    "prefill_tok_s", "decode_tok_s", "weights_bytes", "weights_mib",
+                    "kv_cache_bytes", "kv_cache_mib"):
+            assert key in keys, (cmd, key)
+        assert f"decode_tokens: {6 * batch}" in out
+        times = {k: float(line.split(":")[1]) for line in out.splitlines()
+                 for k in [line.split(":")[0]] if k.startswith("decode_step_")}
+        assert set(times) == {f"decode_step_{c}_ms" for c in
+                              ("products", "attention", "norm_rope_write", "head_sampling",
+                               "other", "step")}
+        assert times["decode_step_products_ms"] > 0 and times["decode_step_attention_ms"] > 0
+        parts = sum(v for k, v in times.items() if k != "decode_step_step_ms")
+        assert 0.5 * times["decode_step_step_ms"] <= parts <= 2.0 * times["decode_step_step_ms"]

@@ -48,6 +48,8 @@ Flags:
   --max-step-tokens <n>        --chunk <n>                --max-seqs <n>
   --ignore-eos                 --device <cuda:0>          --multi-step <n>
   --config <config.json> --random-weights <seed>   (weights drawn from the seed; no folder read)
+  --debug-tables               (every step's block tables and slots checked on the device first)
+  --classes                    (bench, bench-batch: a decode step's time per class of kernels)
 """
 
 
@@ -98,6 +100,8 @@ class Options:
         self.ignore_eos = False
         self.device = "cuda:0"
         self.seed = 0
+        self.debug_tables = False       # check every step's block tables on the device
+        self.classes = False            # bench: a decode step's time per class of kernels
         self.config_path: Optional[str] = None          # with --random-weights: no model folder
         self.random_weights: Optional[int] = None
 
@@ -174,6 +178,10 @@ def parse_flags(flags: List[str], opt: Options) -> None:
             opt.multi_step = int(value())
         elif a == "--ignore-eos":
             opt.ignore_eos = True
+        elif a == "--debug-tables":
+            opt.debug_tables = True
+        elif a == "--classes":
+            opt.classes = True
         elif a == "--device":
             opt.device = value()
         else:
@@ -237,7 +245,7 @@ def _llm(model_dir: str, opt: Options, max_tokens: Optional[int] = None):
     return LLM(model_dir, config=opt.config_path, random_seed=opt.random_weights, dtype=opt.dtype, device=opt.device, page_size=opt.page_size,
                max_tokens=opt.max_tokens or max_tokens, max_step_tokens=opt.max_step_tokens,
                chunk_size=opt.chunk, max_seqs=opt.max_seqs, kv_dtype=kv,
-               multi_step=opt.multi_step)
+               multi_step=opt.multi_step, debug_tables=opt.debug_tables)
 
 
 def _text_hooks(model_dir: str):
@@ -603,7 +611,9 @@ def cmd_bench(args: List[str], mode: str) -> int:
     print(f"model_dir: {model_dir}")
     print(f"backend: {opt.dtype}")
     print(f"kv_cache: {llm.engine.cache.groups[0].k.dtype if llm.engine.cache.groups else '-'}")
+    print("q8_layout: none")                    # (the reference's quantised cache: not built)
     print("kernel_isa: gfx950")
+    print("threads: 0")                         # (no host thread pool: the device's grid)
     if mode == "bench-continuous":
         sched = llm.new_scheduler()
         for _ in range(total):
@@ -648,6 +658,10 @@ def cmd_bench(args: List[str], mode: str) -> int:
                     live[n] = t
         torch.cuda.synchronize()
         t2 = time.perf_counter()
+        classes = None
+        if opt.classes and live and eng.use_graphs:
+            # where a decode step's time goes: the step once per class of kernels
+            classes = eng.class_times([StepEntry(n, [live[n]], [0]) for n in live])
         for n in names:                       # what the requests hold goes back
             eng.release(n)
         eng.cache.check()
@@ -655,10 +669,14 @@ def cmd_bench(args: List[str], mode: str) -> int:
             print(f"batch_size: {batch}")
         print(f"prompt_tokens: {len(ids)}")
         print(f"decode_tokens: {decoded}")
+        print("tokenize_ms: 0.000")             # (the prompt comes as token ids)
         print(f"prefill_ms: {(t1 - t0) * 1e3:.3f}")
         print(f"decode_ms: {(t2 - t1) * 1e3:.3f}")
         print(f"prefill_tok_s: {len(ids) * batch / (t1 - t0):.3f}")
         print(f"decode_tok_s: {decoded / max(t2 - t1, 1e-12):.3f}")
+        if classes is not None:
+            for name, t in classes.items():
+                print(f"decode_step_{name}_ms: {t * 1e3:.4f}")
     wb = _weights_bytes(llm)
     kb = llm.engine.cache.kv_bytes()
     print(f"weights_bytes: {wb}")

@@ -774,3 +774,49 @@ extern "C" int zf_stream_read(const void* src, long long bytes, uint32_t* sink, 
                      (const zf_u32x4_t*)src, (size_t)(bytes / 16), sink);
   ZF_CHECK_LAUNCH();
 }
+
+// ---------------------------------------------------------------- debugging: a step's tables
+// Every page a step's kernels will look up (the first ceil(ctx_len / page_size) entries of a
+// sequence's row) must be a page of the pool, every slot a row of the pool.  Nothing traps:
+// a thread that finds a bad entry writes (1 + kind, sequence or token, index, value) into
+// `report` (kind 0: block table, 1: slot mapping; which of several bad entries is reported is
+// left open), and the host reads it.
+__global__ void check_tables_kernel(const int* __restrict__ block_table,
+                                    const int* __restrict__ ctx_len,
+                                    const int* __restrict__ slot_mapping, int n_seqs,
+                                    int max_pages, int page_size, int num_pages, int n_tokens,
+                                    int* __restrict__ report) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n_seqs * max_pages) {
+    const int s = i / max_pages, p = i % max_pages;
+    const int ctx = ctx_len[s];
+    const bool used = ctx >= 0 && p < (ctx + page_size - 1) / page_size;
+    const int page = block_table[i];
+    if (ctx < 0 || ctx > max_pages * page_size || (used && (page < 0 || page >= num_pages))) {
+      report[1] = s;
+      report[2] = p;
+      report[3] = ctx < 0 || ctx > max_pages * page_size ? ctx : page;
+      report[0] = 1;
+    }
+  }
+  if (slot_mapping != nullptr && i < n_tokens) {
+    const int slot = slot_mapping[i];
+    if (slot < 0 || slot >= num_pages * page_size) {
+      report[1] = i;
+      report[2] = 0;
+      report[3] = slot;
+      report[0] = 2;
+    }
+  }
+}
+
+extern "C" int zf_check_tables(const int* block_table, const int* ctx_len,
+                               const int* slot_mapping, int n_seqs, int max_pages, int page_size,
+                               int num_pages, int n_tokens, int* report, hipStream_t stream) {
+  if (n_seqs <= 0 || max_pages <= 0 || page_size <= 0) return 1;
+  const int n = max(n_seqs * max_pages, n_tokens);
+  hipLaunchKernelGGL(check_tables_kernel, dim3((n + 255) / 256), dim3(256), 0, stream,
+                     block_table, ctx_len, slot_mapping, n_seqs, max_pages, page_size, num_pages,
+                     n_tokens, report);
+  ZF_CHECK_LAUNCH();
+}

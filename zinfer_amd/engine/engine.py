@@ -34,7 +34,8 @@ class Engine:
 
     def __init__(self, model: DecoderModel, *, page_size: int = 16, num_pages: int = 256,
                  max_requests: int = 64, kv_dtype: Optional[torch.dtype] = None,
-                 poison_freed: bool = False, use_graphs: bool = True):
+                 poison_freed: bool = False, use_graphs: bool = True,
+                 debug_tables: bool = False):
         self.model = model
         self.device = model.ctx.device
         if self.device.type == "cuda":
@@ -53,6 +54,9 @@ class Engine:
         # the parts that want to know about a step's shape, one per kind
         self._hint_providers = model.hint_providers()
         self.page_size = page_size
+        # debugging: every step's block tables and slots are checked on the device against the
+        # pool before its kernels run (one small kernel and a wait for its report a step)
+        self.debug_tables = debug_tables and self.device.type == "cuda"
         self._scratch = Scratch(self.device)
         self._meta_host = None          # two pinned buffers that take turns
         self._meta_dev: Optional[torch.Tensor] = None
@@ -108,6 +112,8 @@ class Engine:
                     import time
                     t0 = time.perf_counter()
                 ctx = self._build_context(entries, bucket_pages=decode_only)
+                if self.debug_tables:
+                    self._check_tables(ctx)
                 if traced:
                     t1 = time.perf_counter()
                     before = torch.cuda.Event(enable_timing=True)
@@ -141,6 +147,24 @@ class Engine:
         """The records gathered so far (the list is emptied; tracing stays on)."""
         done, self.step_trace = self.step_trace or [], [] if self.step_trace is not None else None
         return done
+
+    def _check_tables(self, ctx: StepContext) -> None:
+        """The device's own look at what the step's kernels will index with (debugging)."""
+        from .. import ops
+        report = self._scratch.get("table_report", (4,), torch.int32)
+        for g, tables in enumerate(ctx.kv):
+            report.zero_()
+            ops.check_tables(tables.block_table, ctx.ctx_len, tables.slot_mapping, self.page_size,
+                             self.cache.groups[g].pages.num_pages, report)
+            kind, a, b, value = report.tolist()
+            if kind == 1:
+                raise StepError(f"BlockTableOutOfBounds: group {g}, sequence {a}, page index {b}: "
+                                f"{value} is no page of a pool of "
+                                f"{self.cache.groups[g].pages.num_pages} (or a context beyond "
+                                "the table)")
+            if kind == 2:
+                raise StepError(f"SlotOutOfBounds: group {g}, token {a}: slot {value} is no row "
+                                "of the pool")
 
     def _reserve(self, wanted_len) -> List[object]:
         """Adds the requests that are new and reserves every request's pages; returns the

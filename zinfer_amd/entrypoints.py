@@ -24,13 +24,14 @@ class LLM:
                  num_pages: Optional[int] = None, max_step_tokens: int = 2048,
                  chunk_size: Optional[int] = None, max_seqs: int = 64,
                  kv_dtype: Optional[str] = None, multi_step: int = 8,
-                 config=None, random_seed: Optional[int] = None):
+                 config=None, random_seed: Optional[int] = None, debug_tables: bool = False):
         """A model folder, or ``config`` (a typed configuration, a dict of config.json keys or
         the path of a config.json) with ``random_seed``: weights drawn from the seed, the same
         values that ``write_model_dir`` stores for it.  ``max_tokens`` (or ``num_pages``) sizes the cache pool; by default the pool holds
         ``max_seqs`` requests of ``max_position_embeddings`` tokens, capped at 1/2 of the free
         device memory.  ``multi_step``: the most decode steps that run in a row on the device
-        without the host between them (1: the host sees every step)."""
+        without the host between them (1: the host sees every step).  ``debug_tables``: every
+        step's block tables and slots are checked on the device before its kernels run."""
         if (config is None) != (random_seed is None):
             raise ValueError("config and random_seed go together")
         if config is not None:
@@ -47,7 +48,8 @@ class LLM:
         from .models.build import parse_dtype
         self.engine = Engine(self.model, page_size=page_size, num_pages=num_pages,
                              max_requests=max_seqs,
-                             kv_dtype=parse_dtype(kv_dtype) if kv_dtype else None)
+                             kv_dtype=parse_dtype(kv_dtype) if kv_dtype else None,
+                             debug_tables=debug_tables)
         self.scheduler_options = dict(max_step_tokens=max_step_tokens, chunk_size=chunk_size,
                                       max_seqs=max_seqs, eos_token_ids=spec.eos_token_ids,
                                       multi_step=multi_step)
@@ -64,7 +66,8 @@ class LLM:
         per_token, state_bytes = 0, 0
         for need in self.model.cache_needs():
             if isinstance(need, KVNeed):
-                per_token += 2 * need.n_kv_heads * need.head_dim * elem
+                size = elem if need.dtype is None else torch.empty((), dtype=need.dtype).element_size()
+                per_token += need.n_kv_heads * (need.key_width + need.value_width) * size
             elif isinstance(need, StateNeed):
                 n = max_seqs
                 for d in need.shape:

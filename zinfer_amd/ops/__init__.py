@@ -346,6 +346,29 @@ def randinit(out: torch.Tensor, key: int, start: int, kind: str, std: float = 0.
 
 
 @_launches("other")
+def check_tables(block_table: torch.Tensor, ctx_len: torch.Tensor,
+                 slot_mapping: Optional[torch.Tensor], page_size: int, num_pages: int,
+                 report: torch.Tensor) -> None:
+    """Debugging: marks in ``report`` (int32 [4], zeroed by the caller: kind, sequence or token,
+    index, value) a block-table entry among those a step's kernels will look up that is no
+    page of the pool (kind 1), a context longer than the table's row, or a slot that is no row
+    of the pool (kind 2).  The kernels themselves trust their tables; this is the check to
+    switch on when they are in doubt (``Engine(debug_tables=True)``)."""
+    _need_gpu(block_table, ctx_len, slot_mapping, report)
+    for t, name in ((block_table, "block_table"), (ctx_len, "ctx_len"), (report, "report")):
+        _i32(t, name)
+    if slot_mapping is not None:
+        _i32(slot_mapping, "slot_mapping")
+    if block_table.dim() != 2 or ctx_len.shape != (block_table.shape[0],) or report.numel() < 4:
+        raise KernelUnavailable("check_tables: int32 [n, pages] table, [n] contexts, [4] report")
+    lib = build.load("elementwise")
+    _check(lib.zf_check_tables(_ptr(block_table), _ptr(ctx_len), _ptr(slot_mapping),
+                               block_table.shape[0], block_table.shape[1], int(page_size),
+                               int(num_pages), 0 if slot_mapping is None else slot_mapping.shape[0],
+                               _ptr(report), _stream()), "check_tables")
+
+
+@_launches("other")
 def stream_read(buf: torch.Tensor, sink: torch.Tensor, workgroups: int = 2048) -> None:
     """Reads ``buf`` once (16-byte non-temporal loads, 8 in flight a lane) and xors it into
     ``sink`` (int32, one word per workgroup): the read stream the weight-streaming kernels are

@@ -9,7 +9,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Callable, Dict
 
-from . import (advance_decode, apply_penalties, argmax, argmax_no_alloc, cast,
+from . import (advance_decode, apply_penalties, argmax, argmax_no_alloc, cast, check_tables,
                decode_attention_fused, embed, gather_rows, gemm, gemm_emit, gemm_given,
                gemm_partials, gemm_sum_norm, gemm_swiglu, norm_gemm, paged_attention, poison_pages,
                qk_norm_rope_kv_write, randinit, rmsnorm, sample_topk, scale_cap, stream_read,
@@ -58,6 +58,8 @@ KERNELS: Dict[str, KernelEntry] = {
                                    "src/sampling/sampler.zig:186-201"),
     "sample_topk": KernelEntry(sample_topk, "sampling", "src/sampling/sampler.zig:18-91"),
     "randinit": KernelEntry(randinit, "randinit", "own: counter-based random weights"),
+    "check_tables": KernelEntry(check_tables, "elementwise",
+                                "own: a step's block tables and slots against the pool"),
     "stream_read": KernelEntry(stream_read, "elementwise",
                                "own: the read stream bandwidths are measured against"),
 }
