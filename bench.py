@@ -241,13 +241,15 @@ def run_continuous(llm, cfg, elem: int, n_requests: int, lo: int, hi: int, new_t
                    seed: int) -> dict:
     """All requests arrive together; the scheduler admits them, cuts their prompts into
     portions beside the decode tokens of the others, decodes, finishes and frees.  The
-    workload runs twice with the same requests; the second pass is timed (the first settles
-    work buffers and captures the decode graphs of every batch shape that occurs)."""
+    workload runs three times with the same requests; the third pass is timed (the first
+    settles work buffers and captures the decode graph of every batch shape that occurs, the
+    second records the runs of decode steps whose shape came a second time: a server that has
+    been up for a while)."""
     import torch
     from zinfer_amd.sampling import SamplingParams
     eng = llm.engine
     out = {}
-    for timed in (False, True):
+    for timed in (False, False, True):
         g = torch.Generator().manual_seed(seed)
         lens = torch.randint(lo, hi + 1, (n_requests,), generator=g).tolist()
         sched = llm.new_scheduler()
@@ -320,6 +322,7 @@ def main_continuous(args) -> int:
                     multi_step=args.multi_step)
     cfg = llm.config
     build_s = time.perf_counter() - t_build
+    llm.engine.capture_runs = not args.no_run_graphs
     elem = 2 if args.dtype == "bfloat16" else 4
     res = run_continuous(llm, cfg, elem, n, lo, hi, new, args.seed + 7)
     line = {"metric": f"continuous batching tok/s (prompt + generated), "
