@@ -30,7 +30,8 @@ USAGE = """Usage:
   zinfer bench [model_dir] <ids_csv> [max_new_tokens]
   zinfer bench-batch [model_dir] <ids_csv> <batch_size> [max_new_tokens]
   zinfer bench-continuous [model_dir] <ids_csv> <batch_size> <total_requests> [max_new_tokens]
-  zinfer bench-ops [model_dir] [--shape 8b|14b|32b] [--tokens 1,8,64,2048] [--iters N]
+  zinfer bench-ops [model_dir] [--shape 0.6b|1.7b|4b|8b|14b|32b] [--tokens 1,8,64,2048] [--iters N]
+                   [--tune [--plans-out kernel_plans.json]]
   zinfer random-model <config.json> <out_dir> [--seed <u64>] [--dtype bfloat16|float32]
 
 Defaults:
