@@ -244,3 +244,27 @@ def test_a_model_folders_plans_are_checked_and_override_the_table(tmp_path, monk
         p.write_text(json.dumps(bad))
         with pytest.raises(Exception, match="kernel plans"):
             ops.load_plans(str(p))
+
+
+def test_the_last_round_of_large_tiles_is_split_only_where_it_is_short():
+    """`_tile_tail_split`: whole rounds stay whole; a short last round behind one or two whole
+    ones goes to workgroups that share its tiles along K, every part an even number of
+    k-tiles and no more parts than one round holds; a long last round, a product of under one
+    round or of many rounds stays as it is."""
+    from zinfer_amd import ops
+    for M in range(128, 8193, 128):
+        for N, K in ((34816, 5120), (24576, 4096), (5120, 17408), (4096, 12288), (51200, 5120),
+                     (6144, 4096), (24576, 2048), (9728 * 2, 2560)):
+            tiles = ((M + 127) // 128) * ((N + 255) // 256)
+            tail = ops._tile_tail_split(M, N, K)
+            if tail is None:
+                continue
+            whole, split = tail
+            assert whole % ops.TILE_PLACES == 0 and 0 < whole <= 2 * ops.TILE_PLACES
+            assert 0 < tiles - whole < ops.TILE_PLACES and (tiles - whole) * split <= ops.TILE_PLACES
+            assert split >= 2 and (K // 64) % (2 * split) == 0 and K // 64 // split >= 8
+    assert ops._tile_tail_split(512, 34816, 5120) == (512, 4)     # 544 tiles
+    assert ops._tile_tail_split(544, 34816, 5120) is None         # 680: a third of a round
+    assert ops._tile_tail_split(512, 24576, 4096) is None         # 384: under one round
+    assert ops._tile_tail_split(2048, 24576, 4096) is None        # three whole rounds
+    assert ops._tile_tail_split(2048, 34816, 5120) is None        # a last round behind four

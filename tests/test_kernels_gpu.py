@@ -216,8 +216,9 @@ def test_gemm_many_large_tiles(kind, K, M, N, variant):
     _check_tiled(ops, kind, M, N, K, variant)
 
 
-def _check_tiled(ops, kind, M, N, K, variant, seed=35):
+def _check_tiled(ops, kind, M, N, K, variant, seed=35, tile_tail=None):
     """One tiled kernel on pre-tiled W against the plain product."""
+    how = dict(tile_variant=variant) if tile_tail is None else dict(tile_tail=tile_tail)
     a = _rand((M, K), torch.bfloat16, seed)
     w = _rand((N, K), torch.bfloat16, seed + 1, 0.05)
     if kind == "swiglu":
@@ -225,7 +226,7 @@ def _check_tiled(ops, kind, M, N, K, variant, seed=35):
         want = torch.empty((M, N // 2), dtype=torch.bfloat16)
         ref.gemm_swiglu(a, wi.cpu(), want)
         got = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
-        ops.gemm_swiglu(a.to(DEV), ops.pretile_weight(wi), got, w_tiled=True, tile_variant=variant)
+        ops.gemm_swiglu(a.to(DEV), ops.pretile_weight(wi), got, w_tiled=True, **how)
         assert rel_err(got, want) <= tol(torch.bfloat16)
         return
     acc = kind == "accumulate"
@@ -233,8 +234,48 @@ def _check_tiled(ops, kind, M, N, K, variant, seed=35):
     want = base.clone()
     ref.gemm(a, w, want, acc)
     got = base.clone().to(DEV)
-    ops.gemm(a.to(DEV), ops.pretile_weight(w.to(DEV)), got, acc, w_tiled=True, tile_variant=variant)
+    ops.gemm(a.to(DEV), ops.pretile_weight(w.to(DEV)), got, acc, w_tiled=True, **how)
     assert rel_err(got, want) <= (2e-5 if acc else tol(torch.bfloat16))
+
+
+@pytest.mark.parametrize("kind", ["store", "accumulate", "swiglu"])
+@pytest.mark.parametrize("M,N,K,whole,split", [
+    (300, 2112, 1024, 16, 2), (300, 2112, 1024, 20, 8), (257, 2240, 1536, 0, 3),
+    (520, 4160, 640, 80, 5), (4100, 4160, 256, 512, 2), (130, 320, 192, 1, 3),
+    (200, 512, 320, 2, 2)])
+def test_gemm_large_tiles_with_the_last_round_split_along_k(kind, M, N, K, whole, split):
+    """The 128 x 256 tiles with the tiles from ``whole`` on shared by ``split`` workgroups each
+    along K and their partials added by a second kernel: edges in M and N that are no multiple
+    of the tile, parts of an even and an odd number of k-tiles and parts that are not all
+    equal (W one or two k-tiles ahead), every epilogue; against the plain product, and against
+    the same tiles unsplit up to the order of the sums."""
+    ops = _ops()
+    _check_tiled(ops, kind, M, N, K, 10, seed=81, tile_tail=(whole, split))
+
+
+def test_gemm_last_round_split_is_chosen_and_agrees():
+    """Where the rule splits the last round (more than 512 tiles of 128 x 256, a short last
+    round, a long K) the product goes through that path, and its result is the unsplit one's
+    up to the order in which 32-bit sums are added."""
+    ops = _ops()
+    M, N, K = 520, 27648 + 256, 4096         # 5 x 109 = 545 tiles: a last round of 33
+    tail = ops._tile_tail_split(M, N, K)
+    assert tail is not None and tail[0] == 512 and ops._tile_variant(M, N, True, False, K) == 10
+    a = _rand((M, K), torch.bfloat16, 83).to(DEV)
+    wt = ops.pretile_weight(_rand((N, K), torch.bfloat16, 84, 0.05).to(DEV))
+    chosen = torch.empty((M, N), dtype=torch.float32, device=DEV)
+    forced = torch.empty_like(chosen)
+    whole = torch.empty_like(chosen)
+    before = ops.launch_count()
+    ops.gemm(a, wt, chosen, w_tiled=True)
+    assert ops.launch_count() == before + 1
+    ops.gemm(a, wt, forced, w_tiled=True, tile_tail=tail)
+    ops.gemm(a, wt, whole, w_tiled=True, tile_variant=10)
+    assert torch.equal(chosen, forced)
+    assert not torch.equal(chosen, whole) and rel_err(chosen, whole) <= 2e-5
+    # the tiles of the whole rounds have the unsplit product's bits
+    same = (chosen == whole).float().mean().item()
+    assert same > 0.9
 
 
 @pytest.mark.parametrize("kind", ["store", "accumulate", "swiglu"])

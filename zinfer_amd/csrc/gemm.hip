@@ -412,11 +412,17 @@ __device__ __forceinline__ void store_through_slab(f32x16_t (&acc)[FM][FNALL], f
 // banks.  Two stages in two arrays, so that the compiler knows which reads wait for which
 // copies; the barrier is a bare s_barrier behind a wait that lets the W loads issued since
 // (younger than the copies) stay in flight.
+// TAIL: the tiles beyond the last whole round of the chip (the tile order's last `tail` ones)
+// are shared by tail_split workgroups each, along K: workgroups [whole, whole + tail *
+// tail_split) of the grid, which leave float32 partials [tail][tail_split][BM][BN] in tail_ws
+// for tile_tail_reduce_kernel; a short last round then takes 1 / tail_split of a tile's time
+// instead of a whole one.
 template <int BM, int BN, int WM, int WN, int EPI, int TKM = TK, bool W2 = false,
-          bool ADMA = false>
+          bool ADMA = false, bool TAIL = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdirect_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
-    int N, int K, int tiles_m, int tiles_n) {
+    int N, int K, int tiles_m, int tiles_n, int whole, int tail_split,
+    float* __restrict__ tail_ws) {
   // (the host pass, which only needs the launch stub, does not know the buffer descriptor type)
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int NWN = BN / WN, NT = (BM / WM) * NWN * 64;
@@ -427,8 +433,19 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   bf16_t* lds = (bf16_t*)lds_raw;       // two stages of BM rows of LROW elements
 
+  // which tile, and which of how many parts of its k-tiles
+  int tile = blockIdx.x, kpart = blockIdx.y, kparts = gridDim.y;
+  bool in_tail = false;
+  if constexpr (TAIL) {
+    if ((int)blockIdx.x >= whole) {
+      in_tail = true;
+      tile = whole + ((int)blockIdx.x - whole) / tail_split;
+      kpart = ((int)blockIdx.x - whole) % tail_split;
+      kparts = tail_split;
+    }
+  }
   int tm, tn;
-  tile_of_workgroup<(BM >= 128 ? 8 : 1024 / BM)>(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  tile_of_workgroup<(BM >= 128 ? 8 : 1024 / BM)>(tile, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
   const int tid = threadIdx.x;
@@ -470,8 +487,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
   // gridDim.y workgroups share a tile's k-tiles (split-K for products with few tiles); each
   // then leaves a float32 partial [gridDim.y, M, N] in Cv for skinny_reduce_kernel
   const int kt_all = K / TKM;
-  const int kt0 = (int)((long long)blockIdx.y * kt_all / gridDim.y);
-  const int ktiles = (int)((long long)(blockIdx.y + 1) * kt_all / gridDim.y);
+  const int kt0 = (int)((long long)kpart * kt_all / kparts);
+  const int ktiles = (int)((long long)(kpart + 1) * kt_all / kparts);
   if (gridDim.y > 1) Cv = (float*)Cv + (size_t)blockIdx.y * M * N;
   using Buf0 = std::integral_constant<int, 0>;
   using Buf1 = std::integral_constant<int, 1>;
@@ -668,8 +685,62 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
   // (the main loop's last barrier has freed the token stages; the launch sizes the LDS for
   // stages and slabs)
   float* slab = (float*)lds_raw + (size_t)wave * 32 * (WN + 4);
+  if constexpr (TAIL) {
+    if (in_tail) {      // (uniform over the workgroup) the whole tile as it is, rows beyond M too
+      float* part = tail_ws + ((size_t)(tile - whole) * tail_split + kpart) * BM * BN;
+      store_through_slab<FM, FN, WN, EPI_STORE_F32>(acc, slab, wm * WM, wn * WN, BM, BN, part, lane);
+      return;
+    }
+  }
   store_through_slab<FM, FN, WN, EPI>(acc, slab, m0 + wm * WM, n0 + wn * WN, M, N, Cv, lane);
 #endif
+}
+
+// The partials of the tiles that gemm_bf16_tile_wdirect_kernel<.., TAIL> split along K, added
+// in split order, with the product's epilogue at the tile's place.  Grid (tail tiles, BM / 8):
+// a workgroup takes 8 rows of a tile, a thread 8 columns of a row (SwiGLU: 4 gate columns and
+// the 4 up columns that belong to them, which lie 16 further on).
+template <int BM, int BN, int EPI>
+__global__ __launch_bounds__(BN) void tile_tail_reduce_kernel(
+    const float* __restrict__ ws, void* __restrict__ Cv, int M, int N, int tiles_m, int tiles_n,
+    int whole, int split) {
+  static_assert(BN % 32 == 0 && BM % 8 == 0, "a row is BN / 8 threads");
+  constexpr int TPR = BN / 8;                        // threads per row
+  const int t = blockIdx.x;
+  int tm, tn;
+  tile_of_workgroup<(BM >= 128 ? 8 : 1024 / BM)>(whole + t, tiles_m, tiles_n, tm, tn);
+  const int row = blockIdx.y * 8 + threadIdx.x / TPR, q = threadIdx.x % TPR;
+  const int m = tm * BM + row;
+  const int c0 = EPI == EPI_SWIGLU ? (q / 4) * 32 + (q % 4) * 4 : q * 8;
+  const int c1 = EPI == EPI_SWIGLU ? c0 + 16 : c0 + 4;
+  const int n = tn * BN + c0;
+  if (m >= M || n >= N) return;
+  const float* part = ws + ((size_t)t * split * BM + row) * BN;
+  float4 x0 = float4{0.f, 0.f, 0.f, 0.f}, x1 = x0;
+  for (int k = 0; k < split; ++k) {
+    const float4 p0 = *(const float4*)(part + (size_t)k * BM * BN + c0);
+    const float4 p1 = *(const float4*)(part + (size_t)k * BM * BN + c1);
+    x0.x += p0.x; x0.y += p0.y; x0.z += p0.z; x0.w += p0.w;
+    x1.x += p1.x; x1.y += p1.y; x1.z += p1.z; x1.w += p1.w;
+  }
+  if (EPI == EPI_SWIGLU) {
+    const u32x2_t v = u32x2_t{pack_bf16x2(swiglu_f(x0.x, x1.x), swiglu_f(x0.y, x1.y)),
+                              pack_bf16x2(swiglu_f(x0.z, x1.z), swiglu_f(x0.w, x1.w))};
+    *(u32x2_t*)((bf16_t*)Cv + (size_t)m * (N / 2) + (n / 32) * 16 + (n % 32)) = v;
+  } else if (EPI == EPI_STORE_BF16) {
+    *(u32x4_t*)((bf16_t*)Cv + (size_t)m * N + n) =
+        u32x4_t{pack_bf16x2(x0.x, x0.y), pack_bf16x2(x0.z, x0.w), pack_bf16x2(x1.x, x1.y),
+                pack_bf16x2(x1.z, x1.w)};
+  } else {
+    float4* dst = (float4*)((float*)Cv + (size_t)m * N + n);
+    if (EPI == EPI_ACC_F32) {
+      const float4 o0 = dst[0], o1 = dst[1];
+      x0 = float4{o0.x + x0.x, o0.y + x0.y, o0.z + x0.z, o0.w + x0.w};
+      x1 = float4{o1.x + x1.x, o1.y + x1.y, o1.z + x1.z, o1.w + x1.w};
+    }
+    dst[0] = x0;
+    dst[1] = x1;
+  }
 }
 
 // ---------------------------------------------------------------- large M: 256-token tiles, one workgroup to a CU
@@ -986,7 +1057,7 @@ static int launch_tile_wdirect(const void* A, const void* W, void* C, int M, int
       if (e != hipSuccess) return (int)e;                                                     \
     }                                                                                         \
     hipLaunchKernelGGL(kern, grid, block, smem, stream, (const bf16_t*)A, (const bf16_t*)W, C, \
-                       M, N, K, tiles_m, tiles_n);                                            \
+                       M, N, K, tiles_m, tiles_n, 0, 1, (float*)nullptr);                     \
   } while (0)
   void* const final_c = C;
   if (ksplit > 1) {
@@ -999,6 +1070,40 @@ static int launch_tile_wdirect(const void* A, const void* W, void* C, int M, int
   else ZF_WD(EPI_ACC_F32);
 #undef ZF_WD
   if (ksplit > 1 && reduce) return launch_reduce(ws, final_c, M, N, ksplit, final_epi, stream);
+  return (int)hipGetLastError();
+}
+
+// The 128 x 256 tiles with the tile order's tiles from `whole` on shared by `split` workgroups
+// each along K (ws: float32 [tiles - whole][split][128][256]) and the kernel that adds their
+// partials; every epilogue.
+template <bool W2>
+static int launch_tile_tail(const void* A, const void* W, void* C, void* ws, int M, int N, int K,
+                            int epi, int whole, int split, hipStream_t stream) {
+  constexpr int BM = 128, BN = 256, WM = 128, WN = 64, NT = 256;
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  const long long tiles = (long long)tiles_m * tiles_n;
+  if (N % 16 != 0 || K % TK != 0 || ws == nullptr) return -3;
+  if (split < 2 || split > K / TK || whole < 0 || whole >= tiles) return -3;
+  if (W2 && (K / TK) % (2 * split) != 0) return -3;
+  const long long tail = tiles - whole;
+  if (whole + tail * split > 0x7fffffffLL) return -3;
+  const dim3 grid((unsigned)(whole + tail * split)), block(NT);
+  constexpr size_t smem = (size_t)(BM / WM) * (BN / WN) * 32 * (WN + 4) * sizeof(float);
+  static_assert(smem <= 64 * 1024, "the slabs fit the default limit");
+#define ZF_WT(E)                                                                              \
+  do {                                                                                        \
+    hipLaunchKernelGGL((gemm_bf16_tile_wdirect_kernel<BM, BN, WM, WN, E, TK, W2, true, true>), \
+                       grid, block, smem, stream, (const bf16_t*)A, (const bf16_t*)W, C, M, N, \
+                       K, tiles_m, tiles_n, whole, split, (float*)ws);                        \
+    hipLaunchKernelGGL((tile_tail_reduce_kernel<BM, BN, E>), dim3((unsigned)tail, BM / 8),    \
+                       dim3(BN), 0, stream, (const float*)ws, C, M, N, tiles_m, tiles_n,      \
+                       whole, split);                                                         \
+  } while (0)
+  if (epi == EPI_STORE_BF16) ZF_WT(EPI_STORE_BF16);
+  else if (epi == EPI_STORE_F32) ZF_WT(EPI_STORE_F32);
+  else if (epi == EPI_SWIGLU) ZF_WT(EPI_SWIGLU);
+  else ZF_WT(EPI_ACC_F32);
+#undef ZF_WT
   return (int)hipGetLastError();
 }
 
@@ -1073,6 +1178,21 @@ extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, i
     case 4: return launch_tile<256, 256, 128, 64, false>(A, W, C, M, N, K, epi, stream);
     default: return -4;
   }
+}
+
+// The 128 x 256 tiles of variant 10 on pre-tiled W where the tiles do not end on a whole round
+// of the chip: the first `whole` tiles of the tile order run one workgroup each, the rest
+// `split` workgroups each along K, so that the last round is as short as its share of the
+// work (512 tokens into 34816 outputs, K = 5120: 544 tiles for 512 places, 210 -> 150 us).
+// ws: float32 [tiles - whole][split][128][256].
+extern "C" int zf_gemm_bf16_tile_tail(const void* A, const void* W, void* C, void* ws, int M,
+                                      int N, int K, int epi, int whole, int split,
+                                      hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K % 8 != 0 || (epi == EPI_SWIGLU && N % 32 != 0)) return -3;
+  if (K % (2 * TK) == 0 && (K / TK) % (2 * split) == 0)
+    return launch_tile_tail<true>(A, W, C, ws, M, N, K, epi, whole, split, stream);
+  return launch_tile_tail<false>(A, W, C, ws, M, N, K, epi, whole, split, stream);
 }
 
 // 17 to 128 tokens on pre-tiled W.  The weight-streaming kernel below re-reads the tokens for

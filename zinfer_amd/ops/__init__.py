@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes
 import functools
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -703,6 +703,45 @@ def _tile256_time(variant: int, M: int, N: int, K: int) -> float:
     return t * (1.08 if (rounds > 1 and N <= 5120) else 1.0) + 4e-6
 
 
+TILE_PLACES = 512       # workgroups of the 128 x 256 tiles the chip holds at once: two to a CU
+
+
+def _tile_tail_split(M: int, N: int, K: int):
+    """(whole, split) if the 128 x 256 tiles of a product on pre-tiled weights should run with
+    their last, short round split along K, else None: ``whole`` tiles fill whole rounds of the
+    chip's ``TILE_PLACES`` places, and each of the others goes to ``split`` workgroups.  A
+    round of a few tiles takes as long as a full one (512 tokens into the 14B shape's 34816
+    gate and up outputs: 544 tiles, 210 us, of which the last 32 take 80); split in four it
+    takes a quarter of that, plus what the partials cost: 128 KB a workgroup, written and read
+    again, and a second kernel.  The split that the estimate below likes best is taken if it
+    saves a fifth of the round or more, which on MI355X (Qwen3-8B and 14B widths, 512 to 4096
+    tokens) is where the measured gain begins: 210 -> 165 us above, 768 tokens into 24576
+    outputs 156 -> 131, 1024 into 34816 339 -> 307; a last round of more than about 100 tiles
+    stays whole (168 tiles in three parts: 210 -> 255 us).  Only splits that leave every part
+    an even number of k-tiles, which the kernel's deeper prefetch of W needs."""
+    if K % 128 != 0:
+        return None
+    tiles = ((M + 127) // 128) * ((N + 255) // 256)
+    whole = tiles // TILE_PLACES * TILE_PLACES
+    tail = tiles - whole
+    if whole == 0 or tail == 0 or whole > 2 * TILE_PLACES:
+        return None         # (behind three rounds and more the workgroups no longer end together)
+    kt = K // 64
+    per = 2.0 * 128 * 256 * K
+    pair, alone = _TILE128_RATE[10]
+
+    def last_round(workgroups: int, flop: float) -> float:
+        return flop / alone if workgroups <= 256 else 2 * flop / pair
+    best, best_t = None, 0.8 * last_round(tail, per)
+    for split in (2, 4, 8):
+        if tail * split > TILE_PLACES or kt % (2 * split) != 0 or kt // split < 8:
+            continue
+        t = last_round(tail * split, per / split) + 8e-6 + tail * split * 128 * 256 * 4 * 2 / 3e12
+        if t < best_t:
+            best, best_t = split, t
+    return None if best is None else (whole, best)
+
+
 def _tile128_time(M: int, N: int, K: int, variant: int, ksplit: int) -> float:
     """Estimated seconds of the 128-token tile kernels: rounds of up to 512 tiles, two to a CU
     (a last round of up to 256 tiles runs one to a CU, each faster than two)."""
@@ -711,7 +750,14 @@ def _tile128_time(M: int, N: int, K: int, variant: int, ksplit: int) -> float:
     per = 2.0 * 128 * bn * (K / ksplit)
     pair, alone = _TILE128_RATE[variant if ksplit == 1 else 6]
     rem = tiles % 512
-    t = (tiles // 512) * 2 * per / pair + (0.0 if rem == 0 else per / alone if rem <= 256 else 2 * per / pair)
+    tail = _tile_tail_split(M, N, K) if variant == 10 and ksplit == 1 else None
+    if tail is not None:    # the last round split along K, its partials written and read again
+        part, wgs = per / tail[1], rem * tail[1]
+        last = (part / alone if wgs <= 256 else 2 * part / pair) + 8e-6 \
+            + wgs * 128 * 256 * 4 * 2 / 3e12
+    else:
+        last = 0.0 if rem == 0 else per / alone if rem <= 256 else 2 * per / pair
+    t = (tiles // 512) * 2 * per / pair + last
     if ksplit > 1:      # the partials, written and read again, and the second launch
         t += 4e-6 + M * N * 4.0 * ksplit * 2 / 4e12
     return t + 4e-6
@@ -757,12 +803,24 @@ def pretile_weight(w: torch.Tensor) -> torch.Tensor:
     return t.view(N, K)
 
 
+def _gemm_tile_tail(lib, a, w, out, M: int, N: int, K: int, epi: int, tail) -> None:
+    whole, split = tail
+    tiles = ((M + 127) // 128) * ((N + 255) // 256)
+    if not (0 <= whole < tiles and split >= 2):
+        raise KernelUnavailable(f"gemm: tail split {tail} of {tiles} tiles")
+    ws = _workspace("gemm_tile_tail", (tiles - whole) * split * 128 * 256, torch.float32, a.device)
+    _check(lib.zf_gemm_bf16_tile_tail(_ptr(a), _ptr(w), _ptr(out), _ptr(ws), M, N, K, epi, whole,
+                                      split, _stream()), "gemm (tiled, last round split along K)")
+
+
 @_launches("products")
 def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
-         w_tiled: bool = False, tile_variant: Optional[int] = None) -> None:
+         w_tiled: bool = False, tile_variant: Optional[int] = None,
+         tile_tail: Optional[Tuple[int, int]] = None) -> None:
     """out = a w^T (w is [N, K]); with ``accumulate`` out += a w^T, in 32-bit.  ``w_tiled``:
     ``w`` went through ``pretile_weight``.  ``tile_variant`` (tests and measurements): this
-    tiled kernel, whatever the number of rows.
+    tiled kernel, whatever the number of rows; ``tile_tail`` (whole, split): the 128 x 256
+    tiles with the tiles from ``whole`` on split along K (``_tile_tail_split``).
 
     bfloat16 operands with K a multiple of 8 go to the MFMA kernels (weight streaming for up
     to 16 rows of ``a``, and up to 64 where the kernel for 17 to 128 rows does not cover the
@@ -783,7 +841,9 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         epi = _EPI_ACC_F32 if accumulate else \
             (_EPI_STORE_BF16 if out.dtype == torch.bfloat16 else _EPI_STORE_F32)
         plan = _small_plan(M, N, K, w_tiled) if M > 16 else None
-        if tile_variant is not None:
+        if tile_tail is not None:
+            _gemm_tile_tail(lib, a, w, out, M, N, K, epi, tile_tail)
+        elif tile_variant is not None:
             _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, epi, tile_variant,
                                          1 if w_tiled else 0, _stream()), "gemm (tiled)")
         elif plan is not None and plan[0] == "mid":
@@ -813,8 +873,12 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
                                                     K, epi, ksplit, _stream()),
                        "gemm (tiled, split along K)")
                 return
-            _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, epi,
-                                         _tile_variant(M, N, w_tiled, accumulate, K),
+            variant = _tile_variant(M, N, w_tiled, accumulate, K)
+            tail = _tile_tail_split(M, N, K) if variant == 10 else None
+            if tail is not None:
+                _gemm_tile_tail(lib, a, w, out, M, N, K, epi, tail)
+                return
+            _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, epi, variant,
                                          1 if w_tiled else 0, _stream()),
                    "gemm (tiled)")
         return
@@ -1016,7 +1080,8 @@ def can_fuse_swiglu(w: torch.Tensor) -> bool:
 
 @_launches("products")
 def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bool = False,
-                tile_variant: Optional[int] = None) -> None:
+                tile_variant: Optional[int] = None,
+                tile_tail: Optional[Tuple[int, int]] = None) -> None:
     """out[M, I] = silu(a Wg^T) * (a Wu^T) as bfloat16, with ``w`` [2 I, K] from
     ``interleave_gate_up`` (then possibly ``pretile_weight``): the activation is applied to
     the 32-bit sums in the product's epilogue, nothing of width 2 I is written."""
@@ -1031,7 +1096,9 @@ def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bo
         return
     lib = build.load("gemm")
     plan = _small_plan(M, N, K, w_tiled, swiglu=True) if M > 16 else None
-    if tile_variant is not None:
+    if tile_tail is not None:
+        _gemm_tile_tail(lib, a, w, out, M, N, K, _EPI_SWIGLU, tile_tail)
+    elif tile_variant is not None:
         _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, _EPI_SWIGLU,
                                      tile_variant, 1 if w_tiled else 0, _stream()),
                "gemm_swiglu (tiled)")
@@ -1045,10 +1112,13 @@ def gemm_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: bo
                "gemm_swiglu (weight streaming)")
     else:
         big = _tile256_variant(M, N, K) if w_tiled else None
-        _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, _EPI_SWIGLU,
-                                     big if big is not None else
-                                     _tile_variant(M, N, w_tiled, False, K), 1 if w_tiled else 0,
-                                     _stream()),
+        variant = big if big is not None else _tile_variant(M, N, w_tiled, False, K)
+        tail = _tile_tail_split(M, N, K) if variant == 10 else None
+        if tail is not None:
+            _gemm_tile_tail(lib, a, w, out, M, N, K, _EPI_SWIGLU, tail)
+            return
+        _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, _EPI_SWIGLU, variant,
+                                     1 if w_tiled else 0, _stream()),
                "gemm_swiglu (tiled)")
 
 
