@@ -478,7 +478,7 @@ def main_decode(args) -> int:
             d, ctx = run_decode(llm, cfg, b, args.prompt_len, k, args.warmup, args.seed + 3 + b)
             points[f"decode_b{b}"] = round(b * k / d, 1)
             points[f"decode_b{b}_hbm_frac"] = decode_roofline(cfg, elem, b, ctx, d / k)["frac"]
-        for T in (512, 8192):
+        for T in (512, 1024, 8192):
             s = run_prefill(llm, cfg, T, args.seed + 5)
             points[f"prefill_{T}"] = round(T / s, 1)
             points[f"prefill_{T}_frac"] = round(prefill_flops(cfg, T) / s / peak, 4)

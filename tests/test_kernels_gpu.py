@@ -168,7 +168,9 @@ def test_gemm_17_to_128_tokens(M, N, K, kind):
                          # widths with measured plans: the weight-streaming kernel split along K
                          # at 1 to 16 tokens and at 17 to 32, the other kernel above
                          + [(1, 5120, 17408), (8, 5120, 17408), (16, 5120, 25600), (17, 5120, 5120),
-                            (24, 5120, 17408), (32, 5120, 8192), (40, 5120, 5120), (64, 4096, 12288)])
+                            (24, 5120, 17408), (32, 5120, 8192), (40, 5120, 5120), (64, 4096, 12288)]
+                         # several hundred tokens on a long K: 128 x 256 tiles split along K
+                         + [(700, 512, 8192), (1030, 1344, 8448), (1280, 320, 12288)])
 def test_gemm_sum_norm(M, N, K):
     """The residual sum whose split-K partials are added, summed into the residual and normed
     by one kernel, against sum and norm in 64-bit.  Tokens of different scale: another row's
@@ -185,6 +187,8 @@ def test_gemm_sum_norm(M, N, K):
         pytest.skip("this product is not split along K: the norm runs on its own")
     if (N, K) in ((5120, 17408), (5120, 25600), (5120, 5120), (5120, 8192)) and M <= 32:
         assert plan[0] == "skinny" and plan[-1] >= 2, plan
+    if M > 640:
+        assert plan[0] == "wide" and (K // 64) % (2 * plan[1]) == 0, plan
     x = base.double() + a.double() @ w.double().T
     want = torch.empty((M, N), dtype=torch.float64)
     ref.rmsnorm(x, gain, eps, want)

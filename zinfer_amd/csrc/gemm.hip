@@ -1038,7 +1038,7 @@ static int launch_tile_wdirect(const void* A, const void* W, void* C, int M, int
                                hipStream_t stream, void* ws = nullptr, int ksplit = 1,
                                bool reduce = true) {
   if (N % 16 != 0 || K % TKM != 0) return -3;
-  if (W2 && (ksplit != 1 || (K / TKM) % 2 != 0)) return -3;
+  if (W2 && (K / TKM) % (2 * ksplit) != 0) return -3;     // every part an even number of k-tiles
   if (ksplit > 1 && (ws == nullptr || epi == EPI_SWIGLU || ksplit > K / TKM)) return -3;
   constexpr int NT = (BM / WM) * (BN / WN) * 64;
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
@@ -1718,6 +1718,35 @@ extern "C" int zf_gemm_bf16_splitk_sum_norm(const void* A, const void* W, void* 
                                                false);
   if (rc != 0) return rc;
   // a thread per 4 columns up to 1024 threads: every load of a row is in flight at once
+  const int threads = N / 4 >= 1024 ? 1024 : (N / 4 > 256 ? 512 : 256);
+  hipLaunchKernelGGL(reduce_sum_norm_kernel, dim3(M), dim3(threads), 0, stream, (const float*)ws,
+                     (float*)C, gain, (bf16_t*)normed, M, N, ksplit, eps);
+  return (int)hipGetLastError();
+}
+
+// The product with 128 x 256 tiles split along K (for a long K on a narrow output at several
+// hundred tokens) and the kernel that adds the partials.  (K / 64) % (2 ksplit) == 0; ws:
+// float32 [ksplit, M, N]; epi: store bf16, store f32 or add into f32.
+extern "C" int zf_gemm_bf16_wide_splitk(const void* A, const void* W, void* C, void* ws, int M,
+                                        int N, int K, int epi, int ksplit, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (ksplit < 2 || ksplit > 64 || epi == EPI_SWIGLU || ws == nullptr) return -3;
+  return launch_tile_wdirect<128, 256, 128, 64, TK, true, true>(A, W, C, M, N, K, epi, stream, ws,
+                                                                ksplit);
+}
+
+// The same with 128 x 256 tiles (two workgroups to a CU, no two waves load the same part of
+// W): for a long K on a narrow output, where few of these tiles, each split many times, run
+// faster than the 128 x 128 tiles.  (K / 64) % (2 ksplit) == 0.
+extern "C" int zf_gemm_bf16_wide_splitk_sum_norm(const void* A, const void* W, void* C, void* ws,
+                                                 const float* gain, float eps, void* normed,
+                                                 int M, int N, int K, int ksplit,
+                                                 hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (ksplit < 2 || ksplit > 64 || N % 16 != 0 || N > 8192 || ws == nullptr) return -3;
+  const int rc = launch_tile_wdirect<128, 256, 128, 64, TK, true, true>(
+      A, W, C, M, N, K, EPI_ACC_F32, stream, ws, ksplit, false);
+  if (rc != 0) return rc;
   const int threads = N / 4 >= 1024 ? 1024 : (N / 4 > 256 ? 512 : 256);
   hipLaunchKernelGGL(reduce_sum_norm_kernel, dim3(M), dim3(threads), 0, stream, (const float*)ws,
                      (float*)C, gain, (bf16_t*)normed, M, N, ksplit, eps);

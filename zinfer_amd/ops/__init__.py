@@ -861,6 +861,13 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
             _check(lib.zf_gemm_bf16_mid(_ptr(a), _ptr(w), _ptr(out), _ptr(None), M, N, K, epi, 1,
                                         _stream()), "gemm (64-token tiles)")
         else:
+            wide = _wide_ksplit(M, N, K) if w_tiled and accumulate else None
+            if wide is not None:        # as gemm_sum_norm runs it: the same bits
+                ws = _workspace("gemm_splitk", wide * M * N, torch.float32, a.device)
+                _check(lib.zf_gemm_bf16_wide_splitk(_ptr(a), _ptr(w), _ptr(out), _ptr(ws), M, N, K,
+                                                    epi, wide, _stream()),
+                       "gemm (128 x 256 tiles, split along K)")
+                return
             big = _tile256_variant(M, N, K, accumulate) if w_tiled else None
             if big is not None:
                 _check(lib.zf_gemm_bf16_tile(_ptr(a), _ptr(w), _ptr(out), M, N, K, epi, big, 1,
@@ -961,7 +968,7 @@ def sum_norm_plan(M: int, N: int, K: int, w: torch.Tensor, w_tiled: bool):
     """The plan if ``gemm_sum_norm`` covers residual += a w^T: a product that is split along K
     anyway (by measurement at 1 to 64 tokens, by rule at 17 to 128, or a few hundred tokens on
     a narrow output), whose partials one kernel can add, sum into the residual and norm; else
-    None.  ('mid' | 'tile' | 'skinny', [row groups per workgroup,] workgroups along K)."""
+    None.  ('mid' | 'tile' | 'wide' | 'skinny', [row groups per workgroup,] workgroups along K)."""
     if not (w_tiled and w.dtype == torch.bfloat16 and w.is_cuda and N % 16 == 0 and N <= 8192):
         return None
     if M <= NORM_FOLD_MAX_M:
@@ -969,8 +976,28 @@ def sum_norm_plan(M: int, N: int, K: int, w: torch.Tensor, w_tiled: bool):
     if M <= MID_MAX_M:
         plan = _small_plan(M, N, K, True)
         return plan if plan is not None and plan[-1] >= 2 else None
+    wide = _wide_ksplit(M, N, K)
+    if wide is not None:
+        return ("wide", wide)
     ks = _tile_ksplit(M, N, K)
     return ("tile", ks) if ks >= 2 else None
+
+
+def _wide_ksplit(M: int, N: int, K: int):
+    """Workgroups along K if a residual sum with the norm behind it should run through 128 x
+    256 tiles split along K: 641 to 1280 tokens on a long K, where those tiles alone leave
+    half the chip idle (1024 tokens into 4096 outputs: 128 of them) and the 128 x 128 tiles,
+    split or not, are slower per flop.  Two to four parts of an even number of k-tiles each,
+    as close to 512 workgroups as they get.  Measured on MI355X against what ran before (the
+    norm's kernel included): K = 12288 into 4096 at 768 / 1024 / 1280 tokens 113 -> 107, 133
+    -> 113, 171 -> 143 us; K = 17408 into 5120 174 -> 149, 222 -> 209, 254 -> 244; K = 25600
+    253 -> 205 and 314 -> 289.  With K = 4096 or 5120 the partials cost what the split gains,
+    and from 1536 tokens on the tiles fill the chip without it."""
+    if not (640 < M <= 1280 and K >= 8192 and K % 128 == 0 and N % 16 == 0):
+        return None
+    tiles = ((M + 127) // 128) * ((N + 255) // 256)
+    fits = [ks for ks in (2, 3, 4) if (K // 64) % (2 * ks) == 0]
+    return min(fits, key=lambda ks: abs(tiles * ks - TILE_PLACES)) if fits else None
 
 
 @_launches("products")
@@ -993,7 +1020,12 @@ def gemm_sum_norm(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, gain
     ks = plan[-1]
     ws = _workspace("gemm_splitk", ks * M * N, torch.float32, a.device)
     lib = build.load("gemm")
-    if plan[0] == "skinny":
+    if plan[0] == "wide":
+        _check(lib.zf_gemm_bf16_wide_splitk_sum_norm(_ptr(a), _ptr(w), _ptr(residual), _ptr(ws),
+                                                     _ptr(gain), ctypes.c_float(eps), _ptr(normed),
+                                                     M, N, K, ks, _stream()),
+               "gemm_sum_norm (128 x 256 tiles)")
+    elif plan[0] == "skinny":
         _check(lib.zf_gemm_bf16_skinny_sum_norm(_ptr(a), _ptr(w), _ptr(residual), _ptr(ws),
                                                 _ptr(gain), ctypes.c_float(eps), _ptr(normed), M, N,
                                                 K, plan[1], ks, _stream()),
