@@ -136,3 +136,90 @@ def test_random_orders_lose_nothing(seed, window):
         m.release(rid)
     m.check()
     assert all(g.pages.num_free == g.pages.num_pages for g in m.groups)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_native_bookkeeping_follows_the_plain_model(seed):
+    """The native core against a plain model in lists and dicts, call by call under a random
+    order of calls (requests that come, grow in portions, are cut back, end; two groups, one
+    with a window; few pages, so that they run out and are used again): the same block tables
+    page for page, the same free pages and slots, the same answers to what is missing and
+    what fits, the same refusals; and the step tables the core packs are the tables' pages."""
+    import numpy as np
+    from plain_cache import Full, Misuse, PlainCache
+    rng = random.Random(100 + seed)
+    ps, num_pages, max_requests = rng.choice([2, 4, 16]), rng.choice([6, 9, 14]), 3
+    window = rng.choice([3, 7, 20])
+    needs = [KVNeed(1, 4), KVNeed(1, 4, window)]
+    m = CacheManager(needs, [None, None], ps, num_pages, max_requests, torch.float32, "cpu")
+    plain = PlainCache([None, window], ps, num_pages, max_requests)
+    names = ["a", "b", "c", "d", "e"]
+    packed = 0
+    for _ in range(600):
+        rid = rng.choice(names)
+        live = m.has_request(rid)
+        assert live == (rid in plain.requests)
+        op = rng.choice(["add", "grow", "grow", "grow", "trim", "release", "ask"])
+        new_len = (m.length(rid) if live else 0) + rng.randint(0, 3 * ps)
+        assert m.pages_missing(rid, new_len) == plain.pages_missing(rid, new_len)
+        other = rng.choice(names)
+        wanted = [(rid, new_len), (other, rng.randint(1, 4 * ps) +
+                                   (m.length(other) if m.has_request(other) else 0))]
+        assert m.can_reserve(wanted) == plain.can_reserve(wanted)
+        outcome = []
+        for cache, full, misuse in ((m, CacheFull, StepError), (plain, Full, (Misuse, KeyError))):
+            try:
+                if op == "add":
+                    cache.add_request(rid)
+                elif op == "grow":
+                    cache.reserve(rid, new_len)
+                elif op == "trim":
+                    cache.trim(rid)
+                elif op == "release":
+                    cache.release(rid)
+                outcome.append("ok")
+            except full:
+                outcome.append("full")
+            except misuse:
+                outcome.append("misuse")
+        assert outcome[0] == outcome[1], (op, rid, outcome)
+        if op == "grow" and outcome[0] == "ok" and rng.random() < 0.8:
+            m.commit(rid, new_len)
+            plain.commit(rid, new_len)
+        for r, rec in plain.requests.items():
+            assert m.length(r) == rec["length"] and m.state_slot(r) == rec["slot"]
+            for g in range(2):
+                assert m.table(g, r) == rec["tables"][g], (op, rid, r, g)
+        assert m.num_free_pages() == [len(p.free_list) for p in plain.pools]
+        assert m.num_free_slots() == len(plain.slots.free_list)
+        assert [g.pages.handed_out for g in m.groups] == [p.handed_out for p in plain.pools]
+        m.check()
+        # a step of the live requests that hold something: one more token each
+        step = [r for r in plain.requests if plain.requests[r]["length"] > 0]
+        if step and all(m.pages_missing(r, m.length(r) + 1) == [0, 0] for r in step):
+            for g in range(2):
+                starts = [m.length(r) - 1 for r in step]       # the last token held, again
+                width = max(len(plain.requests[r]["tables"][g]) for r in step) + 1
+                table = np.empty((len(step), width), dtype=np.int32)
+                slots = np.empty((len(step),), dtype=np.int32)
+                m.pack_step(g, step, starts, [1] * len(step), width, table, slots)
+                packed += 1
+                for i, r in enumerate(step):
+                    t = plain.requests[r]["tables"][g]
+                    assert list(table[i]) == t + [NO_PAGE] * (width - len(t))
+                    assert slots[i] == t[starts[i] // ps] * ps + starts[i] % ps
+    assert packed > 20
+    # several tokens of a request in one step, and a token whose page is not held
+    for r, rec in plain.requests.items():
+        n, t = rec["length"], rec["tables"][0]
+        if n < 2:
+            continue
+        table = np.empty((1, len(t)), dtype=np.int32)
+        slots = np.empty((n - 1,), dtype=np.int32)
+        m.pack_step(0, [r], [1], [n - 1], len(t), table, slots)
+        assert list(slots) == [t[p // ps] * ps + p % ps for p in range(1, n)]
+        if plain._first_needed(1, n) > 0:       # the window has passed the first page
+            with pytest.raises(StepError, match="not held"):
+                m.pack_step(1, [r], [0], [n], len(rec["tables"][1]),
+                            np.empty((1, len(rec["tables"][1])), dtype=np.int32),
+                            np.empty((n,), dtype=np.int32))

@@ -645,7 +645,6 @@ def test_debug_tables_finds_a_page_that_is_not_the_pools(tmp_path_factory):
     lg = eng.step([StepEntry("x", [1] * 40, [39]), StepEntry("y", [2] * 5, [4])])
     assert lg.shape[0] == 2
     eng.step([StepEntry("x", [3], [0]), StepEntry("y", [4], [0])])      # a graph-captured step
-    table = eng.cache.table(0, "x")
-    table[1] = eng.cache.groups[0].pages.num_pages + 7
+    eng.cache.set_table_entry(0, "x", 1, eng.cache.groups[0].pages.num_pages + 7)
     with pytest.raises(StepError, match=r"BlockTableOutOfBounds: group 0, sequence 1, page index 1"):
         eng.step([StepEntry("y", [5], [0]), StepEntry("x", [6], [0])])

@@ -15,14 +15,16 @@ hands out pages; the layout inside a page belongs to the kernels.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+import ctypes
+from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
-from ..errors import CacheFull, StepError
+from ..errors import StepError
 from ..parts.base import KVNeed, StateNeed
-from .pages import PageAllocator
+from .pages import PoolCounts, core_lib, raise_for
 
 NO_PAGE = -1
 
@@ -38,14 +40,33 @@ class LayerCacheView:
     state: Optional[torch.Tensor]    # [max_requests, *shape] for a StateNeed
 
 
+class _GroupPages(PoolCounts):
+    """The counts of one group's pool of pages (or, group -1, of the request slots)."""
+
+    def __init__(self, manager: "CacheManager", group: int):
+        self._manager, self._group = manager, group
+
+    def _counts(self):
+        lib, h = self._manager._lib, self._manager._core
+        what = (ctypes.c_int * 4)()
+        handed = ctypes.c_longlong()
+        if self._group < 0:
+            lib.zc_slot_counts(h, what)
+        else:
+            lib.zc_group_counts(h, self._group, what, ctypes.byref(handed))
+        return what[0], what[1], what[2], what[3], handed.value
+
+
 class KVGroup:
+    """The pools of one group of layers with the same need; which of their pages are free and
+    which request holds which is the native core's to know (``pages``: its counts)."""
+
     def __init__(self, need: KVNeed, runs: List[int], page_size: int, num_pages: int,
-                 dtype: torch.dtype, device):
+                 dtype: torch.dtype, device, pages: PoolCounts):
         self.need = need
         self.runs = runs                     # schedule positions that own a cache here
         self.page_size = page_size
-        self.pages = PageAllocator(num_pages)
-        self.tables: Dict[object, List[int]] = {}
+        self.pages = pages
         # a need may bring its own dtype and a value row of another width than a key's
         dtype = need.dtype or dtype
         self.k = torch.zeros((len(runs), num_pages, need.n_kv_heads * page_size * need.key_width),
@@ -53,24 +74,12 @@ class KVGroup:
         self.v = torch.zeros((len(runs), num_pages, need.n_kv_heads * page_size * need.value_width),
                              dtype=dtype, device=device)
 
-    def first_needed_page(self, length: int) -> int:
-        """Logical index of the first page a query at position >= ``length`` can still read."""
-        if self.need.window is None:
-            return 0
-        return max(0, length - self.need.window + 1) // self.page_size
-
-    def pages_missing(self, rid, length: int, new_len: int) -> int:
-        table = self.tables[rid]
-        last = (new_len + self.page_size - 1) // self.page_size
-        if self.need.window is None:       # no holes: every page up to len(table) is held
-            return max(0, last - len(table))
-        first = self.first_needed_page(length)
-        return sum(1 for i in range(first, last) if i >= len(table) or table[i] == NO_PAGE)
-
 
 class CacheManager:
     """``needs[pos]`` is the cache need of schedule position ``pos`` (None: no cache of its
-    own); ``reads[pos]`` names the position whose cache a run reads instead."""
+    own); ``reads[pos]`` names the position whose cache a run reads instead.  The pools are
+    tensors of this class; which pages are free, the block tables and the slots are kept by
+    the native core, where a request goes by a number that this class gives it."""
 
     def __init__(self, needs: Sequence[object], reads: Sequence[Optional[int]], page_size: int,
                  num_pages: int, max_requests: int, kv_dtype: torch.dtype, device,
@@ -92,15 +101,49 @@ class CacheManager:
                                                     dtype=need.dtype, device=device)
             elif need is not None:
                 raise StepError(f"unknown cache need {need!r}")
+        self._lib = core_lib()
+        windows = [-1 if need.window is None else int(need.window) for need in by_need]
+        self._core = ctypes.c_void_p(self._lib.zc_create(
+            len(windows), (ctypes.c_int * max(len(windows), 1))(*windows), int(page_size),
+            int(num_pages), int(max_requests)))
+        if not self._core:
+            raise ValueError(f"a cache of {num_pages} pages of {page_size} tokens for "
+                             f"{max_requests} requests cannot be made")
         self._where: Dict[int, Tuple[int, int]] = {}     # schedule position -> (group, run)
         for need, runs in by_need.items():
             g = len(self.groups)
-            self.groups.append(KVGroup(need, runs, page_size, num_pages, kv_dtype, device))
+            self.groups.append(KVGroup(need, runs, page_size, num_pages, kv_dtype, device,
+                                       _GroupPages(self, g)))
             for i, pos in enumerate(runs):
                 self._where[pos] = (g, i)
         self._reads = list(reads)
-        self._slots = PageAllocator(max_requests)        # state slots, same bookkeeping
-        self.requests: Dict[object, dict] = {}
+        self._slots = _GroupPages(self, -1)              # state slots, same bookkeeping
+        self.requests: Dict[object, int] = {}            # live request -> its number in the core
+        self._names: Dict[int, object] = {}
+        self._next_number = 0
+
+    def __del__(self):
+        core, self._core = getattr(self, "_core", None), None
+        if core:
+            self._lib.zc_destroy(core)
+
+    def _number(self, rid) -> int:
+        try:
+            return self.requests[rid]
+        except KeyError:
+            raise StepError(f"request {rid!r} is not live") from None
+
+    def _raise(self, code: int) -> None:
+        """The core's error with the request's own name in place of its number."""
+        if code == 0:
+            return
+        try:
+            raise_for(code, StepError)
+        except Exception as e:  # noqa: BLE001 - re-raised with the name put in
+            text = str(e)
+            for number, rid in self._names.items():
+                text = text.replace(f"request #{number} ", f"request {rid!r} ")
+            raise type(e)(text) from None
 
     # ------------------------------------------------------------------ views
     def view(self, pos: int) -> LayerCacheView:
@@ -117,89 +160,57 @@ class CacheManager:
         return rid in self.requests
 
     def length(self, rid) -> int:
-        return self.requests[rid]["length"]
+        out = ctypes.c_int()
+        self._raise(self._lib.zc_length(self._core, self._number(rid), ctypes.byref(out)))
+        return out.value
 
     def state_slot(self, rid) -> int:
-        return self.requests[rid]["slot"]
+        out = ctypes.c_int()
+        self._raise(self._lib.zc_state_slot(self._core, self._number(rid), ctypes.byref(out)))
+        return out.value
 
     def add_request(self, rid) -> None:
         if rid in self.requests:
             raise StepError(f"request {rid!r} is already live")
-        if self._slots.num_free == 0:
-            raise CacheFull(f"CacheFull: all {self.max_requests} request slots are in use")
-        slot = self._slots.alloc(1)[0]
+        number, slot = self._next_number, ctypes.c_int()
+        self._raise(self._lib.zc_add_request(self._core, number, ctypes.byref(slot)))
+        self._next_number += 1
+        self.requests[rid] = number
+        self._names[number] = rid
         for pool in self.state_pools.values():
-            pool[slot].zero_()
-        self.requests[rid] = {"length": 0, "slot": slot}
-        for grp in self.groups:
-            grp.tables[rid] = []
+            pool[slot.value].zero_()
+
+    def _number_or_new(self, rid) -> int:
+        return self.requests.get(rid, -1)        # no request has the number -1: "not yet live"
 
     def pages_missing(self, rid, new_len: int) -> List[int]:
         """Pages each group would have to hand out for ``rid`` (live or not yet) to hold
         ``new_len`` tokens."""
-        if rid in self.requests:
-            length = self.requests[rid]["length"]
-            return [grp.pages_missing(rid, length, new_len) for grp in self.groups]
-        last = (new_len + self.page_size - 1) // self.page_size
-        return [last - grp.first_needed_page(0) for grp in self.groups]
+        out = (ctypes.c_int * max(len(self.groups), 1))()
+        self._lib.zc_pages_missing(self._core, self._number_or_new(rid), int(new_len), out)
+        return list(out[:len(self.groups)])
 
     def can_reserve(self, wanted: Sequence[Tuple[object, int]]) -> bool:
         """Whether all ``(request, new_len)`` of a step fit together."""
-        total = [0] * len(self.groups)
-        new = 0
-        for rid, new_len in wanted:
-            if rid not in self.requests:
-                new += 1
-            for g, n in enumerate(self.pages_missing(rid, new_len)):
-                total[g] += n
-        return new <= self._slots.num_free and \
-            all(t <= grp.pages.num_free for t, grp in zip(total, self.groups))
+        n = len(wanted)
+        rids = (ctypes.c_longlong * max(n, 1))(*[self._number_or_new(r) for r, _ in wanted])
+        lens = (ctypes.c_int * max(n, 1))(*[int(l) for _, l in wanted])
+        return bool(self._lib.zc_can_reserve(self._core, n, rids, lens))
 
     def reserve(self, rid, new_len: int) -> None:
         """Pages for positions up to ``new_len`` (all groups or none)."""
-        req = self.requests[rid]
-        if new_len < req["length"]:
-            raise StepError(f"request {rid!r} holds {req['length']} tokens, cannot shrink to "
-                            f"{new_len}")
-        missing = self.pages_missing(rid, new_len)
-        for n, grp in zip(missing, self.groups):
-            if n > grp.pages.num_free:
-                raise CacheFull(f"CacheFull: request {rid!r} needs {n} more pages of "
-                                f"{self.page_size} tokens, {grp.pages.num_free} of "
-                                f"{grp.pages.num_pages} free")
-        for grp in self.groups:
-            table = grp.tables[rid]
-            last = (new_len + self.page_size - 1) // self.page_size
-            first = grp.first_needed_page(req["length"])
-            while len(table) < last:
-                table.append(NO_PAGE)
-            for i in range(first, last):
-                if table[i] == NO_PAGE:
-                    table[i] = grp.pages.alloc(1)[0]
+        self._raise(self._lib.zc_reserve(self._core, self._number(rid), int(new_len)))
 
     def commit(self, rid, new_len: int) -> None:
         """The request now holds ``new_len`` tokens; pages a window has passed go back."""
-        req = self.requests[rid]
-        req["length"] = new_len
-        for grp in self.groups:
-            if grp.need.window is None:
-                continue
-            table = grp.tables[rid]
-            first = grp.first_needed_page(new_len)
-            gone = [i for i in range(min(first, len(table))) if table[i] != NO_PAGE]
-            self._give_back(grp, [table[i] for i in gone])
-            for i in gone:
-                table[i] = NO_PAGE
+        self._raise(self._lib.zc_commit(self._core, self._number(rid), int(new_len)))
+        self._poison_freed()
 
     def trim(self, rid) -> None:
         """Gives back the pages reserved beyond the tokens the request holds (a step that
         reserved them did not run)."""
-        req = self.requests[rid]
-        keep = (req["length"] + self.page_size - 1) // self.page_size
-        for grp in self.groups:
-            table = grp.tables[rid]
-            self._give_back(grp, [p for p in table[keep:] if p != NO_PAGE])
-            del table[keep:]
+        self._raise(self._lib.zc_trim(self._core, self._number(rid)))
+        self._poison_freed()
 
     def pages_at_most(self, n_tokens: int, portion: int) -> List[int]:
         """Upper bound, per group, of the pages a request of ``n_tokens`` tokens holds at any
@@ -218,18 +229,24 @@ class CacheManager:
 
     def release(self, rid) -> None:
         """Everything the request holds goes back: pages of every group and the state slot."""
-        req = self.requests.pop(rid, None)
-        if req is None:
-            raise StepError(f"request {rid!r} is not live")
-        for grp in self.groups:
-            table = grp.tables.pop(rid)
-            self._give_back(grp, [p for p in table if p != NO_PAGE])
-        self._slots.free([req["slot"]])
+        number = self._number(rid)
+        self._raise(self._lib.zc_release(self._core, number))
+        del self.requests[rid]
+        del self._names[number]
+        self._poison_freed()
 
-    def _give_back(self, grp: KVGroup, pages: List[int]) -> None:
-        if not pages:
+    def _poison_freed(self) -> None:
+        """(debugging) What the last call gave back is overwritten with NaN, so that a kernel
+        that reads a page it does not hold shows."""
+        if not self.poison_freed:
             return
-        if self.poison_freed:
+        for g, grp in enumerate(self.groups):
+            cap = grp.pages.num_pages
+            out = (ctypes.c_int * max(cap, 1))()
+            n = self._lib.zc_last_freed(self._core, g, out, cap)
+            if n == 0:
+                continue
+            pages = list(out[:n])
             if grp.k.is_cuda:
                 from .. import ops
                 idx = torch.tensor(pages, dtype=torch.int32, device=self.device)
@@ -239,10 +256,42 @@ class CacheManager:
                 idx = torch.tensor(pages, dtype=torch.long, device=self.device)
                 grp.k[:, idx] = float("nan")
                 grp.v[:, idx] = float("nan")
-        grp.pages.free(reversed(pages))
 
     def table(self, group: int, rid) -> List[int]:
-        return self.groups[group].tables[rid]
+        """A copy of the request's block table in a group."""
+        number = self._number(rid)
+        cap = self.groups[group].pages.num_pages + 1
+        while True:
+            out = (ctypes.c_int * cap)()
+            n = self._lib.zc_table(self._core, group, number, out, cap)
+            if n <= cap:
+                return list(out[:n])
+            cap = n
+
+    def set_table_entry(self, group: int, rid, index: int, page: int) -> None:
+        """(debugging) Plants ``page`` in a block table, whatever the pool says: what the
+        device-side check of a step's tables is tested with."""
+        self._raise(self._lib.zc_set_table_entry(self._core, group, self._number(rid),
+                                                 int(index), int(page)))
+
+    def pack_step(self, group: int, rids: Sequence[object], starts: Sequence[int],
+                  q_lens: Sequence[int], max_pages: int, table_out: np.ndarray,
+                  slots_out: np.ndarray) -> None:
+        """A step's block tables ``table_out`` [n, max_pages] (``NO_PAGE`` where a request has
+        none) and slot mapping ``slots_out`` [sum of q_lens] (page * page_size + row of every
+        token's own key and value) of one group, written into int32 arrays of the caller's."""
+        n = len(rids)
+        if table_out.dtype != np.int32 or slots_out.dtype != np.int32 \
+                or not table_out.flags.c_contiguous or not slots_out.flags.c_contiguous \
+                or table_out.size != n * max_pages or slots_out.size != sum(q_lens):
+            raise StepError("pack_step: int32 arrays [n, max_pages] and [tokens] are needed")
+        numbers = (ctypes.c_longlong * max(n, 1))(*[self._number(r) for r in rids])
+        s = (ctypes.c_int * max(n, 1))(*[int(x) for x in starts])
+        q = (ctypes.c_int * max(n, 1))(*[int(x) for x in q_lens])
+        self._raise(self._lib.zc_pack_group(
+            self._core, group, n, numbers, s, q, int(max_pages),
+            table_out.ctypes.data_as(ctypes.POINTER(ctypes.c_int)),
+            slots_out.ctypes.data_as(ctypes.POINTER(ctypes.c_int))))
 
     # ------------------------------------------------------------------ accounting
     def num_free_slots(self) -> int:
@@ -257,11 +306,5 @@ class CacheManager:
 
     def check(self) -> None:
         """No page lost, none held twice: the pages in all tables are exactly the held ones."""
-        for grp in self.groups:
-            grp.pages.check()
-            held = [p for t in grp.tables.values() for p in t if p != NO_PAGE]
-            assert len(held) == len(set(held)), "a page is in two tables"
-            assert len(held) == grp.pages.num_held, "held pages and tables disagree"
-        self._slots.check()
-        slots = [r["slot"] for r in self.requests.values()]
-        assert len(slots) == len(set(slots)) == self._slots.num_held
+        code = self._lib.zc_check(self._core)
+        assert code == 0, self._lib.zc_last_error().decode()

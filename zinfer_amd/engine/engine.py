@@ -13,7 +13,7 @@ from typing import Dict, List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..cache import NO_PAGE, CacheManager
+from ..cache import CacheManager
 from ..errors import (CacheFull, ConfigError, PositionOutOfBounds, StepError,
                       TokenIdOutOfBounds)
 from ..models.decoder import DecoderModel
@@ -512,22 +512,13 @@ class Engine:
         for i, (_, h) in enumerate(hinted):
             for name, arr in h.arrays.items():
                 put(f"hint{i}.{name}", arr.reshape(-1))
+        rids = [e.request_id for e in entries]
         for g in range(n_groups):
-            bt = np.full((n_seqs, max_pages), NO_PAGE, dtype=np.int32)
-            sm = np.empty((T,), dtype=np.int32)
-            for i, e in enumerate(entries):
-                table = self.cache.table(g, e.request_id)
-                bt[i, :len(table)] = table
-                if q_lens[i] == 1:
-                    p = starts[i]
-                    sm[q_start[i]] = table[p // ps] * ps + p % ps
-                else:
-                    pos = np.arange(starts[i], ctx_lens[i])
-                    sm[q_start[i]:q_start[i + 1]] = bt[i, pos // ps] * ps + pos % ps
-            if (sm < 0).any():
-                raise StepError("a token would be written to a page that is not held")
-            put(f"slot_mapping{g}", sm)
-            put(f"block_table{g}", bt.reshape(-1))
+            # the block tables and the slot mapping, written by the cache's native core
+            # straight into their places of the buffer
+            (bo, bn), (so, sn) = offs[f"block_table{g}"], offs[f"slot_mapping{g}"]
+            self.cache.pack_step(g, rids, starts, q_lens, max_pages, host[bo:bo + bn],
+                                 host[so:so + sn])
 
         dev = self._upload(host)
 

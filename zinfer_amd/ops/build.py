@@ -1,10 +1,12 @@
-"""Builds and loads the HIP kernel libraries.
+"""Builds and loads the native libraries.
 
 Each ``csrc/<module>.hip`` becomes one shared library ``_lib/<module>.so`` compiled with
-hipcc for gfx950.  A library is built when it is first needed and its sources have changed
-(or it is missing); the build prints a line now and then so that a first call that compiles
-does not look hung.  When the package folder cannot be written the libraries go to a
-per-user folder under the system's temporary directory.
+hipcc for gfx950; each ``csrc/host/<module>.cpp`` (host code that never touches a device: the
+cache manager's bookkeeping) one compiled with the host's C++ compiler.  A library is built
+when it is first needed and its sources have changed (or it is missing); the build prints a
+line now and then so that a first call that compiles does not look hung.  When the package
+folder cannot be written the libraries go to a per-user folder under the system's temporary
+directory.
 """
 from __future__ import annotations
 
@@ -23,7 +25,9 @@ from ..errors import KernelUnavailable
 
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 MODULES = ("elementwise", "gemm", "attention", "sampling", "randinit")
+HOST_MODULES = ("cache_core",)
 HEADERS = ("zf_common.h", "zf_no_alloc.h")
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
 # -packed-fp32-ops off: hipcc must not form packed 32-bit float instructions by itself
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -42,8 +46,21 @@ def _hipcc() -> str:
                             "the HIP kernels cannot be built")
 
 
+def _host_compiler() -> str:
+    for cand in (os.environ.get("CXX"), "g++", "c++", "clang++"):
+        path = shutil.which(cand) if cand else None
+        if path:
+            return path
+    return _hipcc()          # it compiles plain C++ as well
+
+
 def _source_hash(module: str) -> str:
     h = hashlib.sha256()
+    if module in HOST_MODULES:
+        with open(os.path.join(CSRC, "host", module + ".cpp"), "rb") as f:
+            h.update(f.read())
+        h.update(" ".join(HOST_FLAGS).encode())
+        return h.hexdigest()
     for name in (module + ".hip",) + HEADERS:
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(f.read())
@@ -95,19 +112,25 @@ def is_current(module: str) -> bool:
 
 def compile_module(module: str, verbose: bool = True) -> str:
     """Compiles one module (always) and returns the library's path."""
-    if module not in MODULES:
-        raise KernelUnavailable(f"unknown kernel module {module!r}")
+    if module not in MODULES and module not in HOST_MODULES:
+        raise KernelUnavailable(f"unknown native module {module!r}")
     so, hp = _paths(module)
-    src = os.path.join(CSRC, module + ".hip")
     tmp = f"{so}.{os.getpid()}.tmp"
-    cmd = [_hipcc()] + FLAGS + ["-I", CSRC, src, "-o", tmp]
+    if module in HOST_MODULES:
+        src = os.path.join(CSRC, "host", module + ".cpp")
+        cmd = [_host_compiler()] + HOST_FLAGS + [src, "-o", tmp]
+    else:
+        src = os.path.join(CSRC, module + ".hip")
+        cmd = [_hipcc()] + FLAGS + ["-I", CSRC, src, "-o", tmp]
+    what = os.path.basename(src)
     env = dict(os.environ)
     env.setdefault("HOME", tempfile.gettempdir())
     if not env["HOME"] or not os.access(env["HOME"], os.W_OK):
         env["HOME"] = tempfile.gettempdir()
     t0 = time.time()
     if verbose:
-        print(f"[zinfer_amd] compiling {module}.hip for gfx950 ...", file=sys.stderr, flush=True)
+        print(f"[zinfer_amd] compiling {what}" + ("" if module in HOST_MODULES else " for gfx950")
+              + " ...", file=sys.stderr, flush=True)
     proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, env=env,
                             text=True)
     out_lines: List[str] = []
@@ -119,7 +142,7 @@ def compile_module(module: str, verbose: bool = True) -> str:
             break
         except subprocess.TimeoutExpired:
             if verbose:
-                print(f"[zinfer_amd] still compiling {module}.hip ({time.time() - t0:.0f} s)",
+                print(f"[zinfer_amd] still compiling {what} ({time.time() - t0:.0f} s)",
                       file=sys.stderr, flush=True)
     reader.join()
     if proc.returncode != 0:
@@ -128,7 +151,7 @@ def compile_module(module: str, verbose: bool = True) -> str:
         except OSError:
             pass
         text = "".join(l for l in out_lines if "packed-fp32-ops" not in l)
-        raise KernelUnavailable(f"hipcc failed on {module}.hip:\n{text[-4000:]}")
+        raise KernelUnavailable(f"{os.path.basename(cmd[0])} failed on {what}:\n{text[-4000:]}")
     os.replace(tmp, so)
     with open(hp, "w") as f:
         f.write(_source_hash(module))
@@ -140,7 +163,7 @@ def compile_module(module: str, verbose: bool = True) -> str:
 
 def build_all(verbose: bool = True) -> None:
     """Compiles every module, whether or not a built library is there."""
-    prepare(MODULES, force=True, verbose=verbose)
+    prepare(MODULES + HOST_MODULES, force=True, verbose=verbose)
 
 
 def prepare(modules: Iterable[str], force: bool = False, verbose: bool = True) -> None:
