@@ -268,3 +268,20 @@ def test_the_last_round_of_large_tiles_is_split_only_where_it_is_short():
     assert ops._tile_tail_split(512, 24576, 4096) is None         # 384: under one round
     assert ops._tile_tail_split(2048, 24576, 4096) is None        # three whole rounds
     assert ops._tile_tail_split(2048, 34816, 5120) is None        # a last round behind four
+
+
+def test_residual_sums_of_several_hundred_tokens_over_a_long_k_take_wide_tiles_split():
+    """`_wide_ksplit`: 641 to 1280 tokens over K >= 8192 run through 128 x 256 tiles split two
+    to four times along K, every part an even number of k-tiles; other sizes keep their plan."""
+    from zinfer_amd import ops
+    for M in (641, 768, 1024, 1280):
+        for N, K in ((4096, 12288), (5120, 17408), (5120, 25600), (5120, 8192), (2560, 9728)):
+            ks = ops._wide_ksplit(M, N, K)
+            if K % 128:
+                assert ks is None
+                continue
+            assert ks in (2, 3, 4) and (K // 64) % (2 * ks) == 0, (M, N, K, ks)
+    assert ops._wide_ksplit(1280, 4096, 12288) == 3 and ops._wide_ksplit(768, 5120, 17408) == 4
+    for M, N, K in ((512, 5120, 17408), (640, 4096, 12288), (1281, 4096, 12288), (2048, 4096, 12288),
+                    (1024, 4096, 4096), (1024, 5120, 5120)):
+        assert ops._wide_ksplit(M, N, K) is None, (M, N, K)
