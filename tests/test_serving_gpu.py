@@ -201,3 +201,13 @@ def test_bench_commands_print_the_reference_keys_and_class_times(tmp_path, capsy
         # can outweigh the kernels, so the classes' sum is only bounded from below)
         parts = sum(v for k, v in times.items() if k != "decode_step_step_ms")
         assert parts >= 0.5 * times["decode_step_step_ms"]
+    # the suite: the same report for three prompt lengths on one loaded engine
+    # (`src/app/cli/tools/bench/runtime.zig:101-133`)
+    assert cli.main(["bench-suite", path]) == 0
+    out = capsys.readouterr().out
+    assert out.startswith(f"Zinfer perf-gate suite\nmodel_dir: {path}\n")
+    assert [l.split()[1] for l in out.splitlines() if l.startswith("[suite] ")] == \
+        ["profile=short", "profile=medium", "profile=long"]
+    assert out.count("decode_tokens: 2\n") == 3
+    assert [int(l.split(":")[1]) for l in out.splitlines() if l.startswith("prompt_tokens:")] == \
+        [n for _, n in cli.SUITE_PROFILES]

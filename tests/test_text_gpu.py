@@ -96,3 +96,50 @@ def test_generate_chat_and_serve_batch(model_dir, tmp_path, capsys):
     assert "serve-batch: 3 requests" in capsys.readouterr().err
     rpath.write_text(json.dumps({"id": 1, "prompt": [1], "text": "x"}) + "\n")
     assert cli.main(["serve-batch", model_dir, "--requests", str(rpath)]) == 1
+
+
+def test_chat_turns_history_and_sessions(model_dir, tmp_path, capsys, monkeypatch):
+    """`zinfer chat` over lines of standard input (`src/app/cli/chat.zig:226-312`): every turn
+    is the whole history rendered anew, an earlier answer enters it as the family keeps it,
+    /clear empties it, /save, /load and --save write and read sessions."""
+    import io
+    import sys
+    from zinfer_amd.text import Message, render_messages, strip_historical_thinking
+    from zinfer_amd.text.chat import load_messages
+    tok = Tokenizer.from_dir(model_dir)
+
+    def answer(history):
+        text = tok.decode(_greedy(model_dir, tok.encode(render_messages(history, False)), 6))
+        return text[:analyze_generated_text(text, ["<|im_end|>"])[2]]
+
+    first = answer([Message("system", "Hi"), Message("user", "Hello")])
+    history = [Message("system", "Hi"), Message("user", "Hello"),
+               Message("assistant", strip_historical_thinking(first)), Message("user", "test")]
+    second = answer(history)
+    alone = answer([Message("system", "Hi"), Message("user", "test")])
+    mid, end = tmp_path / "mid.json", tmp_path / "end.json"
+    lines = ["Hello", "", f"/save {mid}", "test", "/clear", "test", f"/load {mid}", "test", "/quit",
+             "never read"]
+    monkeypatch.setattr(sys, "stdin", io.StringIO("\n".join(lines) + "\n"))
+    rc = cli.main(["chat", model_dir, "6", "no-think", "--temperature", "0",
+                   "--repetition-penalty", "1", "--system", "Hi", "--dtype", "float32",
+                   "--save", str(end)])
+    out = capsys.readouterr().out
+    assert rc == 0
+    assert out.startswith(f"Zinfer chat\nmodel_dir: {model_dir}\nmode: no-think\n"
+                          "commands: /exit /quit /clear /save <path> /load <path>\n")
+    said = [piece.split("\n")[0] for piece in out.split("assistant> ")[1:]]
+    assert said == [first.split("\n")[0], second.split("\n")[0], alone.split("\n")[0],
+                    second.split("\n")[0]]
+    assert f"saved: {mid}" in out and "history cleared" in out and f"loaded: {mid}" in out
+    assert [(m.role, m.content) for m in load_messages(str(mid))] == \
+        [(m.role, m.content) for m in history[:3]]
+    kept = load_messages(str(end))
+    assert [m.role for m in kept] == ["system", "user", "assistant", "user", "assistant"]
+    assert kept[-1].content == strip_historical_thinking(second)
+    # a session is a start as well: the answer to the same question is the same again
+    monkeypatch.setattr(sys, "stdin", io.StringIO("test\n"))
+    rc = cli.main(["chat", model_dir, "6", "--temperature", "0", "--repetition-penalty", "1",
+                   "--dtype", "float32", "--load", str(mid), "--stream"])
+    out = capsys.readouterr().out
+    assert rc == 0 and out.split("assistant> ")[1].split("\n")[0] == second.split("\n")[0]

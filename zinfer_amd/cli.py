@@ -20,9 +20,13 @@ USAGE = """Usage:
   zinfer inspect-config [model_dir]
   zinfer inspect-weights [model_dir]
   zinfer inspect-tensor [model_dir] <tensor_name> [count]
+  zinfer probe-linear [model_dir] <tensor_name> [input_index] [rows_to_print]
+  zinfer probe-block [model_dir] [layer_index] [input_index] [count]
+  zinfer probe-model [model_dir] [token_id] [top_k]
   zinfer generate-token-ids [model_dir] <seed_ids_csv> <steps>
   zinfer generate [model_dir] <text|ids_csv> [max_new_tokens] [think|no-think] [flags...]
   zinfer generate-chat [model_dir] <messages_json_path> [max_new_tokens] [think|no-think] [flags...]
+  zinfer chat [model_dir] [max_new_tokens] [think|no-think] [flags...]
   zinfer tokenize [model_dir] <text>
   zinfer decode-ids [model_dir] <ids_csv>
   zinfer serve-batch [model_dir] --requests <file.jsonl> [--out <file.jsonl>] [flags...]
@@ -30,19 +34,21 @@ USAGE = """Usage:
   zinfer bench [model_dir] <ids_csv> [max_new_tokens]
   zinfer bench-batch [model_dir] <ids_csv> <batch_size> [max_new_tokens]
   zinfer bench-continuous [model_dir] <ids_csv> <batch_size> <total_requests> [max_new_tokens]
+  zinfer bench-suite [model_dir]
   zinfer bench-ops [model_dir] [--shape 0.6b|1.7b|4b|8b|14b|32b] [--tokens 1,8,64,2048] [--iters N]
                    [--tune [--plans-out kernel_plans.json]]
   zinfer random-model <config.json> <out_dir> [--seed <u64>] [--dtype bfloat16|float32]
 
 Defaults:
   model_dir = models/Qwen3-0.6B
-  generate max_new_tokens = 64, generate-chat max_new_tokens = 128, bench max_new_tokens = 16
+  generate max_new_tokens = 64, generate-chat/chat max_new_tokens = 128, bench max_new_tokens = 16
 
 Flags:
   --seed <u64>                 --temperature <f32>        --top-p <f32>
   --top-k <usize>              --min-p <f32>              --presence-penalty <f32>
   --frequency-penalty <f32>    --repetition-penalty <f32> --stream
   --system <text>              --stop <text> (repeatable; text prompts only)
+  --load <path>  --save <path> (chat only: a session to start from, and to write at the end)
   --backend <auto|bf16>        --kv-cache <auto|bf16|fp32>
   --threads <usize>            (accepted, unused: the GPU grid replaces the thread pool)
   --dtype <bfloat16|float32>   --page-size <n>            --max-tokens <n>
@@ -103,6 +109,8 @@ class Options:
         self.seed = 0
         self.debug_tables = False       # check every step's block tables on the device
         self.classes = False            # bench: a decode step's time per class of kernels
+        self.load_path: Optional[str] = None            # chat only (`args.zig:437-446`)
+        self.save_path: Optional[str] = None
         self.config_path: Optional[str] = None          # with --random-weights: no model folder
         self.random_weights: Optional[int] = None
 
@@ -113,8 +121,8 @@ _FLOAT_FLAGS = {"--temperature": "temperature", "--top-p": "top_p", "--min-p": "
                 "--repetition-penalty": "repetition_penalty"}
 
 
-def parse_flags(flags: List[str], opt: Options) -> None:
-    """`src/app/cli/args.zig:395-501`."""
+def parse_flags(flags: List[str], opt: Options, chat: bool = False) -> None:
+    """`src/app/cli/args.zig:395-501`.  ``chat``: the flags that only the chat loop has."""
     i = 0
 
     def value() -> str:
@@ -141,6 +149,8 @@ def parse_flags(flags: List[str], opt: Options) -> None:
             opt.stop.append(value())
         elif a == "--system":
             opt.system = value()
+        elif a in ("--load", "--save") and chat:
+            setattr(opt, a[2:] + "_path", value())
         elif a == "--backend":
             v = value()
             if v in ("q8", "q6", "q4"):
@@ -335,6 +345,102 @@ def cmd_inspect_tensor(args: List[str]) -> int:
     return 0
 
 
+def _probe_args(args: List[str], n_numbers: int, defaults, name_first: bool = False):
+    """``[model_dir] [name] [numbers...]`` of the probe commands (`src/app/cli.zig:47-135`):
+    the model folder is the first positional when it is no number (and, for a command that
+    takes a name, when two words come before the numbers); numbers left out take their
+    defaults.  Returns (model_dir, name or None, numbers, options)."""
+    pos, flags = _split_flags(args)
+    words = 0
+    while words < len(pos) and not pos[words].isdigit():
+        words += 1
+    want = 1 if name_first else 0
+    if words not in (want, want + 1) or len(pos) - words > n_numbers:
+        raise CliError("InvalidCommand")
+    model_dir = pos[0] if words == want + 1 else DEFAULT_MODEL_DIR
+    name = pos[words - 1] if name_first else None
+    numbers = [int(v) for v in pos[words:]]
+    numbers += list(defaults[len(numbers):])
+    opt = Options(0)
+    parse_flags(flags, opt)
+    return model_dir, name, numbers, opt
+
+
+def _numbers(values) -> str:
+    return "[" + ", ".join(f"{float(v):.6f}" for v in values) + "]"
+
+
+def cmd_probe_linear(args: List[str]) -> int:
+    """`src/app/cli/inspect.zig:109-151`: a vector that is 1 at ``input_index`` and 0 elsewhere
+    through the matrix ``tensor_name``, by the engine's own product; the first outputs."""
+    import os
+    import torch
+    from .models.build import parse_dtype
+    from .parts import BuildContext
+    from .parts.linear import Linear, place_matrix
+    from .weights import SafetensorsFile
+    model_dir, name, (index, rows_to_print), opt = _probe_args(args, 2, (0, 8), name_first=True)
+    path = os.path.join(model_dir, "model.safetensors")
+    with SafetensorsFile(path) as f:
+        if name not in f.infos:
+            raise CliError(f"TensorNotFound: {name}")
+        if len(f.infos[name].shape) != 2:
+            raise CliError(f"InvalidTensorRank: {name} has shape {list(f.infos[name].shape)}")
+        rows, cols = f.infos[name].shape
+        if index >= cols:
+            raise CliError(f"InputIndexOutOfBounds: {index}, the matrix has {cols} columns")
+        ctx = BuildContext(parse_dtype(opt.dtype), torch.device(opt.device))
+        linear = Linear(place_matrix(f.tensor(name), ctx))
+    x = torch.zeros((1, cols), dtype=ctx.act_dtype, device=ctx.device)
+    x[0, index] = 1.0
+    out = torch.empty((1, rows), dtype=torch.float32, device=ctx.device)
+    linear.forward(x, out)
+    print("Zinfer linear probe")
+    print(f"tensor: {name}")
+    print(f"weights_path: {path}")
+    print(f"shape: [{rows}, {cols}]")
+    print(f"input_index: {index}")
+    print("first_outputs: " + _numbers(out[0, :rows_to_print].tolist()))
+    return 0
+
+
+def cmd_probe_block(args: List[str]) -> int:
+    """`src/app/cli/inspect.zig:153-204`: a hidden vector that is 1 at ``input_index`` through
+    block ``layer_index`` alone, as a new request's first token; the first outputs."""
+    import torch
+    model_dir, _, (layer, index, count), opt = _probe_args(args, 3, (0, 0, 8))
+    llm = _llm(model_dir, opt, max_tokens=64)
+    spec = llm.model.spec
+    if index >= spec.hidden_size:
+        raise CliError(f"InputIndexOutOfBounds: {index}, hidden_size is {spec.hidden_size}")
+    if layer >= len(llm.model.blocks):
+        raise CliError(f"LayerIndexOutOfBounds: {layer}, the model has {len(llm.model.blocks)}")
+    hidden = torch.zeros((1, spec.hidden_size), dtype=torch.float32, device=opt.device)
+    hidden[0, index] = 1.0
+    out, cache_len = llm.engine.probe_block(layer, hidden)
+    print("Zinfer block probe")
+    print(f"layer_index: {layer}")
+    print(f"input_index: {index}")
+    print(f"cache_len: {cache_len}")
+    print("first_outputs: " + _numbers(out[0, :count].tolist()))
+    return 0
+
+
+def cmd_probe_model(args: List[str]) -> int:
+    """`src/app/cli/inspect.zig:206-244`: one token through the whole model as a new request;
+    the largest logits."""
+    from .engine import StepEntry
+    model_dir, _, (token, top_k), opt = _probe_args(args, 2, (0, 8))
+    llm = _llm(model_dir, opt, max_tokens=64)
+    logits = llm.engine.step([StepEntry("probe", [token], [0])], end=["probe"])[0]
+    top = logits.topk(min(top_k, logits.numel()))
+    print("Zinfer model probe")
+    print(f"token_id: {token}")
+    for value, at in zip(top.values.tolist(), top.indices.tolist()):
+        print(f"top_logit token={at} value={value:.6f}")
+    return 0
+
+
 def cmd_generate_token_ids(args: List[str]) -> int:
     """`src/app/cli/inspect.zig:246-312`: greedy from raw ids, no end-of-sequence check;
     prints prompt and generated ids in one list as the reference does."""
@@ -395,21 +501,14 @@ def cmd_generate(args: List[str]) -> int:
     return 0
 
 
-def _generate_text(model_dir: str, prompt_text: str, opt: Options) -> int:
-    """Encodes the rendered prompt, generates until an end-of-sequence id, the token limit or
-    a stop sequence (the family's defaults and ``--stop``), and prints the answer, piece by
-    piece with ``--stream`` (`src/app/cli/runtime/generator.zig:60-140`,
-    `runtime/streaming.zig:41-65`)."""
-    from .text import analyze_generated_text, effective_stop_sequences
-    tok = _text_hooks(model_dir).load_tokenizer(model_dir)
-    ids = tok.encode(prompt_text)
-    if not ids:
-        raise CliError("EmptyPrompt")
-    llm = _llm(model_dir, opt, max_tokens=(len(ids) + opt.max_new_tokens + 63) // 64 * 64)
-    stops = effective_stop_sequences(llm.model.spec.default_stop_sequences, opt.stop)
+def _respond(llm, tok, ids: List[int], opt: Options, stops: List[str]) -> str:
+    """Generates from ``ids`` until an end-of-sequence id, the token limit or a stop sequence
+    and returns the answer; with ``--stream`` it is printed piece by piece on the way, except
+    for a tail that may still grow into a stop sequence
+    (`src/app/cli/runtime/generator.zig:60-140`, `runtime/streaming.zig:41-65`)."""
+    from .text import analyze_generated_text
     sched = llm.new_scheduler()
     rid = sched.add_request(ids, opt.sampling)
-    sys.stdout.write("response: ")
     printed, response, seen = 0, None, 0
     while sched.has_work() and response is None:
         sched.step()
@@ -431,7 +530,22 @@ def _generate_text(model_dir: str, prompt_text: str, opt: Options) -> int:
         response = tok.decode(sched.request(rid).generated)
     if opt.stream:
         sys.stdout.write(response[printed:])
-    else:
+        sys.stdout.flush()
+    return response
+
+
+def _generate_text(model_dir: str, prompt_text: str, opt: Options) -> int:
+    """Encodes the rendered prompt, generates and prints the answer."""
+    from .text import effective_stop_sequences
+    tok = _text_hooks(model_dir).load_tokenizer(model_dir)
+    ids = tok.encode(prompt_text)
+    if not ids:
+        raise CliError("EmptyPrompt")
+    llm = _llm(model_dir, opt, max_tokens=(len(ids) + opt.max_new_tokens + 63) // 64 * 64)
+    stops = effective_stop_sequences(llm.model.spec.default_stop_sequences, opt.stop)
+    sys.stdout.write("response: ")
+    response = _respond(llm, tok, ids, opt, stops)
+    if not opt.stream:
         sys.stdout.write(response)
     sys.stdout.write("\n")
     return 0
@@ -447,6 +561,98 @@ def cmd_generate_chat(args: List[str]) -> int:
     print(f"mode: {'think' if opt.think else 'no-think'}")
     print(f"messages_path: {path}")
     return _generate_text(model_dir, hooks.render_messages(messages, opt.think), opt)
+
+
+def parse_chat(args: List[str]) -> Tuple[str, Options]:
+    """``[model_dir] [max_new_tokens] [think|no-think] [flags]`` (`args.zig:189-226`): a first
+    positional that is no number is the model folder."""
+    pos, flags = _split_flags(args)
+    model_dir, max_new = DEFAULT_MODEL_DIR, 128
+    if pos and not pos[0].isdigit() and pos[0] not in ("think", "no-think"):
+        model_dir, pos = pos[0], pos[1:]
+    if pos and pos[0].isdigit():
+        max_new, pos = int(pos[0]), pos[1:]
+    think = False
+    if pos:
+        if pos[0] not in ("think", "no-think"):
+            raise CliError(f"InvalidThinkingMode: {pos[0]}")
+        think, pos = pos[0] == "think", pos[1:]
+    if pos:
+        raise CliError(f"InvalidCommand: unexpected {pos[0]!r}")
+    opt = Options(max_new, think)
+    opt.max_seqs = 1                    # one conversation: the pool holds one full context
+    parse_flags(flags, opt, chat=True)
+    opt.sampling.max_new_tokens = opt.max_new_tokens
+    opt.sampling.ignore_eos = opt.ignore_eos
+    return model_dir, opt
+
+
+def _session_options(opt: Options) -> dict:
+    """What a saved session says about how it was made (`chat.zig:120-183`)."""
+    s = opt.sampling
+    return {"thinking_mode": "think" if opt.think else "no-think",
+            "max_new_tokens": opt.max_new_tokens, "seed": opt.seed, "backend": opt.dtype,
+            "kv_cache": opt.kv_cache, "stream_output": opt.stream, "system_prompt": opt.system,
+            "sampling": {"temperature": s.temperature, "top_p": s.top_p, "top_k": s.top_k,
+                         "min_p": s.min_p, "presence_penalty": s.presence_penalty,
+                         "frequency_penalty": s.frequency_penalty,
+                         "repetition_penalty": s.repetition_penalty},
+            "stop_sequences": list(opt.stop)}
+
+
+def cmd_chat(args: List[str], lines=None) -> int:
+    """`src/app/cli/chat.zig:226-312`: a conversation line by line on standard input.  Every
+    turn renders the whole history and runs it as a new request; ``/exit`` ``/quit`` end it,
+    ``/clear`` empties the history, ``/save <path>`` and ``/load <path>`` write and read a
+    session; ``--load`` and ``--save`` do the same at the start and at the end."""
+    from .text import Message, effective_stop_sequences
+    from .text.chat import load_messages, with_system
+    from .text.session import save_session
+    model_dir, opt = parse_chat(args)
+    hooks = _text_hooks(model_dir)
+    tok = hooks.load_tokenizer(model_dir)
+    llm = _llm(model_dir, opt)
+    stops = effective_stop_sequences(llm.model.spec.default_stop_sequences, opt.stop)
+    print("Zinfer chat")
+    print(f"model_dir: {model_dir}")
+    print(f"mode: {'think' if opt.think else 'no-think'}")
+    print("commands: /exit /quit /clear /save <path> /load <path>")
+    history = with_system(load_messages(opt.load_path) if opt.load_path else [], opt.system)
+    for raw in (sys.stdin if lines is None else lines):
+        sys.stdout.write("user> ")
+        sys.stdout.flush()
+        line = raw.rstrip("\r\n")
+        if not line:
+            continue
+        if line in ("/exit", "/quit"):
+            break
+        if line == "/clear":
+            history = with_system([], opt.system)
+            print("history cleared")
+            continue
+        if line.startswith("/save ") or line.startswith("/load "):
+            path = line[6:].strip(" ")
+            if not path:
+                raise CliError(f"MissingFlagValue: {line[:5]}")
+            if line.startswith("/save "):
+                save_session(path, history, model_dir, _session_options(opt))
+                print(f"saved: {path}")
+            else:
+                history = with_system(load_messages(path), opt.system)
+                print(f"loaded: {path}")
+            continue
+        history.append(Message("user", line))
+        ids = tok.encode(hooks.render_messages(history, opt.think))
+        sys.stdout.write("assistant> ")
+        response = _respond(llm, tok, ids, opt, stops)
+        if not opt.stream:
+            sys.stdout.write(response)
+        sys.stdout.write("\n")
+        sys.stdout.flush()
+        history.append(Message("assistant", hooks.assistant_history_content(response)))
+    if opt.save_path:
+        save_session(opt.save_path, history, model_dir, _session_options(opt))
+    return 0
 
 
 def _dir_and_one(args: List[str], what: str) -> Tuple[str, str]:
@@ -592,9 +798,10 @@ def _weights_bytes(llm) -> int:
     return total
 
 
-def cmd_bench(args: List[str], mode: str) -> int:
+def cmd_bench(args: List[str], mode: str, llm=None) -> int:
     """`src/app/cli/tools/bench/runtime.zig:12-99` (bench), `:135-224` (bench-batch),
-    `:226-310` (bench-continuous): timers around prefill and decode, greedy, the same keys."""
+    `:226-310` (bench-continuous): timers around prefill and decode, greedy, the same keys.
+    ``llm``: an engine that is already loaded (its pool must hold the run)."""
     import torch
     from .engine import StepEntry
     from .sampling import SamplingParams
@@ -604,7 +811,8 @@ def cmd_bench(args: List[str], mode: str) -> int:
     total = extra[1] if len(extra) > 1 else batch
     per_req = (len(ids) + opt.max_new_tokens + 63) // 64 * 64
     opt.max_seqs = max(batch, 1)
-    llm = _llm(model_dir, opt, max_tokens=per_req * batch)
+    if llm is None:
+        llm = _llm(model_dir, opt, max_tokens=per_req * batch)
     params = SamplingParams(temperature=0.0, max_new_tokens=opt.max_new_tokens,
                             ignore_eos=opt.ignore_eos)
     print({"bench": "Zinfer benchmark", "bench-batch": "Zinfer batch benchmark",
@@ -687,6 +895,40 @@ def cmd_bench(args: List[str], mode: str) -> int:
     return 0
 
 
+SUITE_PROFILES = (("short", 16), ("medium", 32), ("long", 64))
+SUITE_DECODE_TOKENS = 2
+
+
+def cmd_bench_suite(args: List[str]) -> int:
+    """`src/app/cli/tools/bench/runtime.zig:101-133`: the single-request benchmark over a
+    short, a medium and a long prompt with two decoded tokens each, on one loaded engine.
+    The reference's profiles are texts through its tokenizer and run once per quantised
+    backend; here they are prompt lengths in tokens (ids made up), since a folder may bring
+    no tokenizer, and there is the one backend."""
+    pos, flags = _split_flags(args)
+    if len(pos) > 1:
+        raise CliError("InvalidCommand: bench-suite [model_dir]")
+    model_dir = pos[0] if pos else DEFAULT_MODEL_DIR
+    opt = Options(SUITE_DECODE_TOKENS)
+    parse_flags(flags, opt)
+    opt.max_seqs = 1
+    longest = max(n for _, n in SUITE_PROFILES)
+    llm = _llm(model_dir, opt, max_tokens=(longest + SUITE_DECODE_TOKENS + 63) // 64 * 64)
+    vocab = llm.model.spec.vocab_size
+    print("Zinfer perf-gate suite")
+    print(f"model_dir: {model_dir}")
+    print("threads: 0")
+    print(f"kv_cache: {opt.kv_cache}")
+    print("q8_layout: none")
+    print("kernel_isa: gfx950")
+    for name, n in SUITE_PROFILES:
+        print(f"\n[suite] profile={name} backend={opt.dtype} decode_tokens={SUITE_DECODE_TOKENS}")
+        csv = ",".join(str((7 + 13 * i) % vocab) for i in range(n))
+        cmd_bench([model_dir, csv, str(SUITE_DECODE_TOKENS)] + flags + ["--ignore-eos"], "bench",
+                  llm=llm)
+    return 0
+
+
 def cmd_random_model(args: List[str]) -> int:
     """Random-weights mode: a model folder (config.json, model.safetensors) from a
     configuration file and a seed."""
@@ -723,12 +965,20 @@ def main(argv: Optional[List[str]] = None) -> int:
             return cmd_inspect_weights(args)
         if cmd == "inspect-tensor":
             return cmd_inspect_tensor(args)
+        if cmd == "probe-linear":
+            return cmd_probe_linear(args)
+        if cmd == "probe-block":
+            return cmd_probe_block(args)
+        if cmd == "probe-model":
+            return cmd_probe_model(args)
         if cmd == "generate-token-ids":
             return cmd_generate_token_ids(args)
         if cmd == "generate":
             return cmd_generate(args)
         if cmd == "generate-chat":
             return cmd_generate_chat(args)
+        if cmd == "chat":
+            return cmd_chat(args)
         if cmd == "tokenize":
             return cmd_tokenize(args)
         if cmd == "decode-ids":
@@ -740,15 +990,16 @@ def main(argv: Optional[List[str]] = None) -> int:
             return replay_main(args)
         if cmd in ("bench", "bench-batch", "bench-continuous"):
             return cmd_bench(args, cmd)
+        if cmd == "bench-suite":
+            return cmd_bench_suite(args)
         if cmd == "random-model":
             return cmd_random_model(args)
         if cmd == "bench-ops":
             from .bench_ops import main as bench_ops_main
             return bench_ops_main(args)
-        if cmd in ("quantize", "chat", "probe-linear", "probe-block", "probe-model",
-                   "bench-suite"):
-            print(f"zinfer: {cmd!r} belongs to what this engine does not build (interactive "
-                  "chat, quantisation, CPU probes)", file=sys.stderr)
+        if cmd == "quantize":
+            print("zinfer: 'quantize' belongs to what this engine does not build (quantised "
+                  "weights)", file=sys.stderr)
             return 2
         print(f"zinfer: unknown command {cmd!r}\n", file=sys.stderr)     # `cli.zig:286`
         sys.stderr.write(USAGE)

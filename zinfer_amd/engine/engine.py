@@ -138,6 +138,37 @@ class Engine:
             self.cache.release(rid)
         return logits
 
+    def probe_block(self, layer: int, hidden: torch.Tensor):
+        """Block ``layer`` alone (`src/app/cli/inspect.zig:153-204`): ``hidden`` [T, hidden
+        size] is the residual stream at the first T positions of a request made for this
+        call; the block runs once over it, with pages of its own from the pool.  Returns the
+        stream after the block (float32) and the length the request's cache had then.  What
+        the request held goes back before the call returns."""
+        spec = self.model.spec
+        runs = [pos for pos, e in enumerate(spec.schedule)
+                if e.layer == layer and e.cache_of is None]
+        if not runs:
+            raise StepError(f"no run of the schedule has layer {layer} with a cache of its own")
+        T, width = hidden.shape
+        if width != spec.hidden_size or T < 1:
+            raise StepError(f"hidden is {tuple(hidden.shape)}, the stream is [T, {spec.hidden_size}]")
+        rid = object()
+        entry = StepEntry(rid, [0] * T, [])
+        self._check_entries([entry])
+        if not self.cache.can_reserve([(rid, T)]):
+            raise CacheFull("CacheFull: no pages or request slot for the probe")
+        self._reserve([(rid, T)])
+        try:
+            ctx = self._build_context([entry])
+            x = ctx.scratch("residual", (T, spec.hidden_size), torch.float32)
+            x.copy_(hidden)
+            ctx.norm_ready = ctx.norm_after_block = None
+            self.model.blocks[layer].forward(x, ctx, self.views[runs[0]])
+            self.cache.commit(rid, T)
+            return x.clone(), self.cache.length(rid)
+        finally:
+            self.cache.release(rid)
+
     def _trace(self, record) -> None:
         self.step_trace.append(record)
         if len(self.step_trace) > self.STEP_TRACE_MAX:

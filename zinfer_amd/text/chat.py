@@ -74,9 +74,13 @@ def with_system(messages: Sequence[Message], system: Optional[str]) -> List[Mess
 
 
 def load_messages(path: str) -> List[Message]:
-    """A JSON list of {role, content, tool_calls?: [{name, arguments}]}."""
+    """A JSON list of {role, content, tool_calls?: [{name, arguments}]}, or an object that
+    holds such a list under ``messages`` (a saved chat session) (`src/app/cli/messages.zig:
+    13-68`)."""
     with open(path, "r", encoding="utf-8") as f:
         raw = json.load(f)
+    if isinstance(raw, dict):
+        raw = raw.get("messages")
     if not isinstance(raw, list):
         raise ValueError("InvalidMessages: a JSON list of messages is needed")
     out = []
