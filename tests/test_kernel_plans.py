@@ -37,13 +37,18 @@ def test_tiled_products(N, K):
             # evenly than the tiles alone do
             places = lambda n: 256 if n <= 256 else (n + 511) // 512 * 512
             assert tiles < 384 and places(tiles * ks) / (tiles * ks) < places(tiles) / tiles
-        assert ops._tile_variant(M, N, True, False, K) in (6, 10, 16)
+        assert ops._tile_variant(M, N, True, False, K) in (6, 10, 12, 16)
         if ops._tile_variant(M, N, True, False, K) == 16:
             assert K % 128 == 0
+        if ops._tile_variant(M, N, True, False, K) == 12:      # two groups of waves over K
+            assert K % 256 == 0 and ((M + 127) // 128) * ((N + 255) // 256) <= 256
         assert ops._tile_variant(M, N, False) in (0, 4)
     # 2048 tokens at the served widths: 128 x 256 tiles, except where they would fill the chip
     # one and a half times
     assert ops._tile_variant(2048, 24576, True) == 10 and ops._tile_variant(2048, 4096, True) == 10
+    assert ops._tile_variant(2048, 4096, True, True, 4096) == 12
+    assert ops._tile_variant(2048, 4096, True, True, 4096 + 128) == 10
+    assert ops._tile_variant(2048, 24576, True, False, 4096) == 10
     assert ops._tile_variant(2048, 6144, True) == 6
     # measured choices at a few hundred tokens (Qwen3-8B and 14B widths)
     for (M, n, k), want in {(512, 5120, 5120): 3, (512, 5120, 17408): 3, (512, 7168, 5120): 1,

@@ -220,6 +220,31 @@ def test_gemm_many_large_tiles(kind, K, M, N, variant):
     _check_tiled(ops, kind, M, N, K, variant)
 
 
+@pytest.mark.parametrize("kind", ["store", "accumulate", "swiglu"])
+@pytest.mark.parametrize("M,N,K", [(2048, 4096, 4096), (1300, 2112, 512), (130, 320, 256),
+                                   (257, 576, 768), (1999, 4160, 1024)])
+def test_gemm_large_tiles_with_two_groups_of_waves(kind, M, N, K):
+    """The 128 x 256 tiles with two groups of four waves in a workgroup, each over half of K,
+    which hand each other a column block through LDS at the end: edges in M and N, two to 32
+    k-tiles a group, every epilogue, against the plain product; and that the rule takes it
+    where one round holds the tiles and K is long."""
+    ops = _ops()
+    _check_tiled(ops, kind, M, N, K, 12, seed=91)
+    assert ops._tile_variant(2048, 4096, True, True, 12288) == 12
+    assert ops._tile_variant(2048, 4096, True, True, 2048) == 10
+
+
+def test_gemm_two_groups_of_waves_need_whole_steps():
+    """A K whose k-tiles do not divide over the two groups' pairs of steps is refused."""
+    from zinfer_amd.errors import KernelUnavailable
+    ops = _ops()
+    a = _rand((256, 192), torch.bfloat16, 92).to(DEV)
+    wt = ops.pretile_weight(_rand((256, 192), torch.bfloat16, 93).to(DEV))
+    out = torch.zeros((256, 256), dtype=torch.float32, device=DEV)
+    with pytest.raises(KernelUnavailable):
+        ops.gemm(a, wt, out, w_tiled=True, tile_variant=12)
+
+
 def _check_tiled(ops, kind, M, N, K, variant, seed=35, tile_tail=None):
     """One tiled kernel on pre-tiled W against the plain product."""
     how = dict(tile_variant=variant) if tile_tail is None else dict(tile_tail=tile_tail)

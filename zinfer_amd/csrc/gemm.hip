@@ -417,18 +417,26 @@ __device__ __forceinline__ void store_through_slab(f32x16_t (&acc)[FM][FNALL], f
 // tail_split) of the grid, which leave float32 partials [tail][tail_split][BM][BN] in tail_ws
 // for tile_tail_reduce_kernel; a short last round then takes 1 / tail_split of a tile's time
 // instead of a whole one.
+// KG == 2: two groups of waves in one workgroup, each the whole tile over half of the
+// workgroup's k-tiles (its own stages in LDS, its own W), for products whose tiles are so few
+// that a CU holds one workgroup: twice the waves to hide a load behind, and no more traffic
+// than one group has.  At the end each group hands one of its two column blocks to the other
+// through LDS (half the tile's rows at a time), adds what it is handed (first half of K plus
+// second half, whichever group adds) and stores the block it kept.
 template <int BM, int BN, int WM, int WN, int EPI, int TKM = TK, bool W2 = false,
-          bool ADMA = false, bool TAIL = false>
-__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdirect_kernel(
+          bool ADMA = false, bool TAIL = false, int KG = 1>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64 * KG) void gemm_bf16_tile_wdirect_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M,
     int N, int K, int tiles_m, int tiles_n, int whole, int tail_split,
     float* __restrict__ tail_ws) {
   // (the host pass, which only needs the launch stub, does not know the buffer descriptor type)
 #if defined(__HIP_DEVICE_COMPILE__)
-  constexpr int NWN = BN / WN, NT = (BM / WM) * NWN * 64;
+  constexpr int NWN = BN / WN, NT = (BM / WM) * NWN * 64;       // (NT: the threads of a group)
   constexpr int FM = WM / 32, FN = WN / 32;
   constexpr int LROW = TKM + 8, KCH = TKM / 8;      // LDS row in elements; 16-byte chunks per row
   static_assert(BM * KCH % NT == 0 && TKM % 64 == 0, "tile does not divide over the threads");
+  static_assert(KG == 1 || (KG == 2 && ADMA && !TAIL && FN == 2 && FM % 2 == 0),
+                "two groups: tokens copied straight into LDS, two column blocks a wave");
   constexpr int A_CHUNKS = BM * KCH / NT;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   bf16_t* lds = (bf16_t*)lds_raw;       // two stages of BM rows of LROW elements
@@ -448,7 +456,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
   tile_of_workgroup<(BM >= 128 ? 8 : 1024 / BM)>(tile, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
-  const int tid = threadIdx.x;
+  // (a group's threads count from 0: what follows is one group's view)
+  const int kgrp = KG > 1 ? __builtin_amdgcn_readfirstlane((int)threadIdx.x / NT) : 0;
+  const int tid = KG > 1 ? (int)threadIdx.x % NT : (int)threadIdx.x;
+  if (KG > 1) {
+    kpart = kpart * KG + kgrp;
+    kparts *= KG;
+  }
   const int wave = tid / 64, lane = tid % 64;
   const int wm = wave / NWN, wn = wave % NWN;
 
@@ -495,8 +509,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
 
   if constexpr (ADMA) {
     static_assert(TKM == 64, "direct-to-LDS tokens: k-tiles of 64 (rows of 8 pieces)");
-    __shared__ u32x4_t a_stage0[BM * 8];
-    __shared__ u32x4_t a_stage1[BM * 8];
+    __shared__ u32x4_t a_stages0[KG * BM * 8];
+    __shared__ u32x4_t a_stages1[KG * BM * 8];
+    u32x4_t* const a_stage0 = a_stages0 + kgrp * (BM * 8);
+    u32x4_t* const a_stage1 = a_stages1 + kgrp * (BM * 8);
     // the places this thread fills: place p = tid + c NT is row p / 8, slot p % 8, and takes
     // piece slot ^ ((row >> 1) & 7) of the row's 128 bytes (rows beyond M: the last row)
     uint32_t asrc[A_CHUNKS];
@@ -684,6 +700,47 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_tile_wdi
 
   // (the main loop's last barrier has freed the token stages; the launch sizes the LDS for
   // stages and slabs)
+  if constexpr (KG == 2) {
+    // Half the tile's rows at a time: every wave lays down the column block it gives away
+    // (group 0 its second, group 1 its first) where its partner in the other group finds it.
+    constexpr int HALF = FM / 2, PER_WAVE = HALF * 16 * 64;
+    float* const xch = (float*)lds_raw;
+    float* const mine = xch + (size_t)(kgrp * (NT / 64) + wave) * PER_WAVE;
+    const float* const theirs = xch + (size_t)((1 - kgrp) * (NT / 64) + wave) * PER_WAVE;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      __syncthreads();          // (the round before has been read)
+#pragma unroll
+      for (int ii = 0; ii < HALF; ++ii)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int i = half * HALF + ii;
+          mine[(ii * 16 + r) * 64 + lane] = kgrp == 0 ? acc[i][1][r] : acc[i][0][r];
+        }
+      __syncthreads();
+#pragma unroll
+      for (int ii = 0; ii < HALF; ++ii)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int i = half * HALF + ii;
+          const float v = theirs[(ii * 16 + r) * 64 + lane];
+          // kept block = first half of K + second half of K, in either group
+          const float mine0 = acc[i][0][r], mine1 = acc[i][1][r];
+          acc[i][0][r] = kgrp == 0 ? mine0 + v : mine0;
+          acc[i][1][r] = kgrp == 0 ? mine1 : v + mine1;
+        }
+    }
+    __syncthreads();            // the slabs lie where the blocks were handed over
+    f32x16_t kept[FM][1];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) kept[i][0][r] = kgrp == 0 ? acc[i][0][r] : acc[i][1][r];
+    float* slab32 = (float*)lds_raw + (size_t)(kgrp * (NT / 64) + wave) * 32 * (32 + 4);
+    store_through_slab<FM, 1, 32, EPI>(kept, slab32, m0 + wm * WM, n0 + wn * WN + 32 * kgrp, M, N,
+                                       Cv, lane);
+    return;
+  }
   float* slab = (float*)lds_raw + (size_t)wave * 32 * (WN + 4);
   if constexpr (TAIL) {
     if (in_tail) {      // (uniform over the workgroup) the whole tile as it is, rows beyond M too
@@ -1033,25 +1090,32 @@ static int launch_tile256(const void* A, const void* W, void* C, int M, int N, i
 static int launch_reduce(const void* ws, void* C, int M, int N, int ksplit, int epi,
                          hipStream_t stream);
 
-template <int BM, int BN, int WM, int WN, int TKM = TK, bool W2 = false, bool ADMA = false>
+template <int BM, int BN, int WM, int WN, int TKM = TK, bool W2 = false, bool ADMA = false,
+          int KG = 1>
 static int launch_tile_wdirect(const void* A, const void* W, void* C, int M, int N, int K, int epi,
                                hipStream_t stream, void* ws = nullptr, int ksplit = 1,
                                bool reduce = true) {
   if (N % 16 != 0 || K % TKM != 0) return -3;
-  if (W2 && (K / TKM) % (2 * ksplit) != 0) return -3;     // every part an even number of k-tiles
+  // every part (and every group of waves in it) an even number of k-tiles
+  if (W2 && (K / TKM) % (2 * ksplit * KG) != 0) return -3;
+  if (KG > 1 && (K / TKM) % (ksplit * KG) != 0) return -3;      // the groups meet step by step
   if (ksplit > 1 && (ws == nullptr || epi == EPI_SWIGLU || ksplit > K / TKM)) return -3;
-  constexpr int NT = (BM / WM) * (BN / WN) * 64;
+  constexpr int NT = (BM / WM) * (BN / WN) * 64 * KG;
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const dim3 grid(tiles_m * tiles_n, ksplit), block(NT);
   const int final_epi = epi;
   constexpr size_t stages = (size_t)2 * BM * (TKM + 8) * sizeof(bf16_t);
   constexpr size_t slabs = (size_t)(BM / WM) * (BN / WN) * 32 * (WN + 4) * sizeof(float);
+  // two groups: the column blocks handed over (half of every wave's rows, one block)
+  constexpr size_t handed = (size_t)KG * (BM / WM) * (BN / WN) * (WM / 64) * 16 * 64 * sizeof(float);
   // (with the tokens copied straight into LDS the stages are arrays of the kernel's own)
-  const size_t smem = ADMA ? slabs : stages > slabs ? stages : slabs;
+  const size_t smem = KG > 1 ? handed : ADMA ? slabs : stages > slabs ? stages : slabs;
+  static_assert(KG == 1 || handed >= (size_t)KG * (BM / WM) * (BN / WN) * 32 * 36 * sizeof(float),
+                "the slabs of the two groups' waves fit where the blocks are handed over");
 #define ZF_WD(E)                                                                              \
   do {                                                                                        \
-    auto kern = gemm_bf16_tile_wdirect_kernel<BM, BN, WM, WN, E, TKM, W2, ADMA>;              \
-    if (smem > 64 * 1024) {                                                                   \
+    auto kern = gemm_bf16_tile_wdirect_kernel<BM, BN, WM, WN, E, TKM, W2, ADMA, false, KG>;   \
+    if (smem > 64 * 1024 || KG > 1) {                                                         \
       hipError_t e = hipFuncSetAttribute((const void*)kern,                                   \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
       if (e != hipSuccess) return (int)e;                                                     \
@@ -1143,7 +1207,9 @@ static int launch_tile(const void* A, const void* W, void* C, int M, int N, int 
 //          most CUs that was 2 to 18 % faster (qkv at 1024 and 2048 tokens), with one 10 to
 //          34 % slower (512 tokens, or 256 tiles at 1024: nothing hides the copies' longer
 //          way).  7 and 11 are the tiles of 6 and 10 with the tokens through registers, for
-//          comparison.
+//          comparison.  12 = the tiles of 10 with two groups of four waves in a workgroup,
+//          each over half of K (K % 256 == 0): for 256 tiles or fewer, where a CU has one
+//          workgroup either way.
 extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, int N, int K,
                                  int epi, int variant, int w_tiled, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
@@ -1166,6 +1232,9 @@ extern "C" int zf_gemm_bf16_tile(const void* A, const void* W, void* C, int M, i
     if (variant == 20) return launch_tile256<256>(A, W, C, M, N, K, epi, stream);
     if (variant == 21) return launch_tile256<192>(A, W, C, M, N, K, epi, stream);
     if (variant == 22) return launch_tile256<128>(A, W, C, M, N, K, epi, stream);
+    if (variant == 12)         // the tiles of 10 with two groups of waves, each half of K
+      return launch_tile_wdirect<128, 256, 128, 64, TK, true, true, 2>(A, W, C, M, N, K, epi,
+                                                                       stream);
     if (variant == 11) {       // as 10, the tokens through registers into LDS
       if (K % (2 * TK) == 0)
         return launch_tile_wdirect<128, 256, 128, 64, TK, true>(A, W, C, M, N, K, epi, stream);

@@ -619,7 +619,8 @@ def _decode_acc_plan(M: int, N: int, K: int):
 def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = False,
                   K: int = 0) -> int:
     """Which tiled kernel: with pre-tiled weights the kernels that take W straight from
-    memory (10: 128 x 256 tiles, two workgroups to a CU, when they fill the chip; else 128 x
+    memory (10: 128 x 256 tiles, two workgroups to a CU, when they fill the chip; 12: the same
+    tiles with two groups of waves a workgroup where a CU holds one; else 128 x
     128 tiles, 16: with the waves side by side and k-tiles of 128, for a long K or when one
     round of the chip holds the tiles (weights from HBM, 512 tokens: qkv of the 8B shape 43 ->
     38 us), 6: with 2 x 2 waves); otherwise the kernels that stage both operands through LDS
@@ -633,6 +634,11 @@ def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = Fals
         # tiles along the tokens (512 tokens into 24576 outputs) the large tiles still win
         # (five rows of tiles: 544 tokens into 24576 outputs, 480 large tiles, 143 -> 115 us)
         if tiles >= 160 and not (256 < tiles < 512 and tiles_m > 5):
+            # one workgroup to a CU whatever is done: two groups of waves in it, each over
+            # half of a long K (o_proj and down at 1280 to 2048 tokens: 3 to 12 % less; at
+            # K <= 2048 the blocks handed over at the end cost more than the waves gain)
+            if tiles <= TILE_PLACES // 2 and K >= 4096 and K % 256 == 0:
+                return 12
             return 10
         one_round = tiles_m * ((N + 127) // 128) <= 256
         return 16 if K > 0 and K % 128 == 0 and (K >= 8192 or one_round) else 6
@@ -670,7 +676,7 @@ def _tile_ksplit(M: int, N: int, K: int, accumulate: bool = True) -> int:
 # and the 128-token tiles two to a CU ("pair") or one ("alone").
 _TILE256_RATE = {20: 5.18e12, 21: 4.52e12, 22: 3.73e12}
 _TILE256_WIDTH = {20: 256, 21: 192, 22: 128}
-_TILE128_RATE = {10: (5.13e12, 3.85e12), 16: (3.8e12, 2.9e12), 6: (3.77e12, 2.7e12)}
+_TILE128_RATE = {10: (5.13e12, 3.85e12), 12: (5.13e12, 4.05e12), 16: (3.8e12, 2.9e12), 6: (3.77e12, 2.7e12)}
 
 
 @functools.lru_cache(maxsize=None)
@@ -745,7 +751,7 @@ def _tile_tail_split(M: int, N: int, K: int):
 def _tile128_time(M: int, N: int, K: int, variant: int, ksplit: int) -> float:
     """Estimated seconds of the 128-token tile kernels: rounds of up to 512 tiles, two to a CU
     (a last round of up to 256 tiles runs one to a CU, each faster than two)."""
-    bn = 256 if variant == 10 else 128
+    bn = 256 if variant in (10, 12) else 128
     tiles = ((M + 127) // 128) * ((N + bn - 1) // bn) * ksplit
     per = 2.0 * 128 * bn * (K / ksplit)
     pair, alone = _TILE128_RATE[variant if ksplit == 1 else 6]
