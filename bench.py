@@ -106,6 +106,18 @@ def prefill_flops(cfg, T: int) -> float:
     return linear_flops_per_token(cfg) * T + attn + 2.0 * cfg.vocab_size * cfg.hidden_size
 
 
+def prefill_record(cfg, T: int, seconds: float, peak: float, mfma_rate=None) -> dict:
+    """``frac``: of the published peak; ``frac_of_mfma_loop``: of what a loop of MFMAs alone
+    reaches on random operands on this card (``ops.measure_mfma_rate``)."""
+    flops = prefill_flops(cfg, T)
+    out = {"value": round(T / seconds, 1), "tokens": T, "ms": round(seconds * 1e3, 3),
+           "frac": round(flops / seconds / peak, 4)}
+    if mfma_rate:
+        out["mfma_loop_tflops"] = round(mfma_rate / 1e12, 1)
+        out["frac_of_mfma_loop"] = round(flops / seconds / mfma_rate, 4)
+    return out
+
+
 def run_prefill(llm, cfg, T: int, seed: int) -> float:
     import torch
     from zinfer_amd.engine import StepEntry
@@ -386,9 +398,7 @@ def main_long_context(args) -> int:
             "config": config_of(cfg, shape, global_batch=hb, seq_len=context,
                                 pool_tokens=max(batches) * (context + PAGE),
                                 steps_in_a_row=args.multi_step),
-            "prefill": {"value": round(args.prefill_tokens / pre_s, 1),
-                        "tokens": args.prefill_tokens, "ms": round(pre_s * 1e3, 3),
-                        "frac": round(prefill_flops(cfg, args.prefill_tokens) / pre_s / peak, 4)},
+            "prefill": prefill_record(cfg, args.prefill_tokens, pre_s, peak),
             "roofline": {"bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": res[f"decode_b{hb}_hbm_frac"],
                          "achieved": round(res[f"decode_b{hb}_hbm_frac"] * HBM_PEAK_GBS, 1)},
@@ -468,6 +478,9 @@ def main_decode(args) -> int:
     import zinfer_amd.ops as ops
     measured_gbs = ops.measure_read_bandwidth("cuda:0") / 1e9
     pre_s = run_prefill(llm, cfg, args.prefill_tokens, args.seed + 1)
+    # what the matrix cores sustain on random operands with nothing else to do (the chip's
+    # power limit sets it, far under the 2.4 GHz figure): bfloat16 only
+    mfma_rate = ops.measure_mfma_rate("cuda:0") if args.dtype == "bfloat16" else None
     dt, mean_ctx, where = run_decode(llm, cfg, args.batch, args.prompt_len, args.steps,
                                      args.warmup, args.seed + 2, classes=True)
     value = args.batch * args.steps / dt
@@ -491,9 +504,7 @@ def main_decode(args) -> int:
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
         "config": config_of(cfg, shape, global_batch=args.batch, prompt_len=args.prompt_len,
                             seq_len=int(round(mean_ctx)), steps_in_a_row=args.multi_step),
-        "prefill": {"value": round(args.prefill_tokens / pre_s, 1), "tokens": args.prefill_tokens,
-                    "ms": round(pre_s * 1e3, 3),
-                    "frac": round(prefill_flops(cfg, args.prefill_tokens) / pre_s / peak, 4)},
+        "prefill": prefill_record(cfg, args.prefill_tokens, pre_s, peak, mfma_rate),
         "roofline": decode_roofline(cfg, elem, args.batch, mean_ctx, dt / args.steps,
                                     measured_gbs),
         "classes": where,

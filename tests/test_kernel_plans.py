@@ -130,6 +130,7 @@ TESTED_AGAINST = {
     "apply_penalties": "plain.py:adjusted_logit", "sample_topk": "plain.py:sample_token",
     "randinit": "test_kernels_gpu.py:test_randinit_is_the_numpy_draw_bit_for_bit",
     "stream_read": "test_kernels_gpu.py:test_stream_read_reads_every_byte_once",
+    "mfma_loop": "test_kernels_gpu.py:test_mfma_loop_sums_its_products",
     "check_tables": "test_kernels_gpu.py:test_check_tables_reports_and_never_traps",
 }
 

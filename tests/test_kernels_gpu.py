@@ -1219,6 +1219,26 @@ def test_stream_read_reads_every_byte_once():
     assert ops.measure_read_bandwidth(DEV, nbytes=1 << 28, repeats=2) > 1e12
 
 
+def test_mfma_loop_sums_its_products():
+    """The measurement kernel's accumulators are its rounds times the products of the operands
+    it was given, as the lanes of a wave hold them; its rate on zeros is the clock's, on random
+    operands what the power limit leaves."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(9)
+    operands = torch.randn((6, 64, 8), generator=g).to(torch.bfloat16)
+    # operand f as a matrix [32, 16]: lane l holds row l % 32, k 8 (l / 32) .. + 8
+    mats = operands.double().reshape(6, 2, 32, 8).permute(0, 2, 1, 3).reshape(6, 32, 16)
+    out = torch.full((8, 32, 32), float("nan"), dtype=torch.float32, device=DEV)
+    iters = 37
+    ops.mfma_loop(operands.to(DEV), out, 5, iters)
+    for n in range(8):
+        want = iters * (mats[n % 4] @ mats[4 + n // 4].T)
+        assert rel_err(out[n], want) <= 1e-5, n
+    rate_zeros = ops.measure_mfma_rate(DEV, random_operands=False, seconds=0.02)
+    rate_random = ops.measure_mfma_rate(DEV, seconds=0.02)
+    assert 1.0e15 < rate_random <= rate_zeros * 1.02 < 2.6e15, (rate_random, rate_zeros)
+
+
 def test_check_tables_reports_and_never_traps():
     """The debugging check of a step's tables: a page beyond the pool, a page that is not held
     (-1) inside a context, a context longer than the row, a slot beyond the pool are reported;

@@ -1961,3 +1961,59 @@ extern "C" int zf_gemm_bf16_skinny_emit(const void* A, const void* W, float* C,
   if (rg == 2) return launch_skinny<1, 2, true, NORM_NONE, true>(A, W, C, nullptr, M, N, K, EPI_ACC_F32, 1, stream, nrm);
   return -4;
 }
+
+// ---------------------------------------------------------------- measurement: MFMAs alone
+// What the matrix cores sustain on given operands with nothing else to do: every wave keeps
+// four token operands (32 rows x 16 k each) and two weight operands (32 outputs x 16 k) in
+// registers and runs `iters` rounds of the eight 32x32x16 products between them into eight
+// accumulators, so that operands change from one instruction to the next as they do in the
+// products above.  On operands that toggle the multipliers the chip's power limit, not its
+// clock, sets the rate; the rate this reaches is what the tiled products are measured
+// against.  src: bfloat16 [6][64][8], operand f of lane l at src[f][l] (a lane holds row or
+// output l % 32, k 8 (l / 32) .. + 8); operands 0-3 tokens, 4-5 weights.  The first wave of
+// the first workgroup leaves its accumulators in out [8][32][32] (accumulator n = tokens
+// n % 4 against weights n / 4: iters times their product).
+__global__ __launch_bounds__(256) void mfma_loop_kernel(const u32x4_t* __restrict__ src,
+                                                        float* __restrict__ out, int iters) {
+  const int lane = threadIdx.x % 64;
+  u32x4_t a[4], b[2];
+#pragma unroll
+  for (int f = 0; f < 4; ++f) a[f] = src[f * 64 + lane];
+#pragma unroll
+  for (int f = 0; f < 2; ++f) b[f] = src[(4 + f) * 64 + lane];
+  f32x16_t acc[8];
+#pragma unroll
+  for (int n = 0; n < 8; ++n)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[n][r] = 0.f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int n = 0; n < 8; ++n)
+      acc[n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&a[n % 4],
+                                                       *(const bf16x8_t*)&b[n / 4], acc[n], 0, 0, 0);
+  }
+  if (blockIdx.x == 0 && threadIdx.x < 64) {
+#pragma unroll
+    for (int n = 0; n < 8; ++n)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        out[(n * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4) * 32 + lane % 32] = acc[n][r];
+  } else {
+    // (every other wave's sums must count for something, or the compiler drops its loop)
+    float s = 0.f;
+#pragma unroll
+    for (int n = 0; n < 8; ++n)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s += acc[n][r];
+    if (s == 1234.5678f && iters < 0) out[0] = s;
+  }
+}
+
+// workgroups of four waves; 2 * 32 * 32 * 16 * 8 flops a wave and round
+extern "C" int zf_mfma_loop(const void* src, float* out, int workgroups, int iters,
+                            hipStream_t stream) {
+  if (workgroups < 1 || workgroups > 65536 || iters < 1 || iters > (1 << 22)) return 1;
+  hipLaunchKernelGGL(mfma_loop_kernel, dim3(workgroups), dim3(256), 0, stream,
+                     (const u32x4_t*)src, out, iters);
+  ZF_CHECK_LAUNCH();
+}

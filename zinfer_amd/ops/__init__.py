@@ -405,6 +405,50 @@ def measure_read_bandwidth(device, nbytes: int = 2 << 30, repeats: int = 3) -> f
     return best
 
 
+@_launches("other")
+def mfma_loop(operands: torch.Tensor, out: torch.Tensor, workgroups: int, iters: int) -> None:
+    """``iters`` rounds of eight 32x32x16 MFMAs between the operands in ``operands`` (bfloat16
+    [6, 64, 8]: four token operands, two weight operands, as the lanes of a wave hold them) in
+    every wave of ``workgroups`` workgroups of four; ``out`` float32 [8, 32, 32] takes the first
+    wave's accumulators (accumulator n: ``iters`` times tokens n % 4 against weights n / 4).
+    Nothing but MFMAs: the rate the matrix cores sustain (``measure_mfma_rate``)."""
+    _need_gpu(operands, out)
+    if operands.dtype != torch.bfloat16 or tuple(operands.shape) != (6, 64, 8) \
+            or not operands.is_contiguous() or out.dtype != torch.float32 \
+            or tuple(out.shape) != (8, 32, 32) or not out.is_contiguous():
+        raise KernelUnavailable("mfma_loop: operands bfloat16 [6, 64, 8], out float32 [8, 32, 32]")
+    lib = build.load("gemm")
+    _check(lib.zf_mfma_loop(_ptr(operands), _ptr(out), int(workgroups), int(iters), _stream()),
+           "mfma_loop")
+
+
+MFMA_LOOP_FLOPS = 2.0 * 32 * 32 * 16 * 8 * 4       # a workgroup's flops in one round
+
+
+def measure_mfma_rate(device, random_operands: bool = True, seconds: float = 0.03) -> float:
+    """Flops a second of ``mfma_loop`` on the whole chip, sustained over about ``seconds``
+    (launches of a few milliseconds, the first ones untimed: the clock settles under the
+    load).  On random operands the chip's power limit sets it, on zeros its clock."""
+    g = torch.Generator(device="cpu").manual_seed(5)
+    operands = (torch.randn((6, 64, 8), generator=g) if random_operands
+                else torch.zeros((6, 64, 8))).to(torch.bfloat16).to(device)
+    out = torch.zeros((8, 32, 32), dtype=torch.float32, device=device)
+    workgroups, iters = 1024, 8000                  # about 5 ms a launch
+    for _ in range(3):
+        mfma_loop(operands, out, workgroups, iters)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    n = 0
+    a.record()
+    while True:
+        mfma_loop(operands, out, workgroups, iters)
+        n += 1
+        b.record()
+        b.synchronize()
+        dt = a.elapsed_time(b) * 1e-3
+        if dt >= seconds or n >= 64:
+            return MFMA_LOOP_FLOPS * workgroups * iters * n / dt
+
+
 # ------------------------------------------------------------------------- work buffers
 _workspaces = {}
 _workspace_generation = 0

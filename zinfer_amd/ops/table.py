@@ -11,7 +11,8 @@ from typing import Callable, Dict
 
 from . import (advance_decode, apply_penalties, argmax, argmax_no_alloc, cast, check_tables,
                decode_attention_fused, embed, gather_rows, gemm, gemm_emit, gemm_given,
-               gemm_partials, gemm_sum_norm, gemm_swiglu, norm_gemm, paged_attention, poison_pages,
+               gemm_partials, gemm_sum_norm, gemm_swiglu, mfma_loop, norm_gemm, paged_attention,
+               poison_pages,
                qk_norm_rope_kv_write, randinit, rmsnorm, sample_topk, scale_cap, stream_read,
                swiglu)
 
@@ -62,4 +63,6 @@ KERNELS: Dict[str, KernelEntry] = {
                                 "own: a step's block tables and slots against the pool"),
     "stream_read": KernelEntry(stream_read, "elementwise",
                                "own: the read stream bandwidths are measured against"),
+    "mfma_loop": KernelEntry(mfma_loop, "gemm",
+                             "own: MFMAs alone, the rate the tiled products are measured against"),
 }
