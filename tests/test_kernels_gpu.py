@@ -724,6 +724,34 @@ def test_qk_norm_rope_kv_write(dtype, nH, nKV, hd, page_size, use_norm, use_rope
     assert rel_err(got_inplace, want_inplace) <= tol(dtype)
 
 
+@pytest.mark.parametrize("T", [5, 300])
+def test_positions_beyond_the_rotation_tables_read_their_last_row(T):
+    """A position that the tables do not hold (the engine refuses such a step before it runs;
+    a caller of the kernel alone may not) is taken as the tables' last row, or first: the
+    result is that of the clipped positions, and nothing is read out of bounds."""
+    from zinfer_amd.parts.position import rotary_tables
+    ops = _ops()
+    nH, nKV, hd, page_size, rows = 4, 2, 64, 16, 40
+    width = (nH + 2 * nKV) * hd
+    qkv = _rand((T, width), torch.bfloat16, 21).to(DEV)
+    gain = (1 + 0.1 * _rand((hd,), torch.float32, 22)).to(DEV)
+    cos, sin = (t.to(DEV) for t in rotary_tables(hd, 10000.0, rows))
+    positions = (torch.arange(T, dtype=torch.int32) * 17 - 20)         # -20 .. beyond 40
+    assert positions.min() < 0 and positions.max() >= rows
+    slots = torch.arange(T, dtype=torch.int32).to(DEV)
+    n_pages = (T + page_size - 1) // page_size
+    got, want = [], []
+    for pos, into in ((positions, got), (positions.clamp(0, rows - 1), want)):
+        q = torch.empty((T, nH * hd), dtype=torch.bfloat16, device=DEV)
+        kp = torch.zeros((n_pages, nKV * page_size * hd), dtype=torch.bfloat16, device=DEV)
+        vp = torch.zeros_like(kp)
+        ops.qk_norm_rope_kv_write(qkv, gain, gain, 1e-6, cos, sin, pos.to(DEV), slots, kp, vp, q,
+                                  nH, nKV, hd, page_size)
+        into += [q, kp, vp]
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nH,nKV,hd,page_size", [(32, 8, 128, 16), (6, 2, 64, 32), (3, 1, 48, 16),
                                                  (8, 2, 32, 8), (4, 4, 256, 16)])

@@ -410,6 +410,7 @@ struct DecodeFused {
   const float* sin_t;
   const int* positions;     // [n_seqs]
   const int* slot_mapping;  // [n_seqs]: page * page_size + row of the token's own key and value
+  int table_rows;           // positions the tables hold
 };
 
 // A decode step's attention from the q/k/v product's rows [n_seqs, (nH + 2 nKV) * hd], which
@@ -446,7 +447,8 @@ __global__ __launch_bounds__(256, HD <= 128 ? 3 : 1) void attn_decode_fused_kern
   const int kvh = blockIdx.x, sp = blockIdx.y, s = blockIdx.z;
   const int ctx = ctx_len[s], pos = ctx - 1;
   const int slot = fu.slot_mapping[s];
-  const int rope_pos = fu.cos_t ? fu.positions[s] : 0;
+  // (a position beyond the tables reads their last row: wrong, but no access out of bounds)
+  const int rope_pos = fu.cos_t ? min(max(fu.positions[s], 0), fu.table_rows - 1) : 0;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   if (max(lo, sp * DEC_SPLIT) >= min(ctx, (sp + 1) * DEC_SPLIT)) return;   // whole workgroup
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
@@ -724,7 +726,8 @@ extern "C" int zf_attn_decode_bf16(const void* q, const void* k_pool, const void
 // of zf_qk_norm_rope_kv_write.
 extern "C" int zf_attn_decode_fused_bf16(const void* qkv, const float* q_gain,
                                          const float* k_gain, float eps, const float* cos_t,
-                                         const float* sin_t, const int* positions,
+                                         const float* sin_t, int table_rows,
+                                         const int* positions,
                                          const int* slot_mapping, void* k_pool, void* v_pool,
                                          const int* block_table, const int* q_start,
                                          const int* ctx_len, void* out, float* ws_o,
@@ -734,9 +737,9 @@ extern "C" int zf_attn_decode_fused_bf16(const void* qkv, const float* q_gain,
   if (n_seqs <= 0) return 0;
   if (page_size % 16 != 0 || nKV <= 0 || nH % nKV != 0 || nH / nKV > 16) return -2;
   if ((q_gain == nullptr) != (k_gain == nullptr) || (cos_t == nullptr) != (sin_t == nullptr) ||
-      slot_mapping == nullptr || (cos_t != nullptr && positions == nullptr))
+      slot_mapping == nullptr || (cos_t != nullptr && (positions == nullptr || table_rows < 1)))
     return -2;
-  const DecodeFused fu{q_gain, k_gain, eps, cos_t, sin_t, positions, slot_mapping};
+  const DecodeFused fu{q_gain, k_gain, eps, cos_t, sin_t, positions, slot_mapping, table_rows};
   const float scale_log2e = scale * 1.4426950408889634f;
   dim3 grid(nKV, max_splits, n_seqs);
 #define ZF_DEC(HD)                                                                              \

@@ -142,7 +142,7 @@ __global__ void qk_norm_rope_kv_write_kernel(
     float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int* __restrict__ positions, const int* __restrict__ slot_mapping,
     T* __restrict__ k_pool, T* __restrict__ v_pool, T* __restrict__ q_out, int nH, int nKV,
-    int hd, int page_size, int tiled) {
+    int hd, int page_size, int tiled, int table_rows) {
   const int t = blockIdx.x;
   const int head = blockIdx.y;
   const int lane = threadIdx.x;
@@ -195,7 +195,8 @@ __global__ void qk_norm_rope_kv_write_kernel(
     ss = wave_sum(ss);
     inv = 1.0f / sqrtf(ss / (float)hd + eps);
   }
-  const int pos = positions[t];
+  // (a position beyond the tables reads their last row: wrong, but no access out of bounds)
+  const int pos = min(max(positions[t], 0), table_rows - 1);
   for (int i = lane; i < half; i += ZF_WAVE) {
     float x0 = load_as_float<T>(src + i);
     float x1 = load_as_float<T>(src + i + half);
@@ -259,7 +260,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_vec_kernel(
     const int* __restrict__ positions, const int* __restrict__ slot_mapping,
     T* __restrict__ k_pool, T* __restrict__ v_pool, T* __restrict__ q_out, int nH, int nKV,
     int hd, int page_size, int tiled, const float* __restrict__ partials, int ksplit,
-    size_t split_stride, int Tn) {
+    size_t split_stride, int Tn, int table_rows) {
   // TPB: a workgroup takes this many tokens in a row, the same lanes the same head of each:
   // what all of them need from memory is asked for before any arithmetic, and a quarter of
   // the workgroups are handed out (2048 tokens of 48 heads, one token a workgroup: 33 us for
@@ -284,7 +285,8 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_vec_kernel(
     const int t = min(t0 + tt, Tn - 1);
     live[tt] = active && t0 + tt < Tn;
     slot[tt] = slot_mapping ? slot_mapping[t] : 0;
-    pos[tt] = (cos_t && !is_v) ? positions[t] : 0;
+    // (a position beyond the tables reads their last row: wrong, but no access out of bounds)
+    pos[tt] = (cos_t && !is_v) ? min(max(positions[t], 0), table_rows - 1) : 0;
 #pragma unroll
     for (int e = 0; e < 4; ++e) x0[tt][e] = x1[tt][e] = 0.f;
     T* src = qkv + (size_t)t * row_width + (size_t)hh * hd;
@@ -395,8 +397,8 @@ template <typename T, bool PART = false>
 static void launch_qk_vec(T* qkv, const float* q_gain, const float* k_gain, float eps,
                           const float* cos_t, const float* sin_t, const int* positions,
                           const int* slot_mapping, T* k_pool, T* v_pool, T* q_out, int Tn, int nH,
-                          int nKV, int hd, int page_size, int tiled, hipStream_t stream,
-                          const float* partials = nullptr, int ksplit = 0) {
+                          int nKV, int hd, int page_size, int tiled, int table_rows,
+                          hipStream_t stream, const float* partials = nullptr, int ksplit = 0) {
   const int lanes = hd / 8, heads = nH + 2 * nKV;
   const size_t split_stride = (size_t)Tn * heads * hd;
   // from a few hundred tokens on a workgroup takes four tokens in a row
@@ -406,7 +408,7 @@ static void launch_qk_vec(T* qkv, const float* q_gain, const float* k_gain, floa
                      dim3((Tn + TPB - 1) / TPB, (heads + 256 / LPH - 1) / (256 / LPH)),        \
                      dim3(256), 0, stream, qkv, q_gain, k_gain, eps, cos_t, sin_t, positions,  \
                      slot_mapping, k_pool, v_pool, q_out, nH, nKV, hd, page_size, tiled,       \
-                     partials, ksplit, split_stride, Tn)
+                     partials, ksplit, split_stride, Tn, table_rows)
 #define ZF_QKV(LPH)                                                                            \
   do {                                                                                         \
     if constexpr (PART) ZF_QKV_T(LPH, 1);                                                      \
@@ -428,10 +430,11 @@ extern "C" int zf_qk_norm_rope_kv_write(void* qkv, int dtype, const float* q_gai
                                         const float* sin_t, const int* positions,
                                         const int* slot_mapping, void* k_pool, void* v_pool,
                                         void* q_out, int T, int nH, int nKV, int hd,
-                                        int page_size, int tiled, const float* partials,
-                                        int ksplit, hipStream_t stream) {
+                                        int page_size, int tiled, int table_rows,
+                                        const float* partials, int ksplit, hipStream_t stream) {
   if (T <= 0) return 0;
   if (tiled && (page_size % 16 != 0 || hd % 32 != 0)) return -2;
+  if (cos_t != nullptr && table_rows < 1) return -2;        // table_rows: the tables' positions
   if (partials != nullptr) {
     // rows from a split product's partials: bfloat16, q to q_out, k and v into the pools
     if (dtype != ZF_BF16 || hd % 8 != 0 || hd > 512 || ksplit < 1 || q_out == nullptr ||
@@ -439,18 +442,19 @@ extern "C" int zf_qk_norm_rope_kv_write(void* qkv, int dtype, const float* q_gai
       return -2;
     launch_qk_vec<bf16_t, true>(nullptr, q_gain, k_gain, eps, cos_t, sin_t, positions,
                                 slot_mapping, (bf16_t*)k_pool, (bf16_t*)v_pool, (bf16_t*)q_out,
-                                T, nH, nKV, hd, page_size, tiled, stream, partials, ksplit);
+                                T, nH, nKV, hd, page_size, tiled, table_rows, stream, partials,
+                                ksplit);
     ZF_CHECK_LAUNCH();
   }
   if (hd % 8 == 0 && hd <= 512) {
     if (dtype == ZF_F32)
       launch_qk_vec<float>((float*)qkv, q_gain, k_gain, eps, cos_t, sin_t, positions, slot_mapping,
                            (float*)k_pool, (float*)v_pool, (float*)q_out, T, nH, nKV, hd,
-                           page_size, tiled, stream);
+                           page_size, tiled, table_rows, stream);
     else
       launch_qk_vec<bf16_t>((bf16_t*)qkv, q_gain, k_gain, eps, cos_t, sin_t, positions,
                             slot_mapping, (bf16_t*)k_pool, (bf16_t*)v_pool, (bf16_t*)q_out, T, nH,
-                            nKV, hd, page_size, tiled, stream);
+                            nKV, hd, page_size, tiled, table_rows, stream);
     ZF_CHECK_LAUNCH();
   }
   dim3 grid(T, nH + 2 * nKV);
@@ -458,12 +462,12 @@ extern "C" int zf_qk_norm_rope_kv_write(void* qkv, int dtype, const float* q_gai
     hipLaunchKernelGGL(qk_norm_rope_kv_write_kernel<float>, grid, dim3(ZF_WAVE), 0, stream,
                        (float*)qkv, q_gain, k_gain, eps, cos_t, sin_t, positions, slot_mapping,
                        (float*)k_pool, (float*)v_pool, (float*)q_out, nH, nKV, hd, page_size,
-                       tiled);
+                       tiled, table_rows);
   else
     hipLaunchKernelGGL(qk_norm_rope_kv_write_kernel<bf16_t>, grid, dim3(ZF_WAVE), 0, stream,
                        (bf16_t*)qkv, q_gain, k_gain, eps, cos_t, sin_t, positions, slot_mapping,
                        (bf16_t*)k_pool, (bf16_t*)v_pool, (bf16_t*)q_out, nH, nKV, hd, page_size,
-                       tiled);
+                       tiled, table_rows);
   ZF_CHECK_LAUNCH();
 }
 

@@ -222,6 +222,7 @@ def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, cos, sin, positions, slot_ma
         _ptr(sin), _ptr(positions), _ptr(slot_mapping), _ptr(k_pool), _ptr(v_pool), _ptr(q_out),
         T, n_heads, n_kv_heads, head_dim, page_size,
         1 if mfma_attention_covers(row_dtype, n_heads, n_kv_heads, head_dim, page_size) else 0,
+        0 if cos is None else cos.shape[0],
         _ptr(partials), 0 if partials is None else partials.shape[0],
         _stream()), "qk_norm_rope_kv_write")
 
@@ -1273,6 +1274,7 @@ def decode_attention_fused(qkv, q_gain, k_gain, eps, cos, sin, positions, slot_m
     lib = build.load("attention")
     _check(lib.zf_attn_decode_fused_bf16(
         _ptr(qkv), _ptr(q_gain), _ptr(k_gain), ctypes.c_float(eps), _ptr(cos), _ptr(sin),
+        0 if cos is None else cos.shape[0],
         _ptr(positions), _ptr(slot_mapping), _ptr(k_pool), _ptr(v_pool), _ptr(block_table),
         _ptr(q_start), _ptr(ctx_len), _ptr(out), _ptr(ws_o), _ptr(ws_ml), ctypes.c_float(scale),
         int(window), n_seqs, n_heads, n_kv_heads, head_dim, page_size, block_table.shape[1],
