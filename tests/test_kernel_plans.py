@@ -59,6 +59,11 @@ def test_tiled_products(N, K):
     # a stored product whose tiles need a second round anyway stays whole; a residual sum splits
     assert ops._tile_ksplit(768, 6144, 4096, False) == 1 and ops._tile_ksplit(768, 6144, 4096) > 1
     assert ops._tile_ksplit(384, 6144, 4096, False) == 3
+    # one round of large tiles with two groups of waves needs no partials: over a short K it is
+    # taken instead of a split, over a long K the split stays
+    assert ops._tile_ksplit(1280, 4096, 4096) == 1 and ops._tile_variant(1280, 4096, True, True, 4096) == 12
+    assert ops._tile_ksplit(2048, 2560, 4096) == 1
+    assert ops._tile_ksplit(1024, 5120, 17408) == 3
     assert ops._tile_variant(512, 24576, True, False, 4096) == 10
 
 

@@ -706,6 +706,12 @@ def _tile_ksplit(M: int, N: int, K: int, accumulate: bool = True) -> int:
     tiles = ((M + 127) // 128) * ((N + 127) // 128)
     if tiles >= 384 or (tiles > 256 and not accumulate):
         return 1
+    # one round of 128 x 256 tiles with two groups of waves a workgroup needs no partials: on
+    # a short K it beats the split even with the norm's kernel behind it (1280 tokens into
+    # 4096 outputs, K = 4096: 64 + 6 against 76 us; 2048 into 2560: 59 + 8 against 75); on a
+    # long K the split stays ahead (1024 into 5120, K = 17408: 205 against 237)
+    if K < 8192 and _tile_variant(M, N, True, accumulate, K) == 12:
+        return 1
     best, best_cost = 1, None
     for ks in range(1, min(8, K // 64 // 8) + 1):
         wgs = tiles * ks
