@@ -43,13 +43,18 @@ def test_tiled_products(N, K):
         if ops._tile_variant(M, N, True, False, K) == 12:      # two groups of waves over K
             assert K % 256 == 0 and ((M + 127) // 128) * ((N + 255) // 256) <= 256
         assert ops._tile_variant(M, N, False) in (0, 4)
-    # 2048 tokens at the served widths: 128 x 256 tiles, except where they would fill the chip
-    # one and a half times
+    # 2048 tokens at the served widths: 128 x 256 tiles
     assert ops._tile_variant(2048, 24576, True) == 10 and ops._tile_variant(2048, 4096, True) == 10
     assert ops._tile_variant(2048, 4096, True, True, 4096) == 12
     assert ops._tile_variant(2048, 4096, True, True, 4096 + 128) == 10
     assert ops._tile_variant(2048, 24576, True, False, 4096) == 10
+    # between one and two large tiles a CU, many rows of them: 128 x 128 tiles, the waves side
+    # by side where k-tiles of 128 divide K
     assert ops._tile_variant(2048, 6144, True) == 6
+    assert ops._tile_variant(2048, 6144, True, False, 4096) == 16
+    assert ops._tile_variant(2048, 5120, True, True, 5120 + 64) == 6
+    assert ops._tile_variant(512, 20480, True, False, 5120) == 10        # 320 tiles in 4 rows
+    assert ops._tile_variant(192, 19456, True, False, 2560) == 10        # 152 tiles
     # measured choices at a few hundred tokens (Qwen3-8B and 14B widths)
     for (M, n, k), want in {(512, 5120, 5120): 3, (512, 5120, 17408): 3, (512, 7168, 5120): 1,
                             (512, 4096, 4096): 2, (512, 4096, 12288): 2, (512, 6144, 4096): 1,
@@ -89,13 +94,16 @@ def test_64_token_tiles_for_a_few_hundred_tokens_on_a_narrow_output():
 
 def test_256_token_tiles_are_chosen_where_they_fill_the_chip_evenly():
     """Measured on MI355X (Qwen3-8B widths): 2048 tokens into 6144 outputs are 256 tiles of
-    256 x 192 (101 -> 83 us), 3072 into 4096 are 192 of 256 x 256 (110 -> 106; with 12288
-    inputs 322 -> 284); 2048 into 4096 stay with 128 x 256 tiles (256 of them), gate/up with
-    its many tiles too (the two kinds run it equally fast), and a residual sum that is split
-    along K keeps its split."""
+    256 x 192 (101 -> 83 us); 3072 into 4096 (384 tiles of 128 x 256, 192 of 256 x 256: 108
+    against 113 us, with 12288 inputs 283 against 277) and 2048 into 4096 stay with 128 x 256
+    tiles, gate/up with its many tiles too (the two kinds run it equally fast), and a residual
+    sum that is split along K keeps its split."""
     assert ops._tile256_variant(2048, 6144, 4096) == 21
     assert ops._tile256_variant(3072, 4096, 4096, True) == 20
     assert ops._tile256_variant(3072, 4096, 12288, True) == 20
+    # up to 256 tokens too, where one row of tiles fills the chip better than two of 128 tokens
+    # (192 tokens into the 14B shape's 34816 gate and up outputs: 139 -> 118 us)
+    assert ops._tile256_variant(192, 34816, 5120) == 21
     assert ops._tile256_variant(2048, 24576, 4096) is None and ops._tile256_variant(8192, 24576, 4096) is None
     assert ops._tile256_variant(2048, 4096, 4096, True) is None
     assert ops._tile256_variant(2048, 4096, 12288, True) is None

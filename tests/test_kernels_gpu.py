@@ -215,7 +215,8 @@ def test_gemm_many_large_tiles(kind, K, M, N, variant):
     tokens straight into LDS, with edges in M and N that are no multiple of the tile; an odd
     and an even number of k-tiles (W one or two k-tiles ahead) and one."""
     ops = _ops()
-    assert ops._tile_variant(M, N, True, kind == "accumulate", K) == variant
+    assert ops._tile_variant(M, N, True, kind == "accumulate", K) == \
+        (16 if variant == 6 and K % 128 == 0 else variant)
     assert variant == 10 or ((M + 127) // 128) * ((N + 127) // 128) >= 384
     _check_tiled(ops, kind, M, N, K, variant)
 

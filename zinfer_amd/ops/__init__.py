@@ -666,27 +666,31 @@ def _tile_variant(M: int, N: int, w_tiled: bool = False, accumulate: bool = Fals
     """Which tiled kernel: with pre-tiled weights the kernels that take W straight from
     memory (10: 128 x 256 tiles, two workgroups to a CU, when they fill the chip; 12: the same
     tiles with two groups of waves a workgroup where a CU holds one; else 128 x
-    128 tiles, 16: with the waves side by side and k-tiles of 128, for a long K or when one
-    round of the chip holds the tiles (weights from HBM, 512 tokens: qkv of the 8B shape 43 ->
-    38 us), 6: with 2 x 2 waves); otherwise the kernels that stage both operands through LDS
+    128 tiles, 16: with the waves side by side and k-tiles of 128 (weights from HBM, 512
+    tokens: qkv of the 8B shape 43 -> 38 us), 6: with 2 x 2 waves, where K is no multiple of
+    128); otherwise the kernels that stage both operands through LDS
     (4: 256 x 256 when they still fill the chip, else 0: 128 x 128).  Measured on MI355X at the
     Qwen3-8B and Qwen3-14B sizes."""
     if w_tiled:
         tiles_m = (M + 127) // 128
         tiles = tiles_m * ((N + 255) // 256)
-        # between one and two 128 x 256 tiles per CU half the CUs hold two workgroups and half
-        # one, and the smaller tiles finish sooner (2048 tokens into 6144 outputs); with few
-        # tiles along the tokens (512 tokens into 24576 outputs) the large tiles still win
-        # (five rows of tiles: 544 tokens into 24576 outputs, 480 large tiles, 143 -> 115 us)
-        if tiles >= 160 and not (256 < tiles < 512 and tiles_m > 5):
+        # from 144 large tiles on they win or draw (140 to 152 tiles: 0.84 to 1.05 of the
+        # 128 x 128 tiles' time).  Between one and two 128 x 256 tiles per CU half the CUs hold
+        # two workgroups and half one: there the 256-token tiles are measured against the
+        # 128 x 128 ones (2048 tokens into 6144 outputs); with few tiles along the tokens (512
+        # tokens into 24576 outputs) the large tiles still win (five rows of tiles: 544 tokens
+        # into 24576 outputs, 480 large tiles, 143 -> 115 us)
+        if tiles >= 144 and not (256 < tiles < 512 and tiles_m > 5):
             # one workgroup to a CU whatever is done: two groups of waves in it, each over
             # half of a long K (o_proj and down at 1280 to 2048 tokens: 3 to 12 % less; at
             # K <= 2048 the blocks handed over at the end cost more than the waves gain)
-            if tiles <= TILE_PLACES // 2 and K >= 4096 and K % 256 == 0:
+            if 160 <= tiles <= TILE_PLACES // 2 and K >= 4096 and K % 256 == 0:
                 return 12
             return 10
-        one_round = tiles_m * ((N + 127) // 128) <= 256
-        return 16 if K > 0 and K % 128 == 0 and (K >= 8192 or one_round) else 6
+        # (the 128 x 128 tiles of 2 x 2 waves, where two waves load each part of W, only
+        # where k-tiles of 128 do not divide K: in 24 products of 136 to 4096 tokens that had
+        # them, the waves side by side were level or faster, 12 % in all)
+        return 16 if K > 0 and K % 128 == 0 else 6
     tiles = ((M + 255) // 256) * ((N + 255) // 256)
     return 4 if tiles >= 160 else 0
 
@@ -832,7 +836,7 @@ def _tile256_variant(M: int, N: int, K: int, accumulate: bool = False):
     and 32B widths at 512 to 16384 tokens the choice is within 1 % of the best on the whole.
     A residual sum that is split along K keeps its split (the kernel that adds the partials
     also norms)."""
-    if M <= 256 or K % 128 != 0 or N % 16 != 0:
+    if M <= 128 or K % 128 != 0 or N % 16 != 0:
         return None
     ks = _tile_ksplit(M, N, K, accumulate)
     if ks > 1 and accumulate:
